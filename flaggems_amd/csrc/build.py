@@ -1,0 +1,88 @@
+"""Build libfg_mi355.so (gfx950 only) with hipcc: one object per source, compiled in parallel.
+
+Usage: python flaggems_amd/csrc/build.py [--force] [--jobs N]
+The library lands next to the package (flaggems_amd/libfg_mi355.so) so it travels with the tree.
+"""
+import argparse
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(HERE)
+OUT = os.path.join(PKG, "libfg_mi355.so")
+OBJ_DIR = os.path.join(HERE, "build")
+
+SOURCES = [
+    "abi.cpp",
+    "norm.hip",
+    "softmax.hip",
+    "rope.hip",
+    "kvcache.hip",
+    "silu_mul.hip",
+    "gemm.hip",
+    "gemm_skinny.hip",
+    "attn_varlen.hip",
+]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Wall",
+    "-Wno-unused-function",
+    # packed-fp32 arithmetic is switched off for every device function of this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _newer(src_paths, target):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(p) > t for p in src_paths)
+
+
+def _compile(src, force):
+    path = os.path.join(HERE, src)
+    obj = os.path.join(OBJ_DIR, src + ".o")
+    headers = [os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith(".h")]
+    headers.append(os.path.join(os.path.dirname(PKG), "include", "fg_mi355.h"))
+    if not force and not _newer([path] + headers, obj):
+        return obj, ""
+    lang = ["-x", "hip"] if src.endswith(".hip") else []
+    cmd = [HIPCC] + FLAGS + lang + ["-c", path, "-o", obj]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    log = "\n".join(l for l in (p.stdout + p.stderr).splitlines() if "packed-fp32-ops" not in l)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    return obj, log
+
+
+def build(force=False, jobs=None, verbose=True):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(HERE, s))]
+    jobs = jobs or min(8, len(srcs))
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(lambda s: _compile(s, force), srcs))
+    objs = [o for o, _ in results]
+    for _, log in results:
+        if log.strip() and verbose:
+            print(log, file=sys.stderr)
+    if force or _newer(objs, OUT):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise RuntimeError("link failed:\n" + p.stdout + p.stderr)
+    return OUT
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--force", action="store_true")
+    ap.add_argument("--jobs", type=int, default=None)
+    a = ap.parse_args()
+    print(build(force=a.force, jobs=a.jobs))

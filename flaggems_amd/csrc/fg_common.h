@@ -1,0 +1,110 @@
+// Shared device/host helpers for the gfx950 kernels of libfg_mi355.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/fg_mi355.h"
+
+// ---------------------------------------------------------------------------------------------
+// host side: error reporting
+// ---------------------------------------------------------------------------------------------
+void fg_set_error(const char* fmt, ...);
+int fg_check_launch(const char* what);
+
+#define FG_REQUIRE(cond, code, ...) \
+  do {                              \
+    if (!(cond)) {                  \
+      fg_set_error(__VA_ARGS__);    \
+      return (code);                \
+    }                               \
+  } while (0)
+
+static inline bool fg_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+static inline int64_t fg_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------------------------------------
+// element types.  __bf16 / _Float16 are native on gfx950 (v_cvt_pk_bf16_f32 rounds to nearest even).
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16_t f16x4 __attribute__((ext_vector_type(4)));
+typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct fg_type_id;
+template <> struct fg_type_id<f16_t> { static constexpr int value = FG_F16; };
+template <> struct fg_type_id<bf16_t> { static constexpr int value = FG_BF16; };
+template <> struct fg_type_id<float> { static constexpr int value = FG_F32; };
+
+// A VEC-wide pack of T moved with one memory instruction when VEC*sizeof(T) is 4, 8 or 16 bytes.
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) Pack {
+  T v[VEC];
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld_pack(const T* p) {
+  return *reinterpret_cast<const Pack<T, VEC>*>(p);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_pack(T* p, const Pack<T, VEC>& v) {
+  *reinterpret_cast<Pack<T, VEC>*>(p) = v;
+}
+// Streaming variants: data that is touched once should not displace reusable lines in L2.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld_pack_nt(const T* p) {
+  if constexpr (sizeof(T) * VEC == 16) {
+    u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return *reinterpret_cast<Pack<T, VEC>*>(&r);
+  } else if constexpr (sizeof(T) * VEC == 8) {
+    u32x2 r = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    return *reinterpret_cast<Pack<T, VEC>*>(&r);
+  } else {
+    return *reinterpret_cast<const Pack<T, VEC>*>(p);
+  }
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_pack_nt(T* p, const Pack<T, VEC>& v) {
+  if constexpr (sizeof(T) * VEC == 16) {
+    __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(&v), reinterpret_cast<u32x4*>(p));
+  } else if constexpr (sizeof(T) * VEC == 8) {
+    __builtin_nontemporal_store(*reinterpret_cast<const u32x2*>(&v), reinterpret_cast<u32x2*>(p));
+  } else {
+    *reinterpret_cast<Pack<T, VEC>*>(p) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// wavefront-64 reductions.  The first four butterfly steps stay inside a row of 16 lanes and use
+// DPP modifiers (no LDS traffic); the last two cross rows through ds_bpermute.
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+struct OpSum {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct OpMax {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+// All 64 lanes end up with the reduction over the whole wave.
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v, Op op) {
+  v = op(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = op(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = op(v, dpp_mov<0x141>(v));  // row_half_mirror
+  v = op(v, dpp_mov<0x140>(v));  // row_mirror
+  v = op(v, __shfl_xor(v, 16, 64));
+  v = op(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) { return wave_allreduce(v, OpSum()); }
+__device__ __forceinline__ float wave_max(float v) { return wave_allreduce(v, OpMax()); }

@@ -1,0 +1,212 @@
+// Host side of fg_gemm: validation, load-mode and tile selection, schedule selection, launches.
+#include <mutex>
+#include "gemm_tile.h"
+
+namespace fgk {
+
+// implemented in gemm_skinny.hip
+int skinny_supported(const GemmArgs& g, int dtype, bool b_n_contig_vec, bool a_k_contig_vec);
+size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int num_cu);
+int skinny_launch(const GemmArgs& g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st);
+// implemented in gemm_streamk.hip
+size_t streamk_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int num_cu);
+int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace, size_t workspace_bytes, int num_cu,
+                   hipStream_t st);
+
+int num_cus(int device) {
+  static std::mutex mu;
+  static int cached[64] = {0};
+  int dev = device;
+  if (dev < 0) {
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  }
+  if (dev >= 64) dev = 0;
+  std::lock_guard<std::mutex> lk(mu);
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <typename T, int BM, int BN, int AMODE, int BMODE>
+int launch_dp(const GemmArgs& g, hipStream_t st) {
+  typedef TileCompute<T, BM, BN, AMODE, BMODE> TC;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto kern = gemm_dp_kernel<T, BM, BN, AMODE, BMODE>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   TC::LDS_BYTES);
+  });
+  if (attr_err != hipSuccess) {
+    fg_set_error("gemm: cannot reserve %d bytes of LDS: %s", TC::LDS_BYTES, hipGetErrorString(attr_err));
+    return FG_ERR_LAUNCH;
+  }
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kThreads), TC::LDS_BYTES, st, g);
+  return fg_check_launch("gemm");
+}
+
+template <typename T, int BM, int BN>
+int launch_dp_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
+  if constexpr (BM == 256) {
+    // the element-wise stager would not fit the register budget of the large tile
+    if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
+    if (amode == LOAD_K && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_K, LOAD_MN>(g, st);
+    if (amode == LOAD_MN && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_MN, LOAD_K>(g, st);
+    return launch_dp<T, BM, BN, LOAD_MN, LOAD_MN>(g, st);
+  } else if constexpr (sizeof(T) == 2) {
+    if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
+    if (amode == LOAD_K && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_K, LOAD_MN>(g, st);
+    if (amode == LOAD_MN && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_MN, LOAD_K>(g, st);
+    if (amode == LOAD_MN && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_MN, LOAD_MN>(g, st);
+  } else {
+    if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
+  }
+  return launch_dp<T, BM, BN, LOAD_GEN, LOAD_GEN>(g, st);
+}
+
+// Load mode of an operand whose element (row, k) lives at base[row*s_row + k*s_k].
+int pick_mode(const void* base, int64_t rows, int64_t K, int64_t s_row, int64_t s_k, int elem_bytes) {
+  const int epc = 16 / elem_bytes;
+  if (!fg_aligned(base, 16)) return LOAD_GEN;
+  if ((s_k == 1 || K == 1) && K % epc == 0 && (rows == 1 || s_row % epc == 0)) return LOAD_K;
+  if (elem_bytes == 2 && (s_row == 1 || rows == 1) && rows % 8 == 0 && rows >= 8 && (K == 1 || s_k % 8 == 0))
+    return LOAD_MN;
+  return LOAD_GEN;
+}
+
+void set_tiles(GemmArgs& g, int BM, int BN, int BK) {
+  g.tiles_m = (int)fg_cdiv(g.M, BM);
+  g.tiles_n = (int)fg_cdiv(g.N, BN);
+  g.iters_per_tile = (int)fg_cdiv(g.K, BK);
+}
+
+template <typename T>
+int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
+  constexpr int BK = kRowBytes / sizeof(T);
+  if constexpr (sizeof(T) == 2) {
+    // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
+    const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
+    if (amode != LOAD_GEN && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
+      set_tiles(g, 256, 256, BK);
+      return launch_dp_modes<T, 256, 256>(g, amode, bmode, st);
+    }
+  }
+  set_tiles(g, 128, 128, BK);
+  FG_REQUIRE((int64_t)g.tiles_m * g.tiles_n < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "gemm: too many tiles");
+  return launch_dp_modes<T, 128, 128>(g, amode, bmode, st);
+}
+
+}  // namespace fgk
+
+using namespace fgk;
+
+extern "C" int fg_streamk_partition(int64_t tiles, int64_t iters_per_tile, int64_t workers, int64_t* sk_tiles,
+                                    int64_t* begin, int64_t* end) {
+  FG_REQUIRE(tiles >= 0 && iters_per_tile > 0 && workers > 0, FG_ERR_INVALID, "streamk_partition: bad sizes");
+  // Cooperative tiles: the ragged last wave; plus one full wave when the remainder is small
+  // (< half the workers), none when it nearly fills the machine (> 0.8 of the workers) and full
+  // waves exist.  Same rule as the reference's streamk_mm.
+  int64_t sk = tiles % workers;
+  const int64_t full = tiles - sk;
+  if (full > 0 && sk * 2 < workers) sk += workers;
+  else if (full > 0 && sk * 10 > workers * 8) sk = 0;
+  if (sk_tiles) *sk_tiles = sk;
+  const int64_t total = sk * iters_per_tile;
+  const int64_t per = total / workers, rem = total % workers;
+  for (int64_t w = 0; w < workers; ++w) {
+    // workers below `rem` take one extra iteration; ranges are contiguous in tile-major order
+    const int64_t b = w * per + (w < rem ? w : rem);
+    const int64_t e = b + per + (w < rem ? 1 : 0);
+    if (begin) begin[w] = b;
+    if (end) end[w] = e;
+  }
+  return FG_OK;
+}
+
+extern "C" size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, int schedule, int device) {
+  if (schedule == FG_SCHED_DATA_PARALLEL) return 0;
+  const int cu = num_cus(device);
+  size_t a = skinny_workspace_bytes(M, N, K, cu);
+  size_t b = streamk_workspace_bytes(M, N, K, ab_dtype, cu);
+  return a > b ? a : b;
+}
+
+extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                       int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim, int64_t sin_, int64_t scm,
+                       int64_t scn, float alpha, float beta, int ab_dtype, int c_dtype, int bias_dtype, int schedule,
+                       void* workspace, size_t workspace_bytes, int* schedule_used, void* stream) {
+  FG_REQUIRE(M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "gemm: negative size");
+  FG_REQUIRE(ab_dtype == FG_F16 || ab_dtype == FG_BF16 || ab_dtype == FG_F32, FG_ERR_INVALID, "gemm: bad dtype %d",
+             ab_dtype);
+  FG_REQUIRE(c_dtype == ab_dtype, FG_ERR_UNSUPPORTED, "gemm: output dtype %d must equal the input dtype %d", c_dtype,
+             ab_dtype);
+  FG_REQUIRE(bias == nullptr || bias_dtype == ab_dtype, FG_ERR_UNSUPPORTED,
+             "gemm: bias dtype %d must equal the input dtype %d", bias_dtype, ab_dtype);
+  FG_REQUIRE(schedule >= FG_SCHED_AUTO && schedule <= FG_SCHED_STREAM_K, FG_ERR_INVALID, "gemm: bad schedule %d",
+             schedule);
+  if (schedule_used) *schedule_used = FG_SCHED_DATA_PARALLEL;
+  if (M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(K > 0, FG_ERR_INVALID, "gemm: K must be positive (the caller handles K == 0)");
+  FG_REQUIRE(A && B && C, FG_ERR_INVALID, "gemm: null pointer");
+  FG_REQUIRE(M < ((int64_t)1 << 31) && N < ((int64_t)1 << 31) && K < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED,
+             "gemm: extent exceeds 2^31");
+  hipStream_t st = (hipStream_t)stream;
+  GemmArgs g = {};
+  g.A = A; g.B = B; g.bias = bias; g.C = C;
+  g.M = M; g.N = N; g.K = K;
+  g.sam = sam; g.sak = sak; g.sbk = sbk; g.sbn = sbn; g.sim = sim; g.sin = sin_; g.scm = scm; g.scn = scn;
+  g.alpha = alpha; g.beta = beta;
+  const int eb = ab_dtype == FG_F32 ? 4 : 2;
+  int amode = pick_mode(A, M, K, sam, sak, eb);
+  int bmode = pick_mode(B, N, K, sbn, sbk, eb);
+  if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_K || bmode != LOAD_K)))
+    amode = bmode = LOAD_GEN;
+  const int cu = num_cus(-1);
+
+  // ---- schedule --------------------------------------------------------------------------------
+  // Skinny problems (M <= 16 rows) are bandwidth-bound streams of B: their own stream-K kernel.
+  const int sk_ok = skinny_supported(g, ab_dtype, bmode == LOAD_MN, amode == LOAD_K);
+  bool use_skinny = false, use_streamk = false;
+  if (schedule != FG_SCHED_DATA_PARALLEL && workspace != nullptr) {
+    if (sk_ok) {
+      use_skinny = workspace_bytes >= skinny_workspace_bytes(M, N, K, cu);
+    } else if (eb == 2) {
+      const size_t need = streamk_workspace_bytes(M, N, K, ab_dtype, cu);
+      if (need > 0 && workspace_bytes >= need) {
+        if (schedule == FG_SCHED_STREAM_K) {
+          use_streamk = true;
+        } else {
+          // auto: stream-K when the data-parallel grid would leave most of the last wave idle and K
+          // is deep enough to split (at least two K steps per workgroup).
+          const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
+          const int64_t iters = fg_cdiv(K, 64);
+          const int64_t rem = tiles % cu;
+          use_streamk = rem != 0 && rem * 10 <= (int64_t)cu * 8 && tiles < (int64_t)cu * 4 &&
+                        (tiles % cu) * iters >= 2 * (int64_t)cu;
+        }
+      }
+    }
+  }
+  if (schedule == FG_SCHED_STREAM_K && !use_skinny && !use_streamk) {
+    fg_set_error("gemm: the stream-K schedule needs 16-bit inputs and a workspace of %zu bytes (got %zu)",
+                 fg_gemm_workspace_bytes(M, N, K, ab_dtype, schedule, -1), workspace_bytes);
+    return workspace == nullptr || eb == 2 ? FG_ERR_WORKSPACE : FG_ERR_UNSUPPORTED;
+  }
+  if (use_skinny) {
+    if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;
+    return skinny_launch(g, ab_dtype, workspace, workspace_bytes, cu, st);
+  }
+  if (use_streamk) {
+    if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;
+    return streamk_launch(g, ab_dtype, amode, bmode, workspace, workspace_bytes, cu, st);
+  }
+  switch (ab_dtype) {
+    case FG_F16: return run_dp<f16_t>(g, amode, bmode, cu, st);
+    case FG_BF16: return run_dp<bf16_t>(g, amode, bmode, cu, st);
+    default: return run_dp<float>(g, amode, bmode, cu, st);
+  }
+}

@@ -1,0 +1,224 @@
+// rms_norm and fused_add_rms_norm for gfx950: single pass over HBM, the row lives in registers.
+//
+// Layout: x [M, N] with unit column stride and arbitrary row stride.  TPR threads share one row
+// (TPR = 64 .. 1024, a power of two); each thread holds ITERS packs of VEC elements, pack j of
+// thread t covering columns (j*TPR + t)*VEC .. +VEC, so every load instruction of a wave reads
+// 64*VEC*sizeof(T) contiguous bytes (1 KiB at 16 B per lane).  Blocks are 256 threads, so
+// 256/TPR rows share a block when TPR < 256.  Rows too long for the register variant
+// (N > 1024*VEC*8) and rows that defeat vector access (N or strides not a multiple of VEC,
+// unaligned base) go through a looped two-pass kernel that re-reads the row from L2.
+#include "fg_common.h"
+
+namespace {
+
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* smem, int row_in_block, int t) {
+  v = wave_sum(v);
+  if constexpr (TPR > 64) {
+    constexpr int WPR = TPR / 64;  // waves per row
+    const int wave_in_row = t >> 6;
+    __syncthreads();
+    if ((t & 63) == 0) smem[row_in_block * WPR + wave_in_row] = v;
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) s += smem[row_in_block * WPR + i];
+    v = s;
+  }
+  return v;
+}
+
+// FUSED = false: y = x * rrms * w, optional inv_rms.   FUSED = true: r = x + r (stored), x = r*rrms*w.
+template <typename T, int VEC, int ITERS, int TPR, bool FUSED>
+__global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
+    const T* x, T* res, const T* __restrict__ w, T* y,
+    float* __restrict__ inv_rms, int64_t M, int N, int64_t xs, int64_t rs, int64_t ys, float eps) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ float smem[BLOCK / 64];
+  const int tid = threadIdx.x;
+  const int row_in_block = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + row_in_block;
+  const bool row_ok = row < M;
+  const T* xr = x + row * xs;
+
+  float v[ITERS][VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    if (row_ok && col < N) {
+      Pack<T, VEC> px = ld_pack_nt<T, VEC>(xr + col);
+      if constexpr (FUSED) {
+        Pack<T, VEC> pr = ld_pack_nt<T, VEC>(res + row * rs + col);
+        Pack<T, VEC> po;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          v[j][e] = (float)px.v[e] + (float)pr.v[e];
+          po.v[e] = (T)v[j][e];
+        }
+        st_pack_nt<T, VEC>(res + row * rs + col, po);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[j][e] = (float)px.v[e];
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ss += v[j][e] * v[j][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[j][e] = 0.f;
+    }
+  }
+  ss = row_sum<TPR>(ss, smem, row_in_block, t);
+  const float rrms = 1.0f / sqrtf(ss / (float)N + eps);
+  if (!row_ok) return;
+  if constexpr (!FUSED) {
+    if (inv_rms != nullptr && t == 0) inv_rms[row] = rrms;
+  }
+  T* yr = y + row * ys;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    if (col < N) {
+      Pack<T, VEC> po;
+      if (w != nullptr) {
+        Pack<T, VEC> pw = ld_pack<T, VEC>(w + col);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) po.v[e] = (T)(v[j][e] * rrms * (float)pw.v[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) po.v[e] = (T)(v[j][e] * rrms);
+      }
+      st_pack_nt<T, VEC>(yr + col, po);
+    }
+  }
+}
+
+// Any N, any alignment: one 256-thread block per row, element-wise coalesced access, two passes.
+template <typename T, bool FUSED>
+__global__ __launch_bounds__(256) void rms_looped_kernel(const T* x, T* res,
+                                                        const T* __restrict__ w, T* y,
+                                                        float* __restrict__ inv_rms, int64_t M, int64_t N,
+                                                        int64_t xs, int64_t rs, int64_t ys, float eps) {
+  __shared__ float smem[4];
+  const int64_t row = blockIdx.x;
+  const T* xr = x + row * xs;
+  T* rr = FUSED ? res + row * rs : nullptr;
+  T* yr = y + row * ys;
+  float ss = 0.f;
+  for (int64_t c = threadIdx.x; c < N; c += 256) {
+    float v = (float)xr[c];
+    if constexpr (FUSED) v += (float)rr[c];
+    ss += v * v;
+  }
+  ss = row_sum<256>(ss, smem, 0, threadIdx.x);
+  const float rrms = 1.0f / sqrtf(ss / (float)N + eps);
+  if constexpr (!FUSED) {
+    if (inv_rms != nullptr && threadIdx.x == 0) inv_rms[row] = rrms;
+  }
+  // Second pass recomputes the fp32 sum from the still-unmodified inputs (each element is read
+  // and then written by the same thread, so in-place operation is safe).
+  for (int64_t c = threadIdx.x; c < N; c += 256) {
+    float v = (float)xr[c];
+    if constexpr (FUSED) {
+      v += (float)rr[c];
+      rr[c] = (T)v;
+    }
+    const float wv = w != nullptr ? (float)w[c] : 1.0f;
+    yr[c] = (T)(v * rrms * wv);
+  }
+}
+
+template <typename T, int VEC, int ITERS, int TPR, bool FUSED>
+void launch_rows(const T* x, T* res, const T* w, T* y, float* inv_rms, int64_t M, int N, int64_t xs, int64_t rs,
+                 int64_t ys, float eps, hipStream_t st) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  const int64_t grid = fg_cdiv(M, RPB);
+  hipLaunchKernelGGL((rms_rows_kernel<T, VEC, ITERS, TPR, FUSED>), dim3((unsigned)grid), dim3(BLOCK), 0, st, x, res,
+                     w, y, inv_rms, M, N, xs, rs, ys, eps);
+}
+
+template <typename T, bool FUSED>
+int rms_dispatch(const T* x, T* res, const T* w, T* y, float* inv_rms, int64_t M, int64_t N, int64_t xs, int64_t rs,
+                 int64_t ys, float eps, hipStream_t st) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec_ok = (N % VEC == 0) && (xs % VEC == 0) && (ys % VEC == 0) && (!FUSED || rs % VEC == 0) &&
+                      fg_aligned(x, 16) && fg_aligned(y, 16) && (!FUSED || fg_aligned(res, 16)) &&
+                      (w == nullptr || fg_aligned(w, 16));
+  const int64_t packs = vec_ok ? N / VEC : 0;
+  if (M >= (int64_t)1 << 31) {
+    fg_set_error("rms_norm: M=%lld exceeds the grid limit", (long long)M);
+    return FG_ERR_UNSUPPORTED;
+  }
+#define FG_ROWS(ITERS, TPR) launch_rows<T, VEC, ITERS, TPR, FUSED>(x, res, w, y, inv_rms, M, (int)N, xs, rs, ys, eps, st)
+  if (!vec_ok || packs > 1024 * 8) {
+    hipLaunchKernelGGL((rms_looped_kernel<T, FUSED>), dim3((unsigned)M), dim3(256), 0, st, x, res, w, y, inv_rms, M,
+                       N, xs, rs, ys, eps);
+  } else if (packs <= 64) {
+    FG_ROWS(1, 64);
+  } else if (packs <= 128) {
+    FG_ROWS(2, 64);
+  } else if (packs <= 256) {
+    FG_ROWS(4, 64);
+  } else if (packs <= 512) {
+    FG_ROWS(4, 128);
+  } else if (packs <= 1024) {
+    FG_ROWS(4, 256);
+  } else if (packs <= 2048) {
+    FG_ROWS(4, 512);
+  } else if (packs <= 4096) {
+    FG_ROWS(4, 1024);
+  } else {
+    FG_ROWS(8, 1024);
+  }
+#undef FG_ROWS
+  return fg_check_launch(FUSED ? "fused_add_rms_norm" : "rms_norm");
+}
+
+}  // namespace
+
+extern "C" int fg_rms_norm(const void* x, const void* w, void* y, float* inv_rms, int64_t M, int64_t N,
+                           int64_t x_row_stride, int64_t y_row_stride, float eps, int dtype, void* stream) {
+  FG_REQUIRE(M >= 0 && N >= 0, FG_ERR_INVALID, "rms_norm: negative size M=%lld N=%lld", (long long)M, (long long)N);
+  if (M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(x && y, FG_ERR_INVALID, "rms_norm: null pointer");
+  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "rms_norm: N=%lld too large", (long long)N);
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case FG_F16:
+      return rms_dispatch<f16_t, false>((const f16_t*)x, nullptr, (const f16_t*)w, (f16_t*)y, inv_rms, M, N,
+                                        x_row_stride, 0, y_row_stride, eps, st);
+    case FG_BF16:
+      return rms_dispatch<bf16_t, false>((const bf16_t*)x, nullptr, (const bf16_t*)w, (bf16_t*)y, inv_rms, M, N,
+                                         x_row_stride, 0, y_row_stride, eps, st);
+    case FG_F32:
+      return rms_dispatch<float, false>((const float*)x, nullptr, (const float*)w, (float*)y, inv_rms, M, N,
+                                        x_row_stride, 0, y_row_stride, eps, st);
+  }
+  fg_set_error("rms_norm: unsupported dtype %d", dtype);
+  return FG_ERR_INVALID;
+}
+
+extern "C" int fg_fused_add_rms_norm(void* x, void* residual, const void* w, int64_t M, int64_t N,
+                                     int64_t x_row_stride, int64_t r_row_stride, float eps, int dtype, void* stream) {
+  FG_REQUIRE(M >= 0 && N >= 0, FG_ERR_INVALID, "fused_add_rms_norm: negative size");
+  if (M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(x && residual && w, FG_ERR_INVALID, "fused_add_rms_norm: null pointer");
+  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "fused_add_rms_norm: N=%lld too large", (long long)N);
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case FG_F16:
+      return rms_dispatch<f16_t, true>((const f16_t*)x, (f16_t*)residual, (const f16_t*)w, (f16_t*)x, nullptr, M, N,
+                                       x_row_stride, r_row_stride, x_row_stride, eps, st);
+    case FG_BF16:
+      return rms_dispatch<bf16_t, true>((const bf16_t*)x, (bf16_t*)residual, (const bf16_t*)w, (bf16_t*)x, nullptr, M,
+                                        N, x_row_stride, r_row_stride, x_row_stride, eps, st);
+    case FG_F32:
+      return rms_dispatch<float, true>((const float*)x, (float*)residual, (const float*)w, (float*)x, nullptr, M, N,
+                                       x_row_stride, r_row_stride, x_row_stride, eps, st);
+  }
+  fg_set_error("fused_add_rms_norm: unsupported dtype %d", dtype);
+  return FG_ERR_INVALID;
+}

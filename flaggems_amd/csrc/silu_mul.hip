@@ -1,0 +1,65 @@
+// silu_and_mul for gfx950: out[r, c] = a[r, c] / (1 + exp(-a[r, c])) * b[r, c] in fp32.
+//
+// a, b and out are [rows, cols] with unit column stride and independent row strides, which covers
+// the two halves of a fused gate-up projection without a copy.  Packs of 16 bytes are numbered
+// row-major and dealt one per thread.  Rows that defeat 16-byte access are handled one element
+// per thread.
+#include "fg_common.h"
+
+namespace {
+
+__device__ __forceinline__ float silu_mul(float x, float y) { return x / (1.0f + __expf(-x)) * y; }
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* a, const T* b, T* out,
+                                                      int64_t rows, int64_t cols, int64_t as, int64_t bs, int64_t os) {
+  const int64_t ppr = cols / VEC;  // packs per row
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= rows * ppr) return;
+  const int64_t r = item / ppr;
+  const int64_t c = (item - r * ppr) * VEC;
+  Pack<T, VEC> x = ld_pack_nt<T, VEC>(a + r * as + c), y = ld_pack_nt<T, VEC>(b + r * bs + c), o;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) o.v[e] = (T)silu_mul((float)x.v[e], (float)y.v[e]);
+  st_pack_nt<T, VEC>(out + r * os + c, o);
+}
+
+template <typename T>
+int silu_dispatch(const T* a, const T* b, T* out, int64_t rows, int64_t cols, int64_t as, int64_t bs, int64_t os,
+                  hipStream_t st) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec_ok = cols % VEC == 0 && as % VEC == 0 && bs % VEC == 0 && os % VEC == 0 && fg_aligned(a, 16) &&
+                      fg_aligned(b, 16) && fg_aligned(out, 16);
+  const int64_t items = vec_ok ? rows * (cols / VEC) : rows * cols;
+  const int64_t grid = fg_cdiv(items, 256);
+  FG_REQUIRE(grid < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "silu_and_mul: problem too large for one launch");
+  if (vec_ok)
+    hipLaunchKernelGGL((silu_mul_kernel<T, VEC>), dim3((unsigned)grid), dim3(256), 0, st, a, b, out, rows, cols, as, bs, os);
+  else
+    hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((unsigned)grid), dim3(256), 0, st, a, b, out, rows, cols, as, bs, os);
+  return fg_check_launch("silu_and_mul");
+}
+
+}  // namespace
+
+extern "C" int fg_silu_and_mul(const void* a, const void* b, void* out, int64_t rows, int64_t cols,
+                               int64_t a_row_stride, int64_t b_row_stride, int64_t o_row_stride, int dtype,
+                               void* stream) {
+  FG_REQUIRE(rows >= 0 && cols >= 0, FG_ERR_INVALID, "silu_and_mul: negative size");
+  if (rows == 0 || cols == 0) return FG_OK;
+  FG_REQUIRE(a && b && out, FG_ERR_INVALID, "silu_and_mul: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case FG_F16:
+      return silu_dispatch((const f16_t*)a, (const f16_t*)b, (f16_t*)out, rows, cols, a_row_stride, b_row_stride,
+                           o_row_stride, st);
+    case FG_BF16:
+      return silu_dispatch((const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, rows, cols, a_row_stride, b_row_stride,
+                           o_row_stride, st);
+    case FG_F32:
+      return silu_dispatch((const float*)a, (const float*)b, (float*)out, rows, cols, a_row_stride, b_row_stride,
+                           o_row_stride, st);
+  }
+  fg_set_error("silu_and_mul: unsupported dtype %d", dtype);
+  return FG_ERR_INVALID;
+}

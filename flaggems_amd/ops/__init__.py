@@ -1,0 +1,7 @@
+from .addmm import addmm, addmm_out
+from .attention import flash_attn_varlen_func
+from .mm import mm, mm_out
+from .rms_norm import rms_norm
+from .softmax import softmax
+
+__all__ = ["addmm", "addmm_out", "flash_attn_varlen_func", "mm", "mm_out", "rms_norm", "softmax"]

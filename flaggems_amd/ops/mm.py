@@ -1,0 +1,68 @@
+"""aten::mm / aten::mm.out on the gfx950 MFMA GEMM (reference: src/flag_gems/ops/mm.py:137-237)."""
+import logging
+
+import torch
+
+from .. import _C
+from ._gemm import gemm, get_higher_dtype  # noqa: F401
+
+logger = logging.getLogger("flag_gems.ops.mm")
+
+
+def _prepare(a, b):
+    # same contiguity rule as the reference: copy only when both strides exceed one
+    if a.stride(0) > 1 and a.stride(1) > 1:
+        a = a.contiguous()
+    if b.stride(0) > 1 and b.stride(1) > 1:
+        b = b.contiguous()
+    assert a.shape[1] == b.shape[0], "incompatible dimensions"
+    return a, b
+
+
+def _kernel_covers(a, b):
+    return a.dim() == 2 and b.dim() == 2 and _C.supported_dtype(a.dtype) and _C.supported_dtype(b.dtype)
+
+
+def _vendor_mm(a, b, out=None):
+    # bmm is a separate ATen kernel, so this cannot re-enter the override
+    r = torch.bmm(a.unsqueeze(0), b.unsqueeze(0)).squeeze(0)
+    if out is None:
+        return r
+    out.copy_(r)
+    return out
+
+
+def _run(a, b, c):
+    M, K = a.shape
+    N = b.shape[1]
+    logger.debug(
+        "GEMS MM, [shape info]: [-, %s, %s, %s](batch, M, N, K), [A column-major]: %s, [B column-major]: %s",
+        M, N, K, a.stride(0) == 1, b.stride(0) == 1,
+    )
+    if M == 0 or N == 0:
+        return c
+    if K == 0:
+        return c.zero_()
+    if a.dtype != b.dtype:
+        # the reference casts inside the kernel to the higher of the two dtypes
+        hi = get_higher_dtype(a.dtype, b.dtype)
+        a, b = a.to(hi), b.to(hi)
+    return gemm(a, b, None, c, 1.0, 0.0)
+
+
+def mm(a, b):
+    if not _kernel_covers(a, b):
+        return _vendor_mm(a, b)
+    a, b = _prepare(a, b)
+    M, _ = a.shape
+    N = b.shape[1]
+    c = torch.empty((M, N), device=a.device, dtype=get_higher_dtype(a.dtype, b.dtype))
+    return _run(a, b, c)
+
+
+def mm_out(a, b, *, out):
+    if not _kernel_covers(a, b) or not _C.supported_dtype(out.dtype):
+        return _vendor_mm(a, b, out)
+    a, b = _prepare(a, b)
+    assert out.shape == (a.shape[0], b.shape[1]), "incompatible output shape"
+    return _run(a, b, out)

@@ -1,0 +1,35 @@
+"""aten::_softmax forward on the gfx950 kernels (reference: src/flag_gems/ops/softmax.py:283-318)."""
+import logging
+
+import torch
+
+from .. import _C
+
+logger = logging.getLogger("flag_gems.ops.softmax")
+
+
+def softmax(self, dim, half_to_float=False):
+    logger.debug("GEMS SOFTMAX")
+    assert dim >= -self.ndim and dim < self.ndim, "Invalid dim"
+    if not _C.supported_dtype(self.dtype):
+        # the .out overload is a separate ATen kernel that stays on the vendor library
+        out = torch.empty_like(self, memory_format=torch.contiguous_format)
+        return torch.ops.aten._softmax.out(self, dim, half_to_float, out=out)
+    dim = dim % self.ndim
+    M = 1
+    N = self.shape[dim]
+    for i in range(dim):
+        M *= self.shape[i]
+    self = self.contiguous()
+    dtype = torch.float32 if half_to_float else self.dtype
+    out = torch.empty_like(self, dtype=dtype)
+    if self.numel() == 0:
+        return out
+    K = self.numel() // M // N
+    with torch.cuda.device(self.device):
+        rc = _C.lib().fg_softmax(
+            self.data_ptr(), out.data_ptr(), M, N, K, _C.dtype_id(self.dtype), _C.dtype_id(dtype),
+            _C.current_stream(self.device),
+        )
+    _C.check(rc, "fg_softmax")
+    return out

@@ -1,0 +1,167 @@
+/*
+ * fg_mi355.h — C ABI of libfg_mi355.so: hand-written gfx950 (CDNA4) kernels for the
+ * LLM-inference operator path of FlagGems (mm/addmm, softmax, rms_norm, fused_add_rms_norm,
+ * rotary embedding, reshape_and_cache_flash, silu_and_mul, flash_attn_varlen_func).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - sizes and strides are int64 and counted in ELEMENTS, never bytes;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - entry points validate on the host, launch asynchronously on `stream`, never
+ *     synchronise and never allocate device memory;
+ *   - return value: FG_OK (0) or a negative FG_ERR_* code; fg_last_error() gives the
+ *     thread-local message of the last failure.  No C++ exception crosses this boundary.
+ *
+ * Each declaration cites the reference interface it stands in for (paths are relative to
+ * the FlagGems source tree).
+ */
+#ifndef FG_MI355_H
+#define FG_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { FG_F16 = 0, FG_BF16 = 1, FG_F32 = 2 };
+
+enum {
+  FG_OK = 0,
+  FG_ERR_INVALID = -1,     /* bad shape / stride / null pointer / dtype */
+  FG_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+  FG_ERR_LAUNCH = -3,      /* hipGetLastError() reported a failure after the launch */
+  FG_ERR_WORKSPACE = -4    /* workspace missing or too small */
+};
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* fg_last_error(void);
+
+/* ABI version of this header (bumped on any signature change). */
+int fg_abi_version(void);
+
+/* Device facts the host-side heuristics use (CU count stands in for the reference's
+ * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530). */
+int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
+
+/* rms_norm forward.  y[m,:] = x[m,:] * rsqrt(mean(x[m,:]^2) + eps) * w, fp32 arithmetic,
+ * one rounding on store; inv_rms[m] (fp32) is written when non-NULL; w may be NULL (= ones).
+ * Replaces rms_norm_kernel, src/flag_gems/ops/rms_norm.py:15-51, and
+ * flag_gems::rms_norm, lib/rms_norm.cpp:15-71. */
+int fg_rms_norm(const void* x, const void* w, void* y, float* inv_rms, int64_t M, int64_t N,
+                int64_t x_row_stride, int64_t y_row_stride, float eps, int dtype, void* stream);
+
+/* In-place pair update: residual = x + residual (rounded to dtype on store), x =
+ * rmsnorm(unrounded sum) * w.
+ * Replaces fused_add_rms_norm_kernel, src/flag_gems/fused/fused_add_rms_norm.py:14-54, and
+ * flag_gems::fused_add_rms_norm, lib/fused_add_rms_norm.cpp:14-72. */
+int fg_fused_add_rms_norm(void* x, void* residual, const void* w, int64_t M, int64_t N,
+                          int64_t x_row_stride, int64_t r_row_stride, float eps, int dtype,
+                          void* stream);
+
+/* softmax over the middle axis of a contiguous [M, N, K] view (K == 1: innermost axis).
+ * fp32 arithmetic, out_dtype == in_dtype or FG_F32 (half_to_float).
+ * Replaces softmax_kernel_inner / softmax_kernel_non_inner,
+ * src/flag_gems/ops/softmax.py:15-72,87-159, and flag_gems::softmax, lib/softmax.cpp:28-73. */
+int fg_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype,
+               int out_dtype, void* stream);
+
+/* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
+ * {token, head, dim}); cos/sin [max_pos, D/2] with unit inner stride.  pos == NULL means
+ * position = token_index % seq_len.  q_out/k_out may alias q/k (in-place).
+ * Replaces apply_rotary_pos_emb_kernel / _inplace_kernel,
+ * src/flag_gems/fused/rotary_embedding.py:15-178, and flag_gems::rotary_embedding(_inplace),
+ * lib/rotary_embedding.cpp:96-281. */
+int fg_rope(void* q_out, void* k_out, const void* q, const void* k, const void* cos,
+            const void* sin, const void* pos, int pos_is_i64, int64_t n_tokens, int64_t seq_len,
+            int Hq, int Hk, int D, const int64_t q_strides[3], const int64_t k_strides[3],
+            const int64_t qo_strides[3], const int64_t ko_strides[3], int64_t pos_stride,
+            int64_t cos_stride, int64_t sin_stride, int64_t max_pos, int interleaved, int dtype,
+            int cs_dtype, void* stream);
+
+/* Scatter of K/V token rows (H*D dense elements each) into the paged caches
+ * [num_blocks, block_size, H, D]; slot < 0 skips the token.  Pure byte copy.
+ * Replaces reshape_and_cache_flash_kernel, src/flag_gems/fused/reshape_and_cache_flash.py:14-58,
+ * and flag_gems::reshape_and_cache_flash, lib/reshape_and_cache_flash.cpp:11-67. */
+int fg_reshape_and_cache_flash(const void* key, const void* value, void* key_cache,
+                               void* value_cache, const void* slot_mapping, int slot_is_i64,
+                               int64_t num_tokens, int H, int D, int block_size,
+                               int64_t key_stride, int64_t value_stride, int64_t block_stride,
+                               int elem_bytes, void* stream);
+
+/* out[r,c] = silu(a[r,c]) * b[r,c] (fp32 arithmetic), rows of unit inner stride.
+ * Replaces silu_and_mul_kernel, src/flag_gems/fused/silu_and_mul.py:12-17,47-53. */
+int fg_silu_and_mul(const void* a, const void* b, void* out, int64_t rows, int64_t cols,
+                    int64_t a_row_stride, int64_t b_row_stride, int64_t o_row_stride, int dtype,
+                    void* stream);
+
+/* GEMM schedules. */
+enum { FG_SCHED_AUTO = 0, FG_SCHED_DATA_PARALLEL = 1, FG_SCHED_STREAM_K = 2 };
+
+/* Bytes of device scratch fg_gemm needs for this problem under `schedule` (0 for the
+ * data-parallel schedule).  The caller owns the buffer; it need not be zeroed.
+ * Stands in for the per-call `locks`/`P` allocation of src/flag_gems/ops/mm_streamk.py:488-491. */
+size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, int schedule,
+                               int device);
+
+/* C[M,N] = alpha * (A[M,K] . B[K,N]) + beta * bias (bias == NULL: C = A.B), fp32 accumulate.
+ * A, B, C and bias are addressed through (row, col) element strides; bias strides may be 0
+ * (broadcast).  Which schedule ran is reported through *schedule_used when non-NULL.
+ * Replaces mm_kernel_general (src/flag_gems/ops/mm.py:54-134), addmm_kernel
+ * (src/flag_gems/ops/addmm.py:15-80), streamk_mm (src/flag_gems/ops/mm_streamk.py:451-576) and
+ * their C++ twins lib/mm.cpp:71-332, lib/addmm.cpp:11-123. */
+int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+            int64_t K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim,
+            int64_t sin_, int64_t scm, int64_t scn, float alpha, float beta, int ab_dtype,
+            int c_dtype, int bias_dtype, int schedule, void* workspace, size_t workspace_bytes,
+            int* schedule_used, void* stream);
+
+/* Host-side stream-K partition (pure integer function; also used by the tests).
+ * Given `tiles` output tiles of `iters_per_tile` K-iterations each and `workers` persistent
+ * workgroups, worker w owns the half-open range [begin[w], end[w]) of the tile-major iteration
+ * space of the stream-K tiles; *sk_tiles receives how many tiles are cooperative.
+ * Follows the split of src/flag_gems/ops/mm_streamk.py:466-485. */
+int fg_streamk_partition(int64_t tiles, int64_t iters_per_tile, int64_t workers,
+                         int64_t* sk_tiles, int64_t* begin /*host, [workers]*/,
+                         int64_t* end /*host, [workers]*/);
+
+/* POD mirror of the fields of FlashFwdParams (include/flag_gems/operators.h:126-194) that the
+ * varlen paged forward uses. */
+typedef struct FgFlashParams {
+  const void* q;           /* [total_q, Hq, D] */
+  const void* k_cache;     /* [num_pages, page_size, Hk, D] */
+  const void* v_cache;     /* [num_pages, page_size, Hk, D] */
+  void* out;               /* [total_q, Hq, D] */
+  float* lse;              /* [Hq, total_q] fp32, may be NULL */
+  const int32_t* cu_seqlens_q; /* [batch + 1] */
+  const int32_t* seqused_k;    /* [batch] */
+  const int32_t* block_table;  /* [batch, max_pages_per_seq] */
+  const float* alibi_slopes;   /* [Hq] or [batch, Hq], may be NULL */
+  int64_t q_row_stride, q_head_stride;     /* elements */
+  int64_t o_row_stride, o_head_stride;
+  int64_t k_page_stride, k_row_stride, k_head_stride;
+  int64_t v_page_stride, v_row_stride, v_head_stride;
+  int64_t block_table_stride;  /* elements between batch rows of block_table */
+  int64_t alibi_batch_stride;  /* 0 when alibi_slopes is [Hq] */
+  int64_t total_q;
+  int32_t batch, Hq, Hk, D, page_size;
+  int32_t max_seqlen_q, max_seqlen_k;
+  int32_t is_causal;
+  int32_t window_left, window_right; /* -1 = unbounded */
+  float softmax_scale;
+  float softcap;            /* 0 = off */
+  int32_t dtype;            /* FG_F16 or FG_BF16 */
+} FgFlashParams;
+
+/* Forward of variable-length attention over a paged KV cache (FA2 semantics: bottom-right
+ * aligned causal mask, GQA by head mapping, optional sliding window / softcap / alibi).
+ * Replaces flash_varlen_fwd_kernel (src/flag_gems/ops/flash_kernel.py:1216-1577) and the launch
+ * half of mha_varlan_fwd (src/flag_gems/ops/flash_api.py:230-569,
+ * lib/flash_attn_varlen_func.cpp:14-481). */
+int fg_flash_attn_varlen_fwd(const FgFlashParams* p /*host*/, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FG_MI355_H */
