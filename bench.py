@@ -1,0 +1,372 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X-native FlagGems operator path on ONE GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+
+A "step" is one pass of one operator over one batch of synthetic input that is already resident in
+HBM.  The headline workload (the JSON line's metric/value) is the softmax configuration of
+BASELINE.json: softmax over the last axis of a [131072, 2048] bf16 tensor, ~N(0, 4) with 1 % of the
+entries at -inf.  Its 1 GiB of algorithmic traffic (read + write of one tensor) is larger than the
+256 MB Infinity Cache, so the rate is an HBM rate.  The other configurations (fused_add_rms_norm,
+the three GEMMs, varlen GQA prefill attention, the decoder layer) are measured in the same run and
+reported under "configs", each with its own roofline entry.
+
+Timing: W untimed warm-up steps, then exactly K steps bracketed by torch.cuda.synchronize() on both
+sides (one GPU, so the barrier is the synchronize).  ms_per_step / value come from the wall clock
+around the K steps; roofline.achieved comes from HIP events recorded on the stream the kernels are
+launched on (torch's current stream) around the same K steps.
+
+cpu_baseline: the CPU oracle (PyTorch ATen on the host, the computation the reference's --ref cpu
+tests use as ground truth) timed on this machine's cores on a bounded sample of the same workload.
+It is a reported baseline, never the thing optimised.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA, published
+
+
+def _die_multi_gpu(n):
+    print(
+        "bench.py: this build measures one GPU only (--gpus %d requested). The operator path has no "
+        "collective; run it with --gpus 1." % n,
+        file=sys.stderr,
+    )
+    sys.exit(2)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="softmax_c2")
+    ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        _die_multi_gpu(max(args.gpus, int(os.environ.get("WORLD_SIZE", "1"))))
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    import flag_gems
+    from flaggems_amd import _C
+    from flaggems_amd.ops import _gemm
+
+    if not os.path.exists(_C.LIB_PATH):  # load what is built; build only if nothing is
+        import __graft_entry__
+
+        __graft_entry__.build()
+    _C.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    bf16 = torch.bfloat16
+
+    # ------------------------------------------------------------------------------------------
+    def timed(run, steps, warmup):
+        """(wall ms per step, event ms per step) for `steps` calls of run(i)."""
+        for i in range(warmup):
+            run(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            run(i)
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+    def roofline(bound, work, ev_ms, traffic=None):
+        if bound == "hbm":
+            ach = work / ev_ms / 1e6  # GB/s
+            return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic}
+        ach = work / ev_ms / 1e9  # TFLOP/s
+        return {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / MFMA_PEAK_TFLOPS, 4), "traffic": traffic}
+
+    def cpu_time(fn, min_seconds=2.0, max_reps=5):
+        fn()  # warm-up
+        ts = []
+        t_all = time.perf_counter()
+        while len(ts) < max_reps and (len(ts) < 1 or time.perf_counter() - t_all < min_seconds):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    cores = torch.get_num_threads()
+    from oracle import torch_ref as O  # the checker, used here only for the cpu_baseline leg
+
+    # ------------------------------------------------------------------------------------------
+    # workloads: each returns dict(run, work, bound, unit_note, cpu=(fn, sample_work, sample_note), dtype)
+    # ------------------------------------------------------------------------------------------
+    def wl_softmax_c2():
+        g = torch.Generator(device="cpu").manual_seed(0)
+        M, N = 131072, 2048
+        x = torch.empty(M, N, dtype=bf16, device=dev)
+        chunk = 8192
+        for r in range(0, M, chunk):  # generated on the host generator in slices to bound host memory
+            xs = torch.randn(chunk, N, generator=g) * 2.0
+            xs[torch.rand(chunk, N, generator=g) < 0.01] = float("-inf")
+            x[r:r + chunk] = xs.to(bf16).to(dev)
+        state = {}
+
+        def run(i):
+            state["y"] = flag_gems.softmax(x, -1)
+
+        sample = x[:32768].cpu()
+
+        def cpu():
+            O.softmax(sample, -1)
+
+        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16",
+                    workload="softmax dim=-1 [131072,2048] bf16, N(0,4) with 1% -inf (BASELINE.json configs[1])",
+                    cpu=(cpu, 2 * 32768 * N * 2, "oracle softmax (torch CPU, fp64 upcast) on the first 32768 rows"))
+
+    def wl_fused_add_rms_norm_c1():
+        torch.manual_seed(0)
+        M, N, sets = 4096, 4096, 6  # 6 x 64 MiB of x+residual: rotates through more than the 256 MB cache
+        xs = [torch.randn(M, N).to(bf16).to(dev) for _ in range(sets)]
+        rs = [torch.randn(M, N).to(bf16).to(dev) for _ in range(sets)]
+        w = (torch.rand(N) + 0.5).to(bf16).to(dev)
+
+        def run(i):
+            flag_gems.fused_add_rms_norm(xs[i % sets], rs[i % sets], [N], w, 1e-6)
+
+        xc, rc, wc = torch.randn(M, N), torch.randn(M, N), torch.rand(N) + 0.5
+
+        def cpu():
+            O.fused_add_rms_norm(xc, rc, wc, 1e-6)
+
+        return dict(run=run, work=4 * M * N * 2 + N * 2, bound="hbm", dtype="bf16",
+                    workload="fused_add_rms_norm [4096,4096] bf16, eps 1e-6 (configs[0] shape)",
+                    cpu=(cpu, 4 * M * N * 4 + N * 4, "oracle fused_add_rms_norm (torch CPU, fp32 in / fp64 math) on the full [4096,4096]"))
+
+    def wl_mm(M, N, K, name, b_t=False, bias=False, bound="mfma"):
+        def make():
+            torch.manual_seed(0)
+            a = (torch.randn(M, K) / math.sqrt(K)).to(bf16).to(dev)
+            b = ((torch.randn(N, K) / math.sqrt(K)).to(bf16).to(dev).t() if b_t
+                 else (torch.randn(K, N) / math.sqrt(K)).to(bf16).to(dev))
+            bi = (torch.randn(N) * 0.02).to(bf16).to(dev) if bias else None
+            state = {}
+
+            def run(i):
+                state["c"] = flag_gems.addmm(bi, a, b) if bias else flag_gems.mm(a, b)
+
+            rows = min(M, 512)
+            ac, bc = a[:rows].cpu().float(), b.cpu().float()
+
+            def cpu():
+                torch.mm(ac, bc)
+
+            if bound == "hbm":
+                work = (M * K + K * N + M * N) * 2
+                cw = (rows * K + K * N + rows * N) * 2
+            else:
+                work = M * N * (2 * K + 1) if bias else 2 * M * N * K
+                cw = 2 * rows * N * K
+            d = dict(run=run, work=work, bound=bound, dtype="bf16", workload=name,
+                     cpu=(cpu, cw, "torch.mm on the host in fp32, first %d rows of A" % rows))
+            d["post"] = lambda: {"schedule": {1: "data-parallel", 2: "stream-K"}.get(_gemm.last_schedule())}
+            return d
+        return make
+
+    def build_paged(lens, Hk, D, bs, k, v):
+        nblk = sum((l + bs - 1) // bs for l in lens)
+        perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(0))
+        bt = torch.zeros(len(lens), (max(lens) + bs - 1) // bs, dtype=torch.int32)
+        slots, o = [], 0
+        for i, l in enumerate(lens):
+            n = (l + bs - 1) // bs
+            bt[i, :n] = perm[o:o + n]
+            o += n
+            t = torch.arange(l)
+            slots.append(bt[i, t // bs].long() * bs + t % bs)
+        slots = torch.cat(slots).to(dev)
+        kc = torch.zeros(nblk, bs, Hk, D, dtype=bf16, device=dev)
+        vc = torch.zeros_like(kc)
+        flag_gems.reshape_and_cache_flash(k, v, kc, vc, slots, "auto", None, None)
+        return kc, vc, bt.to(dev), slots
+
+    def wl_attn_c4():
+        L = torch.randint(512, 4097, (16,), generator=torch.Generator().manual_seed(0)).tolist()
+        Hq, Hk, D, bs = 32, 8, 128, 16
+        tot = sum(L)
+        torch.manual_seed(0)
+        q = torch.randn(tot, Hq, D).to(bf16).to(dev)
+        k = torch.randn(tot, Hk, D).to(bf16).to(dev)
+        v = torch.randn(tot, Hk, D).to(bf16).to(dev)
+        kc, vc, bt, _ = build_paged(L, Hk, D, bs, k, v)
+        cu = torch.tensor([0] + L, dtype=torch.int32).cumsum(0, dtype=torch.int32).to(dev)
+        sk = torch.tensor(L, dtype=torch.int32, device=dev)
+        state = {}
+
+        def run(i):
+            state["o"] = flag_gems.flash_attn_varlen_func(q, kc, vc, max(L), cu, max(L), seqused_k=sk, causal=True, block_table=bt)
+
+        flops = sum(4 * D * Hq * l * (l + 1) // 2 for l in L)
+        i_short = min(range(16), key=lambda i: L[i])
+        ls = L[i_short]
+        off = sum(L[:i_short])
+        qc = q[off:off + ls].cpu()
+        kcc, vcc, btc = kc.cpu(), vc.cpu(), bt[i_short:i_short + 1].cpu()
+
+        def cpu():
+            O.paged_attention(qc, kcc, vcc, [ls], [ls], btc, D ** -0.5, compute_dtype=torch.float32)
+
+        return dict(run=run, work=flops, bound="mfma", dtype="bf16",
+                    workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
+                    cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
+
+    def wl_layer_c5():
+        torch.manual_seed(0)
+        Hd, H, D, F, bs, B, S = 4096, 32, 128, 11008, 16, 8, 2048
+        T = B * S
+        wqkv = (torch.randn(3 * Hd, Hd) * 0.02).to(bf16).to(dev)
+        wo = (torch.randn(Hd, Hd) * 0.02).to(bf16).to(dev)
+        wgu = (torch.randn(2 * F, Hd) * 0.02).to(bf16).to(dev)
+        wd = (torch.randn(Hd, F) * 0.02).to(bf16).to(dev)
+        n1 = torch.ones(Hd, dtype=bf16, device=dev)
+        n2 = torch.ones(Hd, dtype=bf16, device=dev)
+        h = torch.randn(T, Hd).to(bf16).to(dev)
+        pos = torch.arange(S).repeat(B).to(dev)
+        cos, sin = O.rope_cos_sin(S, D, device=dev)
+        lens = [S] * B
+        zk = torch.zeros(T, H, D, dtype=bf16, device=dev)
+        kc, vc, bt, slots = build_paged(lens, H, D, bs, zk, zk)
+        del zk
+        cu = torch.arange(0, T + 1, S, dtype=torch.int32, device=dev)
+        sk = torch.full((B,), S, dtype=torch.int32, device=dev)
+        lib = torch.library.Library("aten", "IMPL")
+        flag_gems.enable(lib=lib)
+        marks = []
+
+        def run(i, record=None):
+            def mark(name):
+                if record is not None:
+                    e = torch.cuda.Event(enable_timing=True)
+                    e.record()
+                    record.append((name, e))
+            mark("start")
+            x = torch.nn.functional.rms_norm(h, [Hd], n1, 1e-5); mark("rms_norm")
+            qkv = torch.mm(x, wqkv.t()); mark("mm_qkv")
+            q, k, v = (qkv[:, j * Hd:(j + 1) * Hd].view(T, H, D) for j in range(3))
+            flag_gems.apply_rotary_pos_emb(q, k, cos, sin, pos, False, inplace=True); mark("rope")
+            flag_gems.reshape_and_cache_flash(k, v, kc, vc, slots, "auto", None, None); mark("reshape_and_cache_flash")
+            a = flag_gems.flash_attn_varlen_func(q, kc, vc, S, cu, S, seqused_k=sk, causal=True, block_table=bt); mark("flash_attn_varlen")
+            o = torch.mm(a.view(T, Hd), wo.t()); mark("mm_o")
+            y, r = flag_gems.fused_add_rms_norm(o, h.clone(), [Hd], n2, 1e-5); mark("fused_add_rms_norm(+clone)")
+            gu = torch.mm(y, wgu.t()); mark("mm_gate_up")
+            act = flag_gems.silu_and_mul(gu[:, :F], gu[:, F:]); mark("silu_and_mul")
+            out = torch.mm(act, wd.t()); mark("mm_down")
+            out += r; mark("residual_add")
+            return out
+
+        lin = 2 * T * Hd * (3 * Hd + Hd + 2 * F + F)
+        att = B * 4 * D * H * S * (S + 1) // 2
+
+        def post():
+            rec = []
+            run(0, rec)
+            torch.cuda.synchronize()
+            ops = {}
+            for (n0, e0), (n1_, e1) in zip(rec[:-1], rec[1:]):
+                ops[n1_] = round(e0.elapsed_time(e1), 4)
+            lib._destroy()
+            return {"per_op_ms": ops, "linear_flop": lin, "attention_flop": att}
+
+        return dict(run=run, work=lin + att, bound="mfma", dtype="bf16",
+                    workload="Llama-2-7B decoder layer forward under flag_gems.enable(), 8 x 2048-token prefill, paged KV (configs[4])",
+                    cpu=None, post=post)
+
+    workloads = {
+        "softmax_c2": wl_softmax_c2,
+        "fused_add_rms_norm_c1": wl_fused_add_rms_norm_c1,
+        "mm_c3a_8192": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B row-major (configs[2]a)"),
+        "mm_c3a_8192_nt": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B = W^T column-major (configs[2]a, weight layout)", b_t=True),
+        "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),
+        "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
+        "flash_attn_c4": wl_attn_c4,
+        "decoder_layer_c5": wl_layer_c5,
+    }
+    if args.workload not in workloads:
+        print("bench.py: unknown workload %s (have: %s)" % (args.workload, ", ".join(workloads)), file=sys.stderr)
+        sys.exit(2)
+
+    def measure(name, steps, warmup, with_cpu):
+        w = workloads[name]()
+        wall_ms, ev_ms = timed(w["run"], steps, warmup)
+        res = {"workload": w["workload"], "ms_per_step": round(wall_ms, 5), "kernel_ms": round(ev_ms, 5),
+               "roofline": roofline(w["bound"], w["work"], ev_ms)}
+        if w["bound"] == "hbm":
+            res["value"], res["unit"] = round(w["work"] / wall_ms / 1e6, 1), "GB/s"
+        else:
+            res["value"], res["unit"] = round(w["work"] / wall_ms / 1e9, 1), "TFLOP/s"
+        if "post" in w and w["post"] is not None:
+            res.update(w["post"]())
+        if with_cpu and w.get("cpu"):
+            fn, cwork, note = w["cpu"]
+            t = cpu_time(fn)
+            if w["bound"] == "hbm":
+                res["cpu_baseline"] = {"value": round(cwork / t / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port", "sample": note}
+            else:
+                res["cpu_baseline"] = {"value": round(cwork / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port", "sample": note}
+        del w
+        torch.cuda.empty_cache()
+        return res
+
+    head = measure(args.workload, args.steps, args.warmup, not args.no_cpu)
+    extra = {}
+    if not args.no_extra:
+        for name in workloads:
+            if name == args.workload:
+                continue
+            steps = max(3, min(args.steps, 20))
+            if name == "decoder_layer_c5":
+                steps = min(steps, 5)
+            extra[name] = measure(name, steps, min(args.warmup, 3), not args.no_cpu)
+
+    line = {
+        "metric": "% of roofline: GB/s for norm/softmax, TFLOP/s for mm/flash-attn, 1xMI355X",
+        "value": head["value"],
+        "unit": head["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": head["workload"]},
+        "roofline": head["roofline"],
+        "cpu_baseline": head.get("cpu_baseline"),
+        "configs": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

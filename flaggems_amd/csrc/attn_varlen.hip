@@ -1,5 +1,344 @@
+// Variable-length attention forward over a paged KV cache for gfx950 (FA2 semantics).
+//
+// Work split.  A workgroup is 4 waves; a wave owns RW = 32 query rows of one query head and keeps
+// their running max / sum and the output accumulator in registers for the whole KV sweep.  The 4
+// waves of a workgroup share every K/V tile through LDS, and they are chosen to need the same
+// keys: with grouped-query attention the workgroup takes HPB = 4 (or 2) query heads that map to
+// the same KV head over one 32-row (64-row) block, so each K/V byte fetched from the cache feeds
+// 4 heads; with HPB = 1 the waves take 4 consecutive row blocks of one head.
+//
+// Matrix products (MFMA 32x32x16, fp32 accumulate), both computed transposed so that a lane owns
+// ONE query row (lane % 32) and the softmax reductions stay inside the lane:
+//   S^T[key, q] = K[key, :] . Q[q, :]      A operand = K tile rows (LDS, d-contiguous),
+//                                          B operand = Q (registers, loaded once);
+//   O^T[d, q]  += V^T[d, key] . P^T[key, q] A operand = V^T tile rows (LDS, key-contiguous),
+//                                          B operand = P^T straight from the S^T accumulators.
+// The S^T accumulator of lane (q, h = lane/32) holds rows (i/4)*8 + 4h + i%4, i = 0..15.  K rows
+// are fed to the MFMA through the bit permutation sigma below so that those 16 values are keys
+// 16*(i/8) + 8h + i%8: registers 8t..8t+7 are then exactly the 8 consecutive keys the B operand
+// of the t-th PV MFMA wants from this lane, and no data moves between the two products.
+//
+// Softmax runs in the base-2 domain: t = logit * log2(e), p = exp2(t - max), with the logit being
+// scale*S, or softcap*tanh(scale*S/softcap), plus the ALiBi bias, and -inf where masked (keys
+// past the sequence, causal / sliding-window bounds aligned to the bottom-right corner).
+// lse = max*ln2 + ln(sum); rows with no visible key give out = 0, lse = +inf.
+//
+// K/V tiles of 64 keys are gathered page by page (block_table -> page -> row), 16 bytes per lane,
+// zero-filled past the sequence end so stale cache contents can never reach the accumulators.
+// V is transposed on its way into LDS (8x8 register transposes with v_perm_b32).
 #include "fg_common.h"
-extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* p, void* stream) {
-  fg_set_error("flash_attn_varlen_fwd: not built yet");
-  return FG_ERR_UNSUPPORTED;
+
+namespace {
+
+constexpr int kBN = 64;        // keys per tile
+constexpr int kRW = 32;        // query rows per wave
+constexpr int kVtPitch = 144;  // V^T tile: row = 64 keys * 2 B + 16 B pad
+
+template <typename T> struct AttnMfma;
+template <> struct AttnMfma<bf16_t> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct AttnMfma<f16_t> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct AttnArgs {
+  FgFlashParams p;
+  int hpb;            // query heads per workgroup (1, 2 or 4)
+  int rows_per_block; // query rows per workgroup = 128 / hpb
+  int has_right, has_left;  // mask bounds in use
+  int right_off_w, left_off_w;  // window_right / window_left as used by the bounds
+  float scale_log2;   // softmax_scale * log2(e)   (softcap == 0)
+  float cap_in, cap_out_log2;  // softcap: t = cap_out_log2 * tanh(S * cap_in)
+};
+
+// MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
+__device__ __forceinline__ int sigma(int s) {
+  return ((s >> 4) & 1) * 16 + ((s >> 2) & 1) * 8 + ((s >> 3) & 1) * 4 + (s & 3);
+}
+
+template <typename T, int DP>
+__global__ __launch_bounds__(256) void attn_varlen_kernel(AttnArgs a) {
+  typedef typename AttnMfma<T>::Frag Frag;
+  constexpr int KPITCH = DP * 2 + 16;  // bytes per K tile row
+  constexpr int KS = DP / 16;          // MFMA k-steps over the head dim
+  constexpr int DT = DP / 32;          // 32-row output sub-tiles over the head dim
+  __shared__ __attribute__((aligned(16))) char k_lds[kBN * KPITCH];
+  __shared__ __attribute__((aligned(16))) char vt_lds[DP * kVtPitch];
+
+  const FgFlashParams& p = a.p;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, ql = lane & 31;
+  const int m_block = blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+
+  const int q_bos = p.cu_seqlens_q[b];
+  const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
+  const int k_len = p.seqused_k[b];
+  const int block_row0 = m_block * a.rows_per_block;
+  if (block_row0 >= q_len) return;
+
+  // wave -> (head, row block)
+  const int waves_per_head = 4 / a.hpb;
+  const int head = hgroup * a.hpb + wave / waves_per_head;
+  const int row0 = block_row0 + (wave % waves_per_head) * kRW;  // first row of this wave in the sequence
+  const int kv_head = head / (p.Hq / p.Hk);
+  const int D = p.D;
+
+  // ---- key range of the workgroup --------------------------------------------------------------
+  const int shift = k_len - q_len;  // bottom-right alignment
+  int n_max = (k_len + kBN - 1) / kBN;
+  if (a.has_right) {
+    const int last = block_row0 + a.rows_per_block + shift + a.right_off_w;  // exclusive key bound
+    const int lim = last <= 0 ? 0 : (last + kBN - 1) / kBN;
+    n_max = n_max < lim ? n_max : lim;
+  }
+  int n_min = 0;
+  if (a.has_left) {
+    const int first = block_row0 + shift - a.left_off_w;
+    n_min = first <= 0 ? 0 : first / kBN;
+  }
+
+  // ---- Q fragments (B operand): lane (q = ql, half) holds d = 16*ks + 8*half .. +8 ----------------
+  Frag qf[KS];
+  {
+    const int qrow = row0 + ql;
+    const bool row_ok = qrow < q_len;
+    const T* qp = (const T*)p.q + (int64_t)(q_bos + (row_ok ? qrow : 0)) * p.q_row_stride + (int64_t)head * p.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 16 + half * 8;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok && d < D) v = *reinterpret_cast<const u32x4*>(qp + d);
+      qf[ks] = __builtin_bit_cast(Frag, v);
+    }
+  }
+
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  float slope = 0.f;
+  if (p.alibi_slopes != nullptr) slope = p.alibi_slopes[(int64_t)b * p.alibi_batch_stride + head] * 1.4426950408889634f;
+  const bool softcap = p.softcap > 0.f;
+
+  const int32_t* btab = p.block_table + (int64_t)b * p.block_table_stride;
+  const T* kbase = (const T*)p.k_cache + (int64_t)kv_head * p.k_head_stride;
+  const T* vbase = (const T*)p.v_cache + (int64_t)kv_head * p.v_head_stride;
+  const int page_size = p.page_size;
+  const int CPR = D / 8;  // 16-byte chunks per K/V row
+
+  const bool wave_rows_ok = row0 < q_len;
+  const int wave_row_last = (row0 + kRW - 1 < q_len ? row0 + kRW - 1 : q_len - 1);
+
+  for (int nb = n_min; nb < n_max; ++nb) {
+    const int key0 = nb * kBN;
+    __syncthreads();  // the previous tile is fully consumed
+    if (tid >= 128) {
+      // K tile: 16-byte chunks, row-major copy.  chunk index -> (key, d-chunk)
+      for (int idx = tid - 128; idx < kBN * (DP / 8); idx += 128) {
+        const int r = idx / (DP / 8), c = idx - r * (DP / 8);
+        const int key = key0 + r;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (key < k_len && c < CPR) {
+          const int pg = key / page_size;
+          const int64_t page = btab[pg];
+          v = *reinterpret_cast<const u32x4*>(kbase + page * p.k_page_stride + (int64_t)(key - pg * page_size) * p.k_row_stride + c * 8);
+        }
+        *reinterpret_cast<u32x4*>(k_lds + r * KPITCH + c * 16) = v;
+      }
+    } else {
+      // V tile: 8(key) x 8(d) blocks, transposed to V^T[d][key].  block index -> (d-chunk, key block)
+      for (int blk = tid; blk < (kBN / 8) * (DP / 8); blk += 128) {
+        const int c = blk % (DP / 8), kb = blk / (DP / 8);
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = key0 + kb * 8 + j;
+          v[j] = u32x4{0u, 0u, 0u, 0u};
+          if (key < k_len && c < CPR) {
+            const int pg = key / page_size;
+            const int64_t page = btab[pg];
+            v[j] = *reinterpret_cast<const u32x4*>(vbase + page * p.v_page_stride + (int64_t)(key - pg * page_size) * p.v_row_stride + c * 8);
+          }
+        }
+#pragma unroll
+        for (int dd = 0; dd < 8; ++dd) {
+          const unsigned sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+          u32x4 o;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) o[w] = __builtin_amdgcn_perm(v[2 * w + 1][dd >> 1], v[2 * w][dd >> 1], sel);
+          *reinterpret_cast<u32x4*>(vt_lds + (c * 8 + dd) * kVtPitch + kb * 16) = o;
+        }
+      }
+    }
+    __syncthreads();
+
+    if (!wave_rows_ok) continue;
+    // tile visibility for this wave's rows
+    if (a.has_right && key0 > wave_row_last + shift + a.right_off_w) continue;
+    if (a.has_left && key0 + kBN - 1 < row0 + shift - a.left_off_w) continue;
+
+    // ---- S^T = K . Q^T ---------------------------------------------------------------------------
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s_acc[kt][e] = 0.f;
+      const char* krow = k_lds + (kt * 32 + sigma(ql)) * KPITCH + half * 16;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Frag kf = *reinterpret_cast<const Frag*>(krow + ks * 32);
+        s_acc[kt] = AttnMfma<T>::mma(kf, qf[ks], s_acc[kt]);
+      }
+    }
+
+    // ---- logits in the base-2 domain, masks ------------------------------------------------------
+    const int qrow = row0 + ql;  // this lane's query row
+    const bool need_mask = (key0 + kBN > k_len) || (a.has_right && key0 + kBN - 1 > row0 + shift + a.right_off_w) ||
+                           (a.has_left && key0 < wave_row_last + shift - a.left_off_w);
+    const int col_hi = a.has_right ? (qrow + shift + a.right_off_w < k_len - 1 ? qrow + shift + a.right_off_w : k_len - 1)
+                                   : k_len - 1;
+    const int col_lo = a.has_left ? qrow + shift - a.left_off_w : 0;
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int col = key0 + kt * 32 + (e >> 3) * 16 + half * 8 + (e & 7);
+        float t = s_acc[kt][e];
+        if (softcap) t = a.cap_out_log2 * tanhf(t * a.cap_in);
+        else t = t * a.scale_log2;
+        if (p.alibi_slopes != nullptr) {
+          if (p.is_causal) t += slope * (float)(col - k_len + 1);
+          else t -= slope * fabsf((float)(col - shift - qrow));
+        }
+        if (need_mask && (col > col_hi || col < col_lo)) t = -INFINITY;
+        s_acc[kt][e] = t;
+        tmax = fmaxf(tmax, t);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m_run - m_use);
+    float psum = 0.f;
+    Frag pf[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        T tmp[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float pv = exp2f(s_acc[kt][t2 * 8 + e] - m_use);
+          psum += pv;
+          tmp[e] = (T)pv;
+        }
+        pf[kt * 2 + t2] = *reinterpret_cast<Frag*>(tmp);
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+
+    // ---- O^T = O^T * alpha + V^T . P^T ------------------------------------------------------------
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
+      const char* vrow = vt_lds + (dt * 32 + ql) * kVtPitch + half * 16;
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) {
+        Frag vf = *reinterpret_cast<const Frag*>(vrow + t4 * 32);
+        o_acc[dt] = AttnMfma<T>::mma(vf, pf[t4], o_acc[dt]);
+      }
+    }
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------
+  const int qrow = row0 + ql;
+  if (qrow >= q_len) return;
+  const bool empty = l_run == 0.f || l_run != l_run;
+  const float inv = empty ? 1.f : 1.f / l_run;
+  if (p.lse != nullptr && half == 0) {
+    p.lse[(int64_t)head * p.total_q + q_bos + qrow] = empty ? INFINITY : m_run * 0.6931471805599453f + logf(l_run);
+  }
+  T* op = (T*)p.out + (int64_t)(q_bos + qrow) * p.o_row_stride + (int64_t)head * p.o_head_stride;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = dt * 32 + g * 8 + half * 4;
+      if (d < D) {  // D is a multiple of 8, so a group of 4 is all inside or all outside
+        Pack<T, 4> o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.v[e] = (T)(o_acc[dt][g * 4 + e] * inv);
+        st_pack<T, 4>(op + d, o);
+      }
+    }
+}
+
+template <typename T>
+int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
+  const int D = a.p.D;
+  if (D <= 64) hipLaunchKernelGGL((attn_varlen_kernel<T, 64>), grid, dim3(256), 0, st, a);
+  else if (D <= 128) hipLaunchKernelGGL((attn_varlen_kernel<T, 128>), grid, dim3(256), 0, st, a);
+  else if (D <= 192) hipLaunchKernelGGL((attn_varlen_kernel<T, 192>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((attn_varlen_kernel<T, 256>), grid, dim3(256), 0, st, a);
+  return fg_check_launch("flash_attn_varlen_fwd");
+}
+
+}  // namespace
+
+extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
+  FG_REQUIRE(pp != nullptr, FG_ERR_INVALID, "flash_attn_varlen_fwd: null params");
+  const FgFlashParams& p = *pp;
+  FG_REQUIRE(p.dtype == FG_F16 || p.dtype == FG_BF16, FG_ERR_INVALID,
+             "flash_attn_varlen_fwd: only fp16 and bf16 are supported (dtype %d)", p.dtype);
+  FG_REQUIRE(p.batch >= 0 && p.total_q >= 0, FG_ERR_INVALID, "flash_attn_varlen_fwd: negative size");
+  if (p.batch == 0 || p.total_q == 0) return FG_OK;
+  FG_REQUIRE(p.q && p.k_cache && p.v_cache && p.out && p.cu_seqlens_q && p.seqused_k && p.block_table, FG_ERR_INVALID,
+             "flash_attn_varlen_fwd: null pointer (q, k, v, out, cu_seqlens_q, seqused_k and block_table are required)");
+  FG_REQUIRE(p.D > 0 && p.D <= 256 && p.D % 8 == 0, FG_ERR_INVALID,
+             "flash_attn_varlen_fwd: head dim %d must be a multiple of 8 and at most 256", p.D);
+  FG_REQUIRE(p.Hq > 0 && p.Hk > 0 && p.Hq % p.Hk == 0, FG_ERR_INVALID,
+             "flash_attn_varlen_fwd: %d query heads are not a multiple of %d kv heads", p.Hq, p.Hk);
+  FG_REQUIRE(p.page_size > 0, FG_ERR_INVALID, "flash_attn_varlen_fwd: page size must be positive");
+  FG_REQUIRE(p.max_seqlen_q > 0, FG_ERR_INVALID, "flash_attn_varlen_fwd: max_seqlen_q must be positive");
+  auto al = [](const void* q, int64_t s1, int64_t s2) { return fg_aligned(q, 16) && s1 % 8 == 0 && s2 % 8 == 0; };
+  FG_REQUIRE(al(p.q, p.q_row_stride, p.q_head_stride) && al(p.k_cache, p.k_row_stride, p.k_head_stride) &&
+                 al(p.v_cache, p.v_row_stride, p.v_head_stride) && p.k_page_stride % 8 == 0 && p.v_page_stride % 8 == 0,
+             FG_ERR_UNSUPPORTED, "flash_attn_varlen_fwd: q/k/v rows must be 16-byte aligned");
+  FG_REQUIRE(fg_aligned(p.out, 8) && p.o_row_stride % 4 == 0 && p.o_head_stride % 4 == 0, FG_ERR_UNSUPPORTED,
+             "flash_attn_varlen_fwd: out rows must be 8-byte aligned");
+  FG_REQUIRE(p.batch < 65536 && p.Hq < 65536, FG_ERR_UNSUPPORTED, "flash_attn_varlen_fwd: batch/heads exceed the grid");
+
+  AttnArgs a;
+  a.p = p;
+  const int ratio = p.Hq / p.Hk;
+  a.hpb = ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1);
+  a.rows_per_block = 128 / a.hpb;
+  // Mask bounds (bottom-right aligned): keys col with col > row + shift + right or col < row + shift - left are
+  // masked.  causal forces right = 0; a one-sided window leaves the other side open.
+  int wl = p.window_left, wr = p.window_right;
+  if (p.is_causal) wr = 0;
+  a.has_right = wr >= 0;
+  a.has_left = wl >= 0;
+  a.right_off_w = wr >= 0 ? wr : 0;
+  a.left_off_w = wl >= 0 ? wl : 0;
+  const float log2e = 1.4426950408889634f;
+  a.scale_log2 = p.softmax_scale * log2e;
+  a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
+  a.cap_out_log2 = p.softcap * log2e;
+  dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
+  hipStream_t st = (hipStream_t)stream;
+  if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
+  return attn_dispatch<bf16_t>(a, grid, st);
 }

@@ -23,6 +23,7 @@ SOURCES = [
     "silu_mul.hip",
     "gemm.hip",
     "gemm_skinny.hip",
+    "gemm_streamk.hip",
     "attn_varlen.hip",
 ]
 

@@ -5,9 +5,10 @@
 namespace fgk {
 
 // implemented in gemm_skinny.hip
-int skinny_supported(const GemmArgs& g, int dtype, bool b_n_contig_vec, bool a_k_contig_vec);
+int skinny_supported(const GemmArgs& g, int dtype, int amode, int bmode);
 size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int num_cu);
-int skinny_launch(const GemmArgs& g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st);
+int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, size_t workspace_bytes, int num_cu,
+                  hipStream_t st);
 // implemented in gemm_streamk.hip
 size_t streamk_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int num_cu);
 int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace, size_t workspace_bytes, int num_cu,
@@ -169,7 +170,7 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
 
   // ---- schedule --------------------------------------------------------------------------------
   // Skinny problems (M <= 16 rows) are bandwidth-bound streams of B: their own stream-K kernel.
-  const int sk_ok = skinny_supported(g, ab_dtype, bmode == LOAD_MN, amode == LOAD_K);
+  const int sk_ok = skinny_supported(g, ab_dtype, amode, bmode);
   bool use_skinny = false, use_streamk = false;
   if (schedule != FG_SCHED_DATA_PARALLEL && workspace != nullptr) {
     if (sk_ok) {
@@ -180,13 +181,11 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
         if (schedule == FG_SCHED_STREAM_K) {
           use_streamk = true;
         } else {
-          // auto: stream-K when the data-parallel grid would leave most of the last wave idle and K
-          // is deep enough to split (at least two K steps per workgroup).
+          // auto: stream-K when the tiles cannot fill half the machine and K is deep enough to hand
+          // every workgroup at least four K steps; fuller grids run data-parallel.
           const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
           const int64_t iters = fg_cdiv(K, 64);
-          const int64_t rem = tiles % cu;
-          use_streamk = rem != 0 && rem * 10 <= (int64_t)cu * 8 && tiles < (int64_t)cu * 4 &&
-                        (tiles % cu) * iters >= 2 * (int64_t)cu;
+          use_streamk = tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;
         }
       }
     }
@@ -198,7 +197,7 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
   }
   if (use_skinny) {
     if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;
-    return skinny_launch(g, ab_dtype, workspace, workspace_bytes, cu, st);
+    return skinny_launch(g, ab_dtype, sk_ok, workspace, workspace_bytes, cu, st);
   }
   if (use_streamk) {
     if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;

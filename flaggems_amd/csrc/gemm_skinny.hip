@@ -1,8 +1,276 @@
+// Skinny GEMM (M <= 16) with a stream-K schedule for gfx950.
+//
+// With so few rows the product is a bandwidth-bound stream of B (arithmetic intensity ~ M flop per
+// byte), so the schedule's only job is to keep every CU streaming an equal share of B.  The output
+// is cut into tiles of 16 rows x 128 columns and K into steps of 32; the (tile, k-step) units, in
+// tile-major order, are dealt in equal contiguous ranges to one persistent workgroup per CU
+// (stream-K).  A workgroup walks its range segment by segment (a segment = its units inside one
+// tile); its 8 waves split the segment's k-steps, accumulate in registers with
+// v_mfma_f32_16x16x32_{bf16,f16}, and add their accumulators up through LDS.
+//
+// A segment that covers its tile's whole K range is finished on the spot.  A tile split between
+// workgroups is finished by whichever of them arrives LAST: every contributor writes its fp32
+// partial tile to its own slot of the workspace (device-coherent stores), then takes a ticket from
+// the tile's counter (one device-scope atomic add).  The contributor that draws the last ticket
+// reads all slots of the tile in workgroup order, adds them in that fixed order (so the result is
+// bit-reproducible whoever finishes), applies the epilogue, stores C and resets the counter.
+// Nobody ever waits for anybody, so there is nothing to deadlock or time out.
+//
+// B feeds the MFMA "A" operand (rows = output columns), the activations feed the "B" operand, so
+// the accumulators hold C^T: lane (m = lane%16, g = lane/16) owns column slots 4g..4g+3.
+//   B row-major (N contiguous): a lane loads an 8(k) x 8(n) block as eight 16-byte rows and
+//     transposes it in registers (v_perm_b32); MFMA c of 8 then covers columns n0 + 8*slot + c.
+//   B = W^T (K contiguous): a lane loads 16 bytes = 8 k of one column directly; MFMA c covers
+//     columns n0 + 16*c + slot.
+#include <atomic>
+#include <stdlib.h>
 #include "gemm_tile.h"
+
 namespace fgk {
-int skinny_supported(const GemmArgs&, int, bool, bool) { return 0; }
-size_t skinny_workspace_bytes(int64_t, int64_t, int64_t, int) { return 0; }
-int skinny_launch(const GemmArgs&, int, void*, size_t, int, hipStream_t) { return FG_ERR_UNSUPPORTED; }
-size_t streamk_workspace_bytes(int64_t, int64_t, int64_t, int, int) { return 0; }
-int streamk_launch(GemmArgs, int, int, int, void*, size_t, int, hipStream_t) { return FG_ERR_UNSUPPORTED; }
+
+namespace {
+
+constexpr int kTileN = 128, kStepK = 32, kWaves = 8, kBlock = kWaves * 64;
+constexpr int kTileElems = 16 * kTileN;  // fp32 partial tile
+constexpr int kEPT = kTileElems / kBlock;  // tile elements per thread in the block-wide phases
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x4v mma(Frag a, Frag b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x4v mma(Frag a, Frag b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct SkinnyArgs {
+  GemmArgs g;
+  int tiles_n, ksteps;  // output tiles along N, k-steps per tile
+  int64_t per, rem;     // units per workgroup, and how many workgroups take one more
+  int workers;
+  float* partials;      // [workers][2][kTileElems]
+  unsigned* tickets;    // [kMaxWorkers], zero between launches
+};
+
+__device__ __host__ __forceinline__ int64_t range_begin(int64_t per, int64_t rem, int64_t w) {
+  return w * per + (w < rem ? w : rem);
 }
+// workgroup that owns unit u
+__device__ __forceinline__ int worker_of(int64_t per, int64_t rem, int64_t u) {
+  const int64_t big = rem * (per + 1);
+  return (int)(u < big ? u / (per + 1) : rem + (u - big) / per);
+}
+
+// Device-coherent accesses to the partial tiles: they must be seen by CUs behind another L2.
+__device__ __forceinline__ void st_coherent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_coherent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, bool B_ROWMAJOR>
+__global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
+  typedef typename Mfma16<T>::Frag Frag;
+  __shared__ float red[kWaves][kTileElems];  // accumulators of every wave, element-major [c][i][lane]
+  __shared__ unsigned ticket_s;
+  const GemmArgs& g = a.g;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, grp = lane >> 4;
+  const int w = blockIdx.x;
+  const int M = (int)g.M, N = (int)g.N, K = (int)g.K;
+  const T* A = (const T*)g.A;
+  const T* B = (const T*)g.B;
+
+  const int64_t u_begin = range_begin(a.per, a.rem, w);
+  const int64_t u_end = range_begin(a.per, a.rem, w + 1);
+  int64_t u = u_begin;
+  while (u < u_end) {
+    const int tile = (int)(u / a.ksteps);
+    const int64_t tile_begin = (int64_t)tile * a.ksteps;
+    const int64_t tile_end = tile_begin + a.ksteps;
+    const int ks0 = (int)(u - tile_begin);
+    const int ks1 = (int)((u_end < tile_end ? u_end : tile_end) - tile_begin);
+    const int n0 = tile * kTileN;
+
+    // ---- this wave's share of the segment's k-steps --------------------------------------------
+    const int nsteps = ks1 - ks0;
+    const int share = (nsteps + kWaves - 1) / kWaves;
+    const int my0 = ks0 + wave * share;
+    const int my1 = (my0 + share < ks1) ? my0 + share : ks1;
+
+    f32x4v acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = f32x4v{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 bv[8], bn[8];
+    u32x4 av, an;
+    auto load_step = [&](int ks, u32x4 (&bd)[8], u32x4& ad) {
+      const int k0 = ks * kStepK;
+      const int ka = k0 + grp * 8;
+      ad = u32x4{0u, 0u, 0u, 0u};
+      if (m < M && ka < K) ad = *reinterpret_cast<const u32x4*>(A + (int64_t)m * g.sam + ka);
+      if constexpr (B_ROWMAJOR) {
+        const int n = n0 + m * 8;  // m doubles as the column-slot index of this lane
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int k = k0 + grp * 8 + j;
+          bd[j] = u32x4{0u, 0u, 0u, 0u};
+          if (k < K && n < N)
+            bd[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B + (int64_t)k * g.sbk + n));
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int n = n0 + 16 * c + m;
+          bd[c] = u32x4{0u, 0u, 0u, 0u};
+          if (ka < K && n < N)
+            bd[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B + (int64_t)n * g.sbn + ka));
+        }
+      }
+    };
+    auto compute = [&](u32x4 (&bd)[8], u32x4& ad) {
+      const Frag af = __builtin_bit_cast(Frag, ad);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        u32x4 o;
+        if constexpr (B_ROWMAJOR) {
+          // column c of the 8x8 block as a K-run: dword d = { k = 2d (low half), k = 2d+1 (high half) }
+          const unsigned sel = (c & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) o[d] = __builtin_amdgcn_perm(bd[2 * d + 1][c >> 1], bd[2 * d][c >> 1], sel);
+        } else {
+          o = bd[c];
+        }
+        acc[c] = Mfma16<T>::mma(__builtin_bit_cast(Frag, o), af, acc[c]);
+      }
+    };
+    if (my0 < my1) {
+      load_step(my0, bv, av);
+      for (int ks = my0; ks < my1; ks += 2) {
+        if (ks + 1 < my1) load_step(ks + 1, bn, an);
+        compute(bv, av);
+        if (ks + 1 < my1) {
+          if (ks + 2 < my1) load_step(ks + 2, bv, av);
+          compute(bn, an);
+        }
+      }
+    }
+
+    // ---- add the 8 waves' accumulators through LDS; thread t ends up with elements t + kBlock*j --
+    __syncthreads();  // red[] of the previous segment is no longer read
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][(c * 4 + i) * 64 + lane] = acc[c][i];
+    __syncthreads();
+    float sum[kEPT];
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+      float s = 0.f;
+#pragma unroll
+      for (int v = 0; v < kWaves; ++v) s += red[v][tid + kBlock * j];
+      sum[j] = s;
+    }
+
+    bool finish = (ks0 == 0 && ks1 == a.ksteps);  // the whole tile was ours
+    if (!finish) {
+      // slot 0 of a workgroup: the segment it starts in; slot 1: a tile it enters from the left
+      float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * kTileElems;
+#pragma unroll
+      for (int j = 0; j < kEPT; ++j) st_coherent(slot + tid + kBlock * j, sum[j]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __syncthreads();  // every thread's slice of the partial tile is out
+      const int w_first = worker_of(a.per, a.rem, tile_begin);
+      const int w_last = worker_of(a.per, a.rem, tile_end - 1);
+      if (tid == 0)
+        ticket_s = __hip_atomic_fetch_add(a.tickets + w_first, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (ticket_s == (unsigned)(w_last - w_first)) {
+        finish = true;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+        for (int j = 0; j < kEPT; ++j) sum[j] = 0.f;
+        for (int w2 = w_first; w2 <= w_last; ++w2) {
+          const float* src =
+              a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * kTileElems;
+#pragma unroll
+          for (int j = 0; j < kEPT; ++j) sum[j] += ld_coherent(src + tid + kBlock * j);
+        }
+        if (tid == 0) __hip_atomic_store(a.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (finish) {
+      T* C = (T*)g.C;
+      const T* bias = (const T*)g.bias;
+#pragma unroll
+      for (int j = 0; j < kEPT; ++j) {
+        const int e = tid + kBlock * j;           // element (c, i, lane) of the tile
+        const int el = e & 63, ci = e >> 6;
+        const int em = el & 15, eg = el >> 4;
+        const int c = ci >> 2, i = ci & 3;
+        const int n = n0 + (B_ROWMAJOR ? 8 * (4 * eg + i) + c : 16 * c + 4 * eg + i);
+        if (em < M && n < N) {
+          float v = sum[j];
+          if (bias != nullptr) v = v * g.alpha + (float)bias[(int64_t)em * g.sim + (int64_t)n * g.sin] * g.beta;
+          else if (g.alpha != 1.0f) v = v * g.alpha;
+          C[(int64_t)em * g.scm + (int64_t)n * g.scn] = (T)v;
+        }
+      }
+    }
+    u = tile_begin + ks1;
+  }
+}
+
+}  // namespace
+
+// 0: not a case for this kernel; 1: B row-major (N contiguous); 2: B = W^T (K contiguous)
+int skinny_supported(const GemmArgs& g, int dtype, int amode, int bmode) {
+  if (dtype != FG_F16 && dtype != FG_BF16) return 0;
+  if (g.M > 16 || amode != LOAD_K) return 0;
+  if (g.K < 1024) return 0;  // worth it only when K is deep enough to give every CU several k-steps
+  if (bmode == LOAD_K) return 2;
+  if (bmode == LOAD_MN) return 1;
+  return 0;
+}
+
+size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int num_cu) {
+  if (M > 16 || K < 1024) return 0;
+  return kPartialOffset + (size_t)num_cu * 2 * kTileElems * sizeof(float);
+}
+
+int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, size_t workspace_bytes, int num_cu,
+                  hipStream_t st) {
+  FG_REQUIRE(workspace_bytes >= skinny_workspace_bytes(g.M, g.N, g.K, num_cu), FG_ERR_WORKSPACE,
+             "gemm(stream-K): workspace too small");
+  FG_REQUIRE(fg_aligned(workspace, 256), FG_ERR_WORKSPACE, "gemm(stream-K): workspace must be 256-byte aligned");
+  SkinnyArgs a;
+  a.g = g;
+  a.tiles_n = (int)fg_cdiv(g.N, kTileN);
+  a.ksteps = (int)fg_cdiv(g.K, kStepK);
+  const int64_t units = (int64_t)a.tiles_n * a.ksteps;
+  if (num_cu > kMaxWorkers) num_cu = kMaxWorkers;
+  a.workers = (int)(units < num_cu ? units : num_cu);
+  a.per = units / a.workers;
+  a.rem = units % a.workers;
+  char* ws = (char*)workspace;
+  a.tickets = (unsigned*)(ws + kTicketOffset);
+  a.partials = (float*)(ws + kPartialOffset);
+  dim3 grid((unsigned)a.workers), block(kBlock);
+  if (dtype == FG_BF16) {
+    if (b_kind == 1) hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, false>), grid, block, 0, st, a);
+  } else {
+    if (b_kind == 1) hipLaunchKernelGGL((gemm_skinny_kernel<f16_t, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_kernel<f16_t, false>), grid, block, 0, st, a);
+  }
+  return fg_check_launch("gemm(stream-K, skinny)");
+}
+
+}  // namespace fgk

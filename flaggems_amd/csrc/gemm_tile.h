@@ -31,6 +31,13 @@ enum { LOAD_K = 0, LOAD_MN = 1, LOAD_GEN = 2 };
 constexpr int kRowBytes = 128;   // K bytes per tile row per stage
 constexpr int kPitch = 144;      // LDS pitch of a tile row
 constexpr int kThreads = 256;
+// Stream-K workspace layout shared by every kernel that uses it: a fixed table of ticket counters
+// (indexed by the first workgroup that contributes to a split tile, so kMaxWorkers entries are
+// enough), then the fp32 partial tiles.  Only tickets ever live in the table, and every kernel
+// returns them to zero, so kernels with different partial-tile sizes can share one buffer.
+constexpr int kMaxWorkers = 1024;
+constexpr size_t kTicketOffset = 256;
+constexpr size_t kPartialOffset = kTicketOffset + kMaxWorkers * sizeof(unsigned);
 
 struct GemmArgs {
   const void* A;
@@ -41,13 +48,14 @@ struct GemmArgs {
   int64_t sam, sak, sbk, sbn, sim, sin, scm, scn;
   float alpha, beta;
   int tiles_m, tiles_n;
+  int tile_base;        // first tile id of a data-parallel launch (tiles below it belong to stream-K)
   // stream-K (unused by the data-parallel launch)
-  float* partials;      // [workers][BM*BN] fp32
-  unsigned* flags;      // [workers]
+  float* partials;      // [workers][2][BM*BN] fp32
+  unsigned* tickets;    // [kMaxWorkers], zero between launches
   int sk_tiles;         // tiles shared between workers
   int iters_per_tile;   // K steps per tile
   int sk_workers;       // persistent workgroups
-  unsigned epoch;       // value a ready flag must hold (changes on every launch)
+  int64_t sk_per, sk_rem;  // K steps per worker, and how many workers take one more
 };
 
 template <typename T> struct Mfma;
@@ -296,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void gemm_dp_kernel(GemmArgs g) {
   typedef TileCompute<T, BM, BN, AMODE, BMODE> TC;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
-  tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
   f32x16 acc[TC::TM][TC::TN];
 #pragma unroll
   for (int i = 0; i < TC::TM; ++i)
@@ -306,6 +314,97 @@ __global__ __launch_bounds__(kThreads) void gemm_dp_kernel(GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   TC::run(g, lds, tm, tn, 0, g.iters_per_tile, acc);
   TC::epilogue(g, tm, tn, acc);
+}
+
+// ---------------------------------------------------------------------------------------------
+// stream-K over the same tile: `sk_workers` persistent workgroups share the K steps of tiles
+// [0, sk_tiles) in equal contiguous ranges (tile-major).  A range is walked segment by segment
+// (the part inside one tile).  Segments that span a tile's whole K are finished directly.  A tile
+// split across workgroups is finished by the contributor that arrives last: each writes its fp32
+// partial tile to its own workspace slot with device-coherent stores and draws a ticket from the
+// tile's counter (device-scope atomic add); the holder of the last ticket adds all slots in
+// workgroup order (bit-reproducible whoever finishes), runs the epilogue and resets the counter.
+// No workgroup ever waits for another.
+// ---------------------------------------------------------------------------------------------
+__device__ __host__ __forceinline__ int64_t sk_begin(int64_t per, int64_t rem, int64_t w) {
+  return w * per + (w < rem ? w : rem);
+}
+__device__ __forceinline__ int sk_worker_of(int64_t per, int64_t rem, int64_t u) {
+  const int64_t big = rem * (per + 1);
+  return (int)(u < big ? u / (per + 1) : rem + (u - big) / per);
+}
+
+template <typename T, int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(kThreads) void gemm_streamk_kernel(GemmArgs g) {
+  typedef TileCompute<T, BM, BN, AMODE, BMODE> TC;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  __shared__ unsigned ticket_s;
+  const int w = blockIdx.x, tid = threadIdx.x;
+  const int64_t u_begin = sk_begin(g.sk_per, g.sk_rem, w);
+  const int64_t u_end = sk_begin(g.sk_per, g.sk_rem, w + 1);
+  int64_t u = u_begin;
+  while (u < u_end) {
+    const int tile = (int)(u / g.iters_per_tile);
+    const int64_t tile_begin = (int64_t)tile * g.iters_per_tile;
+    const int64_t tile_end = tile_begin + g.iters_per_tile;
+    const int it0 = (int)(u - tile_begin);
+    const int it1 = (int)((u_end < tile_end ? u_end : tile_end) - tile_begin);
+    int tm, tn;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
+    f32x16 acc[TC::TM][TC::TN];
+#pragma unroll
+    for (int i = 0; i < TC::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TC::TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    TC::run(g, lds, tm, tn, it0, it1, acc);
+    bool finish = (it0 == 0 && it1 == g.iters_per_tile);
+    if (!finish) {
+      // slot 0 of a workgroup: the tile it starts in; slot 1: a tile it enters from the left
+      float* slot = g.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * (BM * BN);
+#pragma unroll
+      for (int i = 0; i < TC::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TC::TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            __hip_atomic_store(slot + ((i * TC::TN + j) * 16 + e) * kThreads + tid, acc[i][j][e], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      __syncthreads();  // every thread's slice of the partial tile is out
+      const int w_first = sk_worker_of(g.sk_per, g.sk_rem, tile_begin);
+      const int w_last = sk_worker_of(g.sk_per, g.sk_rem, tile_end - 1);
+      if (tid == 0)
+        ticket_s = __hip_atomic_fetch_add(g.tickets + w_first, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (ticket_s == (unsigned)(w_last - w_first)) {
+        finish = true;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+        for (int i = 0; i < TC::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TC::TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int w2 = w_first; w2 <= w_last; ++w2) {
+          const float* src =
+              g.partials + ((int64_t)w2 * 2 + (sk_begin(g.sk_per, g.sk_rem, w2) < tile_begin ? 1 : 0)) * (BM * BN);
+#pragma unroll
+          for (int i = 0; i < TC::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TC::TN; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e)
+                acc[i][j][e] += __hip_atomic_load(src + ((i * TC::TN + j) * 16 + e) * kThreads + tid, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid == 0) __hip_atomic_store(g.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (finish) TC::epilogue(g, tm, tn, acc);
+    u = tile_begin + it1;
+  }
 }
 
 }  // namespace fgk

@@ -32,7 +32,8 @@ def _workspace(device, stream, nbytes):
     key = (device.index, stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        # zero-filled once: the kernels return their ticket counters to zero after every launch
+        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
 

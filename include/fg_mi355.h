@@ -100,7 +100,9 @@ int fg_silu_and_mul(const void* a, const void* b, void* out, int64_t rows, int64
 enum { FG_SCHED_AUTO = 0, FG_SCHED_DATA_PARALLEL = 1, FG_SCHED_STREAM_K = 2 };
 
 /* Bytes of device scratch fg_gemm needs for this problem under `schedule` (0 for the
- * data-parallel schedule).  The caller owns the buffer; it need not be zeroed.
+ * data-parallel schedule).  The caller owns the buffer: 256-byte aligned, zero-filled ONCE when
+ * it is allocated (the kernels leave their ticket counters at zero), and used by one stream at a
+ * time.
  * Stands in for the per-call `locks`/`P` allocation of src/flag_gems/ops/mm_streamk.py:488-491. */
 size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, int schedule,
                                int device);

@@ -1,0 +1,203 @@
+"""CPU oracle for the floating-point operators of the path: PyTorch ATen on the host, restating the
+expected-value computations of the reference's own accuracy tests.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product package may import this module; it is used by
+tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py, always as the checker
+and never as the thing shipped or measured as the product.
+
+Each function cites the reference test it follows (paths relative to the FlagGems tree).  The
+reference holds no golden vectors for these operators (every expectation is computed live from
+torch), so the pinning of this module is: (a) the torch library routines themselves for mm, addmm
+and softmax, (b) closed forms and invariants checked in tests/test_oracle.py for the rest.
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def to_reference(t, upcast=False):
+    """tests/accuracy_utils.py:175-186 with --ref cpu: move to the host, optionally widen to fp64."""
+    if t is None:
+        return None
+    r = t.detach().to("cpu")
+    if upcast and r.is_floating_point():
+        r = r.to(torch.float64)
+    return r
+
+
+def mm(a, b):
+    """tests/test_blas_ops.py:119-136: torch.mm on fp64 copies."""
+    return torch.mm(to_reference(a, True), to_reference(b, True))
+
+
+def addmm(bias, a, b, alpha=1, beta=1):
+    """tests/test_blas_ops.py:24-60: torch.addmm on fp64 copies."""
+    return torch.addmm(to_reference(bias, True), to_reference(a, True), to_reference(b, True), alpha=alpha, beta=beta)
+
+
+def softmax(x, dim):
+    """tests/test_reduction_ops.py:507-523: F.softmax on an fp64 copy."""
+    return F.softmax(to_reference(x, True), dim=dim)
+
+
+def rms_norm(x, weight, eps):
+    """tests/test_norm_ops.py:539-544: fp32 normalisation, cast to the input dtype, then the weight
+    multiply (the test does not widen to fp64 for this operator)."""
+    x = to_reference(x)
+    weight = to_reference(weight)
+    xf = x.to(torch.float32)
+    var = xf.pow(2).mean(-1, keepdim=True)
+    h = xf * torch.rsqrt(var + eps)
+    return weight * h.to(x.dtype)
+
+
+def fused_add_rms_norm(x, residual, weight, eps):
+    """tests/test_norm_ops.py:614-618: fp64 sum, normalise, weight.  Returns (normed, new_residual)."""
+    x = to_reference(x, True)
+    r = to_reference(residual, True)
+    w = to_reference(weight, True)
+    s = x + r
+    var = s.pow(2).mean(-1, keepdim=True)
+    return s * torch.rsqrt(var + eps) * w, s
+
+
+def rope_cos_sin(max_pos, dim, base=10000.0, dtype=torch.float32, device="cpu"):
+    """tests/test_special_ops.py:106-112: inv_freq = base^(-2i/dim), cos/sin of the outer product."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=torch.float32, device=device) / dim))
+    t = torch.arange(max_pos, dtype=torch.float32, device=device)
+    freqs = torch.outer(t, inv_freq)
+    return freqs.cos().to(dtype), freqs.sin().to(dtype)
+
+
+def _rotate_half(x):
+    h = x.shape[-1] // 2
+    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+
+def _rotate_interleave(x):
+    x1 = x[..., ::2]
+    x2 = x[..., 1::2]
+    return torch.stack((-x2, x1), dim=-1).flatten(-2)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids=None, rotary_interleaved=False):
+    """tests/test_special_ops.py:133-161: q, k in fp32, cos/sin widened to fp64 and expanded to the
+    full head dim; q*cos + rotate(q)*sin.  Without position ids the position is the index along
+    dim -3."""
+    q = to_reference(q).float()
+    k = to_reference(k).float()
+    cos = to_reference(cos, True)
+    sin = to_reference(sin, True)
+    if position_ids is None:
+        cos = cos[None, : q.size(-3), None, :]
+        sin = sin[None, : q.size(-3), None, :]
+    else:
+        pid = to_reference(position_ids).long()
+        cos = cos[pid].unsqueeze(-2)
+        sin = sin[pid].unsqueeze(-2)
+    if rotary_interleaved:
+        cos = torch.repeat_interleave(cos, 2, dim=-1)
+        sin = torch.repeat_interleave(sin, 2, dim=-1)
+        rot = _rotate_interleave
+    else:
+        cos = torch.cat([cos, cos], dim=-1)
+        sin = torch.cat([sin, sin], dim=-1)
+        rot = _rotate_half
+    return q * cos + rot(q) * sin, k * cos + rot(k) * sin
+
+
+def silu_and_mul(a, b):
+    """tests/test_binary_pointwise_ops.py:1377-1403: F.silu(a) * b on fp64 copies."""
+    return F.silu(to_reference(a, True)) * to_reference(b, True)
+
+
+def alibi_bias(slopes, seqlen_q, seqlen_k, causal):
+    """tests/test_attention_ops.py:804-816: slopes [batch, heads] -> bias broadcastable to
+    [batch, heads, seqlen_q, seqlen_k]."""
+    slopes = slopes.unsqueeze(-1).unsqueeze(-1)
+    if causal:
+        return torch.arange(-seqlen_k + 1, 1, dtype=torch.float32) * slopes
+    row = torch.arange(seqlen_q, dtype=torch.long).unsqueeze(-1)
+    col = torch.arange(seqlen_k, dtype=torch.long)
+    rel = torch.abs(row + seqlen_k - seqlen_q - col)
+    return -slopes * rel.to(slopes.dtype)
+
+
+def paged_attention(query, key_cache, value_cache, query_lens, kv_lens, block_tables, scale, causal=True,
+                    attn_bias=None, sliding_window=None, soft_cap=None, window=None, compute_dtype=None,
+                    return_lse=False):
+    """tests/test_attention_ops.py:819-881 (ref_paged_attn): per sequence, gather the pages named by
+    the block table, scaled q . k^T per head (GQA by repeat_interleave), optional soft cap, causal
+    mask triu(diagonal = kv_len - q_len + 1), optional sliding window, optional additive bias,
+    softmax cast to v's dtype, weighted sum of v.
+
+    Extensions used by this repo's tests: `causal=False`, a two-sided `window=(left, right)`,
+    `compute_dtype` (run the arithmetic in a wider type than the inputs), and `return_lse`
+    (log-sum-exp of the masked, biased logits: [heads, total_q])."""
+    query = to_reference(query)
+    key_cache = to_reference(key_cache)
+    value_cache = to_reference(value_cache)
+    block_tables = to_reference(block_tables).numpy()
+    if compute_dtype is not None:
+        query, key_cache, value_cache = (t.to(compute_dtype) for t in (query, key_cache, value_cache))
+    _, block_size, num_kv_heads, head_size = key_cache.shape
+    outputs, lses = [], []
+    start = 0
+    for i, (q_len, kv_len) in enumerate(zip(query_lens, kv_lens)):
+        q = query[start : start + q_len].clone()
+        q *= scale
+        nblk = (kv_len + block_size - 1) // block_size
+        idx = block_tables[i, :nblk]
+        k = key_cache[idx].view(-1, num_kv_heads, head_size)[:kv_len]
+        v = value_cache[idx].view(-1, num_kv_heads, head_size)[:kv_len]
+        if q.shape[1] != k.shape[1]:
+            k = torch.repeat_interleave(k, q.shape[1] // k.shape[1], dim=1)
+            v = torch.repeat_interleave(v, q.shape[1] // v.shape[1], dim=1)
+        attn = torch.einsum("qhd,khd->hqk", q, k)
+        ones = torch.ones(q_len, kv_len)
+        mask = torch.zeros(q_len, kv_len, dtype=torch.bool)
+        if causal:
+            mask |= torch.triu(ones, diagonal=kv_len - q_len + 1).bool()
+        if sliding_window is not None:
+            mask |= torch.triu(ones, diagonal=kv_len - (q_len + sliding_window) + 1).bool().logical_not()
+        if window is not None:
+            left, right = window
+            if right >= 0 and not causal:
+                mask |= torch.triu(ones, diagonal=kv_len - q_len + right + 1).bool()
+            if left >= 0:
+                mask |= torch.tril(ones, diagonal=kv_len - q_len - left - 1).bool()
+        if soft_cap is not None:
+            attn = soft_cap * torch.tanh(attn / soft_cap)
+        attn.masked_fill_(mask, float("-inf"))
+        if attn_bias is not None:
+            attn = attn + attn_bias[i, :, :q_len, :kv_len].to(attn.dtype)
+        lses.append(torch.logsumexp(attn.float(), dim=-1))
+        probs = torch.softmax(attn, dim=-1).to(v.dtype)
+        probs = torch.nan_to_num(probs, nan=0.0)  # rows with no visible key
+        outputs.append(torch.einsum("hqk,khd->qhd", probs, v))
+        start += q_len
+    out = torch.cat(outputs, dim=0)
+    if return_lse:
+        return out, torch.cat(lses, dim=1)
+    return out
+
+
+def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping):
+    """tests/test_attention_ops.py:1459-1467: python loop scatter.  Returns updated clones."""
+    key, value = to_reference(key), to_reference(value)
+    kc, vc = to_reference(key_cache).clone(), to_reference(value_cache).clone()
+    block_size = kc.shape[1]
+    slots = to_reference(slot_mapping).tolist()
+    for i, s in enumerate(slots):
+        if s < 0:
+            continue
+        kc[s // block_size, s % block_size] = key[i]
+        vc[s // block_size, s % block_size] = value[i]
+    return kc, vc
+
+
+def gems_tolerance(dtype, reduce_dim=1, atol=1e-4):
+    """(atol, rtol) of src/flag_gems/testing/__init__.py:41-49."""
+    rtol = {torch.float16: 1e-3, torch.bfloat16: 0.016, torch.float32: 1.3e-6, torch.float64: 1e-7}[dtype]
+    return atol * reduce_dim, rtol

@@ -1,0 +1,139 @@
+"""GPU parity of mm / addmm (data-parallel and stream-K schedules) against the CPU oracle.
+Shapes, scalars and layouts follow tests/test_blas_ops.py:17-136 of the reference."""
+import numpy as np
+import pytest
+import torch
+
+import flag_gems
+from flaggems_amd import _C
+from flaggems_amd.ops import _gemm
+from oracle import torch_ref as O
+
+from helpers import FLOAT_DTYPES, MNK_SHAPES, SCALARS, gems_assert_close
+
+pytestmark = pytest.mark.gpu
+
+EXTRA_SHAPES = [(256, 256, 256), (300, 520, 264), (1024, 768, 512), (64, 4096, 136)]
+
+
+def _operand(rows, cols, dtype, dev, transposed):
+    if transposed:
+        return torch.randn(cols, rows, dtype=dtype, device=dev).t()
+    return torch.randn(rows, cols, dtype=dtype, device=dev)
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("M,N,K", MNK_SHAPES + EXTRA_SHAPES)
+@pytest.mark.parametrize("b_col_major", [False, True])
+@pytest.mark.parametrize("a_col_major", [False, True])
+def test_mm(gpu, M, N, K, dtype, a_col_major, b_col_major):
+    torch.manual_seed(0)
+    a = _operand(M, K, dtype, gpu, a_col_major)
+    b = _operand(K, N, dtype, gpu, b_col_major)
+    ref = O.mm(a, b)
+    with flag_gems.use_gems():
+        res = torch.mm(a, b)
+    gems_assert_close(res, ref, dtype, reduce_dim=K)
+    out = torch.empty(M, N, dtype=dtype, device=gpu)
+    with flag_gems.use_gems():
+        torch.mm(a, b, out=out)
+    gems_assert_close(out, ref, dtype, reduce_dim=K)
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("M,N,K", MNK_SHAPES + EXTRA_SHAPES[:2])
+@pytest.mark.parametrize("scalar", SCALARS)
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_addmm(gpu, M, N, K, scalar, dtype, b_col_major):
+    torch.manual_seed(0)
+    a = torch.randn(M, K, dtype=dtype, device=gpu)
+    b = _operand(K, N, dtype, gpu, b_col_major)
+    for bias in (torch.randn(N, dtype=dtype, device=gpu), torch.randn(M, N, dtype=dtype, device=gpu)):
+        ref = O.addmm(bias, a, b, alpha=scalar, beta=scalar)
+        with flag_gems.use_gems():
+            res = torch.addmm(bias, a, b, alpha=scalar, beta=scalar)
+        gems_assert_close(res, ref, dtype, reduce_dim=K)
+    out = torch.empty(M, N, dtype=dtype, device=gpu)
+    with flag_gems.use_gems():
+        torch.addmm(bias, a, b, alpha=scalar, beta=scalar, out=out)
+    gems_assert_close(out, ref, dtype, reduce_dim=K)
+
+
+def test_addmm_special_cases(gpu):
+    torch.manual_seed(1)
+    a = torch.randn(33, 40, device=gpu); b = torch.randn(40, 17, device=gpu); bias = torch.randn(17, device=gpu)
+    # alpha = 0: out = beta * bias exactly (fp32)
+    res = flag_gems.addmm(bias, a, b, alpha=0, beta=3)
+    assert torch.equal(res, (bias * 3).expand(33, 17))
+    # identity B
+    eye = torch.eye(40, device=gpu)
+    assert torch.equal(flag_gems.mm(a, eye), a)
+    # mixed dtypes promote to the higher one
+    res = flag_gems.mm(a.half(), b.bfloat16())
+    assert res.dtype == torch.bfloat16
+    # empty and K == 0
+    assert flag_gems.mm(a[:0], b).shape == (0, 17)
+    assert torch.equal(flag_gems.mm(a[:, :0], b[:0]), torch.zeros(33, 17, device=gpu))
+    # scalar (0-d) and column bias broadcast through zero strides
+    for bb in (torch.tensor(2.0, device=gpu), torch.randn(33, 1, device=gpu)):
+        gems_assert_close(flag_gems.addmm(bb, a, b), O.addmm(bb, a, b), torch.float32, reduce_dim=40)
+    # dtypes without a kernel go to the vendor library and still give the right answer
+    with flag_gems.use_gems():
+        r64 = torch.mm(a.double(), b.double())
+    assert r64.dtype == torch.float64 and torch.allclose(r64.cpu(), O.mm(a, b))
+
+
+SK_CASES = [
+    # (M, N, K, schedule)               skinny stream-K kernel (M <= 16) ...
+    (16, 4096, 14336, _C.SCHED_AUTO), (1, 4096, 4096, _C.SCHED_AUTO), (7, 1000, 2048, _C.SCHED_AUTO),
+    (16, 152, 1024, _C.SCHED_AUTO), (3, 11008, 4096, _C.SCHED_STREAM_K), (13, 128, 40960, _C.SCHED_AUTO),
+    # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
+    (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
+    (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,schedule", SK_CASES)
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_stream_k(gpu, M, N, K, schedule, dtype, b_col_major):
+    torch.manual_seed(2)
+    a = torch.randn(M, K, dtype=dtype, device=gpu) / K ** 0.5
+    b = _operand(K, N, dtype, gpu, b_col_major) / K ** 0.5
+    bias = torch.randn(N, dtype=dtype, device=gpu).broadcast_to(M, N)
+    ref = O.mm(a, b) * 0.5 + bias.double().cpu() * 2.0
+    c = torch.empty(M, N, dtype=dtype, device=gpu)
+    _gemm.gemm(a, b, bias, c, 0.5, 2.0, schedule=schedule)
+    assert _gemm.last_schedule() == _C.SCHED_STREAM_K
+    gems_assert_close(c, ref, dtype, reduce_dim=K)
+    # same answer as the data-parallel schedule up to fp32 re-association, and bit-identical run to run
+    d = torch.empty_like(c)
+    _gemm.gemm(a, b, bias, d, 0.5, 2.0, schedule=_C.SCHED_DATA_PARALLEL)
+    assert _gemm.last_schedule() == _C.SCHED_DATA_PARALLEL
+    gems_assert_close(d, ref, dtype, reduce_dim=K)
+    for _ in range(10):
+        e = torch.empty_like(c)
+        _gemm.gemm(a, b, bias, e, 0.5, 2.0, schedule=schedule)
+        assert torch.equal(c, e)
+
+
+def test_stream_k_needs_workspace(gpu):
+    a = torch.randn(8, 2048, dtype=torch.bfloat16, device=gpu); b = torch.randn(2048, 256, dtype=torch.bfloat16, device=gpu)
+    c = torch.empty(8, 256, dtype=torch.bfloat16, device=gpu)
+    rc = _C.lib().fg_gemm(a.data_ptr(), b.data_ptr(), None, c.data_ptr(), 8, 256, 2048, 2048, 1, 256, 1, 0, 0, 256, 1,
+                          1.0, 0.0, _C.FG_BF16, _C.FG_BF16, _C.FG_BF16, _C.SCHED_STREAM_K, None, 0, None, None)
+    assert rc == -4 and "workspace" in _C.last_error()
+
+
+def test_mm_full_size_properties(gpu):
+    """8192^3 bf16 (the benchmark shape): sampled rows against the oracle, plus linearity in A."""
+    torch.manual_seed(3)
+    n = 8192
+    a = torch.randn(n, n, dtype=torch.bfloat16, device=gpu) / n ** 0.5
+    b = torch.randn(n, n, dtype=torch.bfloat16, device=gpu) / n ** 0.5
+    for bb in (b, b.t()):
+        c = flag_gems.mm(a, bb)
+        rows = torch.tensor([0, 1, 255, 256, 4095, 4097, 8190, 8191], device=gpu)
+        gems_assert_close(c[rows], O.mm(a[rows], bb), torch.bfloat16, reduce_dim=n)
+        # doubling A doubles C exactly (power-of-two scaling commutes with every rounding)
+        assert torch.equal(flag_gems.mm(a * 2, bb), c * 2)

@@ -1,0 +1,212 @@
+"""CPU-side tests: the drop-in boundary (registration, signatures, error behaviour) and the C ABI
+loading with every symbol the header declares.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import flag_gems
+import flaggems_amd
+from flaggems_amd import _C
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_package_surface():
+    assert flag_gems.device == "cuda"
+    assert flag_gems.vendor_name == "amd"
+    assert flag_gems.__version__
+    for name in [
+        "enable", "use_gems", "all_ops", "mm", "mm_out", "addmm", "addmm_out", "softmax", "rms_norm",
+        "fused_add_rms_norm", "apply_rotary_pos_emb", "reshape_and_cache_flash", "silu_and_mul",
+        "silu_and_mul_out", "flash_attn_varlen_func",
+    ]:
+        assert callable(getattr(flag_gems, name)), name
+    assert flag_gems.ops.flash_attn_varlen_func is flaggems_amd.ops.flash_attn_varlen_func
+    assert flag_gems.testing.assert_close and flag_gems.testing.assert_equal
+    assert flag_gems.runtime.device.support_bf16 and flag_gems.runtime.device.support_fp64
+    assert flag_gems.runtime.torch_device_fn is torch.cuda
+    assert flag_gems.config.use_c_extension is False
+
+
+def _cuda_kernel_of(op):
+    table = torch._C._dispatch_dump_table(op)
+    for line in table.splitlines():
+        if line.startswith("CUDA:"):
+            return line
+    return ""
+
+
+def test_use_gems_registers_and_unregisters():
+    before = _cuda_kernel_of("aten::mm")
+    with flag_gems.use_gems():
+        assert sorted(flag_gems.all_ops()) == sorted(["_softmax", "addmm", "addmm.out", "mm", "mm.out", "rms_norm"])
+        inside = _cuda_kernel_of("aten::mm")
+        assert "flaggems_amd" in inside
+        assert "flaggems_amd" in _cuda_kernel_of("aten::rms_norm")
+        assert "flaggems_amd" in _cuda_kernel_of("aten::_softmax")
+    after = _cuda_kernel_of("aten::mm")
+    assert after == before and "flaggems_amd" not in after
+
+
+def test_unused_filters_by_function_name():
+    with flag_gems.use_gems(unused=["mm", "softmax"]):
+        ops = flag_gems.all_ops()
+        assert "mm" not in ops and "_softmax" not in ops
+        assert "mm.out" in ops and "addmm" in ops  # mm_out is a different python function
+        assert "flaggems_amd" not in _cuda_kernel_of("aten::mm")
+
+
+def test_enable_record_writes_log(tmp_path):
+    import logging
+
+    lib = torch.library.Library("aten", "IMPL")
+    path = tmp_path / "oplist.log"
+    try:
+        flag_gems.enable(lib=lib, record=True, once=True, path=str(path))
+        logging.getLogger("flag_gems.ops.mm").debug("GEMS MM probe")
+        for h in logging.getLogger("flag_gems").handlers:
+            h.flush()
+        assert "GEMS MM probe" in path.read_text()
+    finally:
+        lib._destroy()
+        lg = logging.getLogger("flag_gems")
+        for h in lg.handlers[:]:
+            lg.removeHandler(h)
+            h.close()
+
+
+def test_registration_error_is_wrapped():
+    class Boom:
+        def impl(self, *a):
+            raise ValueError("no")
+
+    with pytest.raises(RuntimeError) as ei:
+        flaggems_amd.runtime.Register((("mm", flag_gems.mm),), lib=Boom())
+    assert "An error was encountered while registering the triton operator." in str(ei.value.args)
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fg_mi355.h")).read()
+    declared = set(re.findall(r"\b(fg_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    handle = ctypes.CDLL(_C.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in include/fg_mi355.h but not exported"
+    assert declared == set(_C.exported_symbols()), "python binding and header disagree"
+    assert _C.lib().fg_abi_version() == 1
+
+
+def test_struct_mirror_matches_header_order():
+    header = open(os.path.join(ROOT, "include", "fg_mi355.h")).read()
+    body = header[header.index("typedef struct FgFlashParams {"):header.index("} FgFlashParams;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    body = body[body.index("{") + 1:]
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        parts = decl.replace("*", " ").split(",")
+        first = parts[0].split()
+        names.append(first[-1])
+        names.extend(p.strip() for p in parts[1:])
+    assert names == [f[0] for f in _C.FgFlashParams._fields_]
+
+
+def test_abi_validation_errors_without_gpu():
+    lib = _C.lib()
+    # invalid arguments are rejected on the host before any launch
+    assert lib.fg_softmax(None, None, -1, 4, 1, _C.FG_F32, _C.FG_F32, None) == -1
+    assert "negative" in _C.last_error()
+    assert lib.fg_softmax(None, None, 4, 4, 1, _C.FG_F32, _C.FG_F32, None) == -1  # null pointers
+    assert lib.fg_rms_norm(None, None, None, None, 4, 4, 4, 4, 1e-5, _C.FG_F32, None) == -1
+    assert lib.fg_rms_norm(None, None, None, None, 0, 4, 4, 4, 1e-5, _C.FG_F32, None) == 0  # empty: nothing to do
+    assert lib.fg_silu_and_mul(None, None, None, 2, 2, 2, 2, 2, 7, None) == -1
+    assert lib.fg_reshape_and_cache_flash(None, None, None, None, None, 1, 4, 2, 8, 0, 16, 16, 256, 2, None) == -1
+    assert "block_size" in _C.last_error()
+    one = ctypes.c_void_p(256)
+    rc = lib.fg_gemm(one, one, None, one, 4, 4, 4, 4, 1, 4, 1, 0, 0, 4, 1, 1.0, 0.0, _C.FG_F16, _C.FG_F32, _C.FG_F16,
+                     0, None, 0, None, None)
+    assert rc == -2 and "output dtype" in _C.last_error()
+    rc = lib.fg_gemm(one, one, None, one, 4, 4, 0, 4, 1, 4, 1, 0, 0, 4, 1, 1.0, 0.0, _C.FG_F16, _C.FG_F16, _C.FG_F16,
+                     0, None, 0, None, None)
+    assert rc == -1 and "K must be positive" in _C.last_error()
+    p = _C.FgFlashParams()
+    p.dtype = _C.FG_F32
+    assert lib.fg_flash_attn_varlen_fwd(ctypes.byref(p), None) == -1
+    assert "fp16 and bf16" in _C.last_error()
+    with pytest.raises(RuntimeError):
+        _C.check(-1, "probe")
+
+
+def test_python_wrappers_assert_like_the_reference():
+    a = torch.randn(4, 5)
+    b = torch.randn(6, 7)
+    with pytest.raises(AssertionError, match="incompatible dimensions"):
+        from flaggems_amd.ops.mm import _prepare
+
+        _prepare(a, b)
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        flag_gems.addmm(torch.randn(7), a, b)
+    with pytest.raises(AssertionError, match="Incompatible input shape"):
+        flag_gems.addmm(torch.randn(3), a, torch.randn(5, 7))
+    with pytest.raises(AssertionError, match="Invalid dim"):
+        flag_gems.softmax(torch.randn(3, 3), 2)
+    q = torch.randn(2, 3, 4, 8)
+    with pytest.raises(AssertionError, match="same last dimension"):
+        flag_gems.apply_rotary_pos_emb(q, torch.randn(2, 3, 4, 16), torch.randn(8, 4), torch.randn(8, 4))
+    with pytest.raises(AssertionError, match="half of q/k dim"):
+        flag_gems.apply_rotary_pos_emb(q, q, torch.randn(8, 8), torch.randn(8, 8))
+    with pytest.raises(AssertionError, match="4 dimensions"):
+        flag_gems.apply_rotary_pos_emb(q[0], q[0], torch.randn(8, 4), torch.randn(8, 4))
+    cu = torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(AssertionError, match="cu_seqlens_k or seqused_k must be provided"):
+        flag_gems.flash_attn_varlen_func(q[0], q, q, 3, cu, 3)
+    with pytest.raises(AssertionError, match="cannot be provided at the same time"):
+        flag_gems.flash_attn_varlen_func(q[0], q, q, 3, cu, 3, cu_seqlens_k=cu, seqused_k=cu[:1])
+    with pytest.raises(RuntimeError, match="Only FA2"):
+        flag_gems.flash_attn_varlen_func(q[0], q, q, 3, cu, 3, seqused_k=cu[:1], fa_version=3)
+    with pytest.raises(RuntimeError, match="num_splits"):
+        flag_gems.flash_attn_varlen_func(q[0], q, q, 3, cu, 3, seqused_k=cu[:1], num_splits=2)
+
+
+def test_broadcastable_and_dtype_order():
+    from flaggems_amd.ops._gemm import get_higher_dtype
+    from flaggems_amd.ops.addmm import broadcastable_to
+
+    assert broadcastable_to((), (3, 4)) and broadcastable_to((4,), (3, 4)) and broadcastable_to((1, 4), (3, 4))
+    assert broadcastable_to((3, 1), (3, 4)) and not broadcastable_to((3,), (3, 4)) and not broadcastable_to((2, 3, 4), (3, 4))
+    assert not broadcastable_to((4,), ())
+    f16, bf16, f32 = torch.float16, torch.bfloat16, torch.float32
+    assert get_higher_dtype(f16, bf16) is bf16 and get_higher_dtype(bf16, f32) is f32 and get_higher_dtype(f16, f16) is f16
+
+
+def test_assert_close_rule():
+    from flag_gems.testing import assert_close
+
+    ref = torch.tensor([1.0, 100.0], dtype=torch.float64)
+    assert_close(torch.tensor([1.0, 101.5], dtype=torch.bfloat16), ref, torch.bfloat16)  # rtol 1.6e-2
+    with pytest.raises(AssertionError):
+        assert_close(torch.tensor([1.0, 103.0], dtype=torch.bfloat16), ref, torch.bfloat16)
+    assert_close(torch.tensor([1.05, 100.0], dtype=torch.float32), ref, torch.float32, reduce_dim=1000)  # atol 0.1
+    with pytest.raises(AssertionError):
+        assert_close(torch.tensor([1.0], dtype=torch.float32), ref[:1], torch.float16)  # dtype must match
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_C, "_lib", None)
+    monkeypatch.setattr(_C, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_C.ExtensionMissing):
+        _C.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "flaggems_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text.replace("the oracle", ""), f"{f} mentions the oracle package"

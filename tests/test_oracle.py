@@ -1,0 +1,316 @@
+"""Pins the CPU oracle: closed forms, invariants, brute force on tiny inputs, the committed golden
+fixtures, and agreement of the plain-C restatements with independent Python loops.  A plausible
+mistake in the oracle (dropped term, wrong sign or index, transposed operand) fails one of these.
+Runs on the CPU."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref
+from oracle import torch_ref as O
+
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_v1.npz"))
+
+
+def t(name, dtype=None):
+    x = torch.from_numpy(GOLD[name])
+    return x.to(dtype) if dtype is not None else x
+
+
+# ---------------------------------------------------------------------------------------------
+# golden fixtures: the oracle of today reproduces the committed numbers
+# ---------------------------------------------------------------------------------------------
+def test_oracle_reproduces_golden():
+    bf16, f16 = torch.bfloat16, torch.float16
+    for tag, dt in (("bf16", bf16), ("f16", f16)):
+        x, r, w = t(f"rms_{tag}_x", dt), t(f"rms_{tag}_r", dt), t(f"rms_{tag}_w", dt)
+        torch.testing.assert_close(O.rms_norm(x, w, 1e-5).double(), t(f"rms_{tag}_y"), atol=0, rtol=0)
+        y, s = O.fused_add_rms_norm(x, r, w, 1e-5)
+        torch.testing.assert_close(y, t(f"fused_{tag}_y"), atol=1e-12, rtol=1e-12)
+        torch.testing.assert_close(s, t(f"fused_{tag}_res"), atol=0, rtol=0)
+    torch.testing.assert_close(O.softmax(t("softmax_bf16_x", bf16), -1), t("softmax_bf16_y"), atol=1e-12, rtol=1e-12,
+                               equal_nan=True)
+    a, b, bias = t("mm_f16_a", f16), t("mm_f16_b", f16), t("mm_f16_bias", f16)
+    torch.testing.assert_close(O.mm(a, b), t("mm_f16_c"), atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(O.addmm(bias, a, b, alpha=-0.999, beta=100.001), t("addmm_f16_c"), atol=1e-10, rtol=1e-12)
+    q, k = t("rope_q", bf16), t("rope_k", bf16)
+    for inter in (False, True):
+        oq, ok = O.apply_rotary_pos_emb(q, k, t("rope_cos"), t("rope_sin"), t("rope_pos"), inter)
+        torch.testing.assert_close(oq, t(f"rope_oq_{int(inter)}"), atol=1e-12, rtol=1e-12)
+        torch.testing.assert_close(ok, t(f"rope_ok_{int(inter)}"), atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(O.silu_and_mul(t("silu_a", f16), t("silu_b", f16)), t("silu_y"), atol=1e-12, rtol=1e-12)
+    out, lse = O.paged_attention(t("attn_q", bf16), t("attn_kc", bf16), t("attn_vc", bf16), GOLD["attn_qlens"].tolist(),
+                                 GOLD["attn_klens"].tolist(), t("attn_bt"), 0.25, causal=True,
+                                 compute_dtype=torch.float64, return_lse=True)
+    torch.testing.assert_close(out, t("attn_out"), atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(lse.double(), t("attn_lse"), atol=1e-5, rtol=1e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# norms
+# ---------------------------------------------------------------------------------------------
+def test_rms_norm_closed_form_and_loops():
+    # constant row, unit weight: y = c / sqrt(c^2 + eps)
+    for c in (0.5, -3.0):
+        x = torch.full((2, 16), c)
+        y = O.rms_norm(x, torch.ones(16), 1e-3)
+        assert torch.allclose(y, torch.full((2, 16), c / math.sqrt(c * c + 1e-3)), atol=1e-6)
+    # independent numpy loop
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((3, 7)).astype(np.float32)
+    w = rng.standard_normal(7).astype(np.float32)
+    ref = np.stack([row / np.sqrt((row.astype(np.float64) ** 2).sum() / 7 + 1e-5) * w for row in x])
+    assert np.allclose(O.rms_norm(torch.from_numpy(x), torch.from_numpy(w), 1e-5).numpy(), ref, atol=1e-5)
+    # weight scales the output linearly; scaling x by a large factor leaves y (almost) unchanged
+    y1 = O.rms_norm(torch.from_numpy(x), torch.from_numpy(w), 0.0)
+    y2 = O.rms_norm(torch.from_numpy(x * 8), torch.from_numpy(w), 0.0)
+    assert torch.allclose(y1, y2, atol=1e-5)
+
+
+def test_fused_add_rms_norm_both_outputs():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((4, 9)); r = rng.standard_normal((4, 9)); w = rng.standard_normal(9)
+    y, s = O.fused_add_rms_norm(torch.from_numpy(x), torch.from_numpy(r), torch.from_numpy(w), 1e-6)
+    assert np.allclose(s.numpy(), x + r)
+    for i in range(4):
+        row = x[i] + r[i]
+        assert np.allclose(y[i].numpy(), row / math.sqrt((row ** 2).mean() + 1e-6) * w)
+    # residual = 0 reduces to rms_norm of x
+    y0, _ = O.fused_add_rms_norm(torch.from_numpy(x), torch.zeros(4, 9, dtype=torch.float64), torch.from_numpy(w), 1e-6)
+    assert torch.allclose(y0.float(), O.rms_norm(torch.from_numpy(x).float(), torch.from_numpy(w).float(), 1e-6), atol=1e-5)
+    # the scalar C port agrees
+    xf, rf, wf = x.astype(np.float32).copy(), r.astype(np.float32).copy(), w.astype(np.float32)
+    cref.fused_add_rms_norm_f32(xf, rf, wf, 1e-6)
+    assert np.allclose(rf, (x + r).astype(np.float32), atol=1e-6) and np.allclose(xf, y.numpy(), atol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------------------------
+def test_softmax_invariants():
+    x = torch.randn(6, 11, generator=torch.Generator().manual_seed(2))
+    x[0, 3] = float("-inf"); x[2] = float("-inf")
+    y = O.softmax(x, -1)
+    assert torch.allclose(y[[0, 1, 3, 4, 5]].sum(-1), torch.ones(5, dtype=torch.float64))
+    assert y[0, 3] == 0 and torch.isnan(y[2]).all()
+    assert torch.allclose(O.softmax(x[1:2] + 5.0, -1), y[1:2])  # shift invariance
+    # brute force
+    row = x[4].double()
+    e = torch.tensor([math.exp(v - float(row.max())) for v in row.tolist()], dtype=torch.float64)
+    assert torch.allclose(y[4], e / e.sum())
+    # a middle axis
+    z = torch.randn(3, 5, 4)
+    assert torch.allclose(O.softmax(z, 1).sum(1), torch.ones(3, 4, dtype=torch.float64))
+
+
+# ---------------------------------------------------------------------------------------------
+# mm / addmm (library routines: only the argument roles can go wrong)
+# ---------------------------------------------------------------------------------------------
+def test_mm_addmm_roles():
+    a = torch.tensor([[1.0, 2.0], [3.0, 4.0], [5.0, 6.0]]); b = torch.tensor([[1.0, 0.0, 2.0, 0.0], [0.0, 1.0, 0.0, 3.0]])
+    assert torch.equal(O.mm(a, b), torch.tensor([[1, 2, 2, 6], [3, 4, 6, 12], [5, 6, 10, 18]], dtype=torch.float64))
+    bias = torch.tensor([10.0, 20.0, 30.0, 40.0])
+    assert torch.equal(O.addmm(bias, a, b, alpha=2, beta=0.5), 2 * O.mm(a, b) + 0.5 * bias.double())
+    assert torch.equal(O.addmm(bias, a, b, alpha=0, beta=1), bias.double().expand(3, 4))
+
+
+# ---------------------------------------------------------------------------------------------
+# rope
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("inter", [False, True])
+def test_rope_brute_force_and_invariants(inter):
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(2, 4, 3, 8, generator=g); k = torch.randn(2, 4, 1, 8, generator=g)
+    cos, sin = O.rope_cos_sin(16, 8)
+    assert torch.allclose(cos[:, 0], torch.cos(torch.arange(16.0))) and torch.allclose(sin[3, 1], torch.sin(torch.tensor(3.0 / 10000 ** 0.25)))
+    pos = torch.randint(0, 16, (2, 4), generator=g)
+    oq, ok = O.apply_rotary_pos_emb(q, k, cos, sin, pos, inter)
+    for b in range(2):
+        for s in range(4):
+            p = int(pos[b, s])
+            for (x, o) in ((q, oq), (k, ok)):
+                for h in range(x.shape[2]):
+                    for j in range(4):
+                        i0, i1 = (2 * j, 2 * j + 1) if inter else (j, j + 4)
+                        c, sn = float(cos[p, j]), float(sin[p, j])
+                        x0, x1 = float(x[b, s, h, i0]), float(x[b, s, h, i1])
+                        assert abs(float(o[b, s, h, i0]) - (x0 * c - x1 * sn)) < 1e-6
+                        assert abs(float(o[b, s, h, i1]) - (x1 * c + x0 * sn)) < 1e-6
+    # position 0 is the identity; rotations preserve the norm of every pair, hence of the head
+    o0, _ = O.apply_rotary_pos_emb(q, k, cos, sin, torch.zeros(2, 4, dtype=torch.long), inter)
+    assert torch.allclose(o0, q.double())
+    assert torch.allclose(oq.norm(dim=-1), q.double().norm(dim=-1))
+    # without position ids the position is the index along dim -3
+    o1, _ = O.apply_rotary_pos_emb(q, k, cos, sin, None, inter)
+    o2, _ = O.apply_rotary_pos_emb(q, k, cos, sin, torch.arange(4).expand(2, 4), inter)
+    assert torch.allclose(o1, o2)
+
+
+def test_silu_and_mul_closed_form():
+    a = torch.tensor([0.0, 1.0, -2.0, 30.0]); b = torch.tensor([3.0, 2.0, 0.5, 1.0])
+    ref = torch.tensor([0.0, 2.0 / (1 + math.exp(-1.0)), -1.0 / (1 + math.exp(2.0)), 30.0 / (1 + math.exp(-30.0))], dtype=torch.float64)
+    assert torch.allclose(O.silu_and_mul(a, b), ref)
+
+
+# ---------------------------------------------------------------------------------------------
+# paged attention
+# ---------------------------------------------------------------------------------------------
+def brute_attention(q, kc, vc, qlens, klens, bt, scale, causal, window=None, softcap=None, slopes=None):
+    """Scalar loops: the definition itself."""
+    H, Hk = q.shape[1], kc.shape[2]
+    bs = kc.shape[1]
+    outs, lses = [], []
+    start = 0
+    for i, (ql, kl) in enumerate(zip(qlens, klens)):
+        o = torch.zeros(ql, H, q.shape[2], dtype=torch.float64)
+        l = torch.zeros(H, ql, dtype=torch.float64)
+        for r in range(ql):
+            for h in range(H):
+                kh = h // (H // Hk)
+                logits = []
+                for c in range(kl):
+                    page = int(bt[i, c // bs])
+                    kv = kc[page, c % bs, kh].double()
+                    s = float((q[start + r, h].double() * kv).sum()) * scale
+                    if softcap:
+                        s = softcap * math.tanh(s / softcap)
+                    rel = r + kl - ql
+                    masked = (causal and c > rel)
+                    if window is not None:
+                        left, right = window
+                        if left >= 0 and c < rel - left:
+                            masked = True
+                        if right >= 0 and not causal and c > rel + right:
+                            masked = True
+                    if slopes is not None:
+                        s += float(slopes[i, h]) * ((c - kl + 1) if causal else -abs(rel - c))
+                    logits.append(-math.inf if masked else s)
+                m = max(logits) if logits else -math.inf
+                if m == -math.inf:
+                    l[h, r] = math.inf  # marks "no visible key"
+                    continue
+                w = [math.exp(v - m) for v in logits]
+                z = sum(w)
+                l[h, r] = m + math.log(z)
+                for c in range(kl):
+                    page = int(bt[i, c // bs])
+                    o[r, h] += (w[c] / z) * vc[page, c % bs, kh].double()
+        outs.append(o); lses.append(l)
+        start += ql
+    return torch.cat(outs), torch.cat(lses, dim=1)
+
+
+def _tiny_attn(seed=4):
+    g = torch.Generator().manual_seed(seed)
+    qlens, klens = [1, 3, 6, 2], [7, 3, 4, 9]   # includes q_len > k_len (rows without any visible key)
+    q = torch.randn(sum(qlens), 4, 8, generator=g)
+    kc, vc = torch.randn(6, 4, 2, 8, generator=g), torch.randn(6, 4, 2, 8, generator=g)
+    bt = torch.randint(0, 6, (4, 3), generator=g, dtype=torch.int32)
+    return q, kc, vc, qlens, klens, bt
+
+
+@pytest.mark.parametrize("causal,window,softcap,alibi", [
+    (True, None, None, False), (False, None, None, False), (True, (2, 0), None, False),
+    (False, (1, 2), None, False), (True, None, 5.0, False), (True, None, None, True), (False, None, None, True),
+])
+def test_paged_attention_vs_brute_force(causal, window, softcap, alibi):
+    q, kc, vc, qlens, klens, bt = _tiny_attn()
+    slopes = torch.tensor([[0.5, 0.25, 0.125, 0.0625]] * 4) if alibi else None
+    bias = None
+    if alibi:
+        bias = torch.zeros(4, 4, max(qlens), max(klens))
+        for i, (ql, kl) in enumerate(zip(qlens, klens)):
+            bias[i, :, :ql, :kl] = O.alibi_bias(slopes[i:i + 1], ql, kl, causal)[0]
+    ref, rlse = brute_attention(q, kc, vc, qlens, klens, bt, 0.3, causal, window, softcap, slopes)
+    out, lse = O.paged_attention(q, kc, vc, qlens, klens, bt, 0.3, causal=causal, window=window, soft_cap=softcap,
+                                 attn_bias=bias, compute_dtype=torch.float64, return_lse=True)
+    assert torch.allclose(out, ref, atol=1e-9)
+    fin = torch.isfinite(rlse)
+    assert torch.allclose(lse.double()[fin], rlse[fin], atol=1e-5)
+    assert (lse[~fin] == -math.inf).all()  # logsumexp of an empty row; the kernel reports +inf there
+
+
+def test_paged_attention_special_cases():
+    q, kc, vc, qlens, klens, bt = _tiny_attn(5)
+    # one key: the output is that key's value row, whatever the scores
+    out = O.paged_attention(q[:1], kc, vc, [1], [1], bt[:1], 1.0, causal=True, compute_dtype=torch.float64)
+    for h in range(4):
+        assert torch.allclose(out[0, h], vc[int(bt[0, 0]), 0, h // 2].double())
+    # zero queries: uniform weights, the output is the mean of the visible values
+    out = O.paged_attention(torch.zeros(1, 4, 8), kc, vc, [1], [7], bt[:1], 1.0, causal=True, compute_dtype=torch.float64)
+    vals = torch.stack([vc[int(bt[0, c // 4]), c % 4] for c in range(7)]).double()
+    assert torch.allclose(out[0, 0], vals[:, 0].mean(0)) and torch.allclose(out[0, 3], vals[:, 1].mean(0))
+    # the sliding_window argument of the reference equals window=(w - 1, 0) under causal
+    o1 = O.paged_attention(q, kc, vc, qlens, klens, bt, 0.3, causal=True, sliding_window=3, compute_dtype=torch.float64)
+    o2 = O.paged_attention(q, kc, vc, qlens, klens, bt, 0.3, causal=True, window=(2, 0), compute_dtype=torch.float64)
+    assert torch.allclose(o1, o2)
+
+
+# ---------------------------------------------------------------------------------------------
+# byte / integer work: the C restatements
+# ---------------------------------------------------------------------------------------------
+def test_cache_scatter_c_vs_python_loop():
+    rng = np.random.default_rng(6)
+    for dtype, D, bs in ((np.float32, 5, 4), (np.uint16, 8, 2), (np.uint8, 3, 7)):
+        nt, H, nb = 9, 2, 6
+        packed = rng.integers(0, 250, size=(nt, 3, H, D)).astype(dtype)       # key/value are strided views
+        key, val = packed[:, 1], packed[:, 2]
+        kc = rng.integers(0, 250, size=(nb, bs, H, D)).astype(dtype); vc = kc[::-1].copy()
+        slots = rng.permutation(nb * bs)[:nt].astype(np.int64); slots[4] = -1
+        ek, ev = kc.copy(), vc.copy()
+        for i, s in enumerate(slots):
+            if s >= 0:
+                ek[s // bs, s % bs] = key[i]; ev[s // bs, s % bs] = val[i]
+        stride = 3 * H * D
+        cref.reshape_and_cache_flash(packed.reshape(-1)[H * D:], packed.reshape(-1)[2 * H * D:], kc, vc, slots, stride, stride, bs * H * D)
+        assert np.array_equal(kc, ek) and np.array_equal(vc, ev)
+        # the torch loop of the reference's test agrees
+        tk, tv = O.reshape_and_cache_flash(torch.from_numpy(key.astype(np.float32)), torch.from_numpy(val.astype(np.float32)),
+                                           torch.from_numpy(ek.astype(np.float32)), torch.from_numpy(ev.astype(np.float32)),
+                                           torch.from_numpy(slots))
+        assert np.array_equal(tk.numpy(), ek.astype(np.float32))
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_v1.npz"))
+    kc, vc = g["cache_kc0"].copy(), g["cache_vc0"].copy()
+    cref.reshape_and_cache_flash(g["cache_key"].reshape(-1), g["cache_val"].reshape(-1), kc, vc, g["cache_slots"], 16, 16, 64)
+    assert np.array_equal(kc, g["cache_kc1"]) and np.array_equal(vc, g["cache_vc1"])
+    assert np.array_equal(kc[1, 3], g["cache_key"][0]) and np.array_equal(kc[0, 0], g["cache_key"][1])  # slots 7 and 0
+
+
+def test_virtual_to_cache():
+    table = np.array([5, 0, 9, 2], dtype=np.int32)
+    for virt in range(16 * 4):
+        assert cref.virtual_to_cache(virt, table, 16, 1024) == (int(table[virt // 16]) * 16 + virt % 16) * 1024
+
+
+def test_streamk_partition_rule_and_abi_agreement():
+    import ctypes
+    from flaggems_amd import _C
+
+    # closed form: 32 tiles of 112 iterations over 256 programs -> 32 cooperative tiles, 14 iterations each
+    coop, b, e = cref.streamk_partition(32, 112, 256)
+    assert coop == 32 and (e - b == 14).all() and b[0] == 0 and e[-1] == 32 * 112
+    for tiles, iters, workers in [(1, 1, 4), (5, 3, 4), (7, 10, 3), (300, 8, 256), (470, 4, 256), (256, 5, 256), (3, 7, 8), (100, 1, 7)]:
+        coop, b, e = cref.streamk_partition(tiles, iters, workers)
+        rem = tiles % workers
+        expect = rem
+        if tiles - rem > 0 and rem < workers * 0.5:
+            expect = rem + workers
+        elif tiles - rem > 0 and rem > workers * 0.8:
+            expect = 0
+        assert coop == expect
+        # every (tile, iteration) unit of the cooperative tiles is covered exactly once, in order
+        cover = np.zeros(coop * iters, dtype=np.int64)
+        for w in range(workers):
+            cover[b[w]:e[w]] += 1
+            assert 0 <= e[w] - b[w] - (coop * iters) // workers <= 1
+            if w:
+                assert b[w] == e[w - 1]
+        assert (cover == 1).all()
+        # the product's host function gives the same split
+        sk = ctypes.c_int64()
+        pb = (ctypes.c_int64 * workers)(); pe = (ctypes.c_int64 * workers)()
+        assert _C.lib().fg_streamk_partition(tiles, iters, workers, ctypes.byref(sk), pb, pe) == 0
+        assert sk.value == coop and list(pb) == b.tolist() and list(pe) == e.tolist()
