@@ -139,7 +139,9 @@ def main():
         def cpu():
             O.softmax(sample, -1)
 
-        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16",
+        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
+        # read for a plain 512 MiB copy (profiles/softmax_c2_hbm_traffic.txt)
+        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=1073820700,
                     workload="softmax dim=-1 [131072,2048] bf16, N(0,4) with 1% -inf (BASELINE.json configs[1])",
                     cpu=(cpu, 2 * 32768 * N * 2, "oracle softmax (torch CPU, fp64 upcast) on the first 32768 rows"))
 
@@ -300,6 +302,18 @@ def main():
                     workload="Llama-2-7B decoder layer forward under flag_gems.enable(), 8 x 2048-token prefill, paged KV (configs[4])",
                     cpu=None, post=post)
 
+    def wl_copy_ref():
+        # plain device copy of known size (torch's elementwise copy kernel): the yardstick the
+        # FETCH_SIZE / WRITE_SIZE counters are scaled by; not part of the operator path
+        x = torch.randn(131072, 2048, device=dev).to(bf16)
+        y = torch.empty_like(x)
+
+        def run(i):
+            y.copy_(x)
+
+        return dict(run=run, work=2 * x.numel() * 2, bound="hbm", dtype="bf16",
+                    workload="reference: torch copy of a [131072,2048] bf16 tensor (512 MiB read + 512 MiB written)", cpu=None)
+
     workloads = {
         "softmax_c2": wl_softmax_c2,
         "fused_add_rms_norm_c1": wl_fused_add_rms_norm_c1,
@@ -309,6 +323,7 @@ def main():
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "decoder_layer_c5": wl_layer_c5,
+        "copy_ref": wl_copy_ref,
     }
     if args.workload not in workloads:
         print("bench.py: unknown workload %s (have: %s)" % (args.workload, ", ".join(workloads)), file=sys.stderr)
@@ -318,7 +333,7 @@ def main():
         w = workloads[name]()
         wall_ms, ev_ms = timed(w["run"], steps, warmup)
         res = {"workload": w["workload"], "ms_per_step": round(wall_ms, 5), "kernel_ms": round(ev_ms, 5),
-               "roofline": roofline(w["bound"], w["work"], ev_ms)}
+               "roofline": roofline(w["bound"], w["work"], ev_ms, w.get("traffic"))}
         if w["bound"] == "hbm":
             res["value"], res["unit"] = round(w["work"] / wall_ms / 1e6, 1), "GB/s"
         else:
@@ -340,7 +355,7 @@ def main():
     extra = {}
     if not args.no_extra:
         for name in workloads:
-            if name == args.workload:
+            if name == args.workload or name == "copy_ref":
                 continue
             steps = max(3, min(args.steps, 20))
             if name == "decoder_layer_c5":
