@@ -243,18 +243,30 @@ template <typename T, int BM, int BN, int AMODE, int BMODE> struct TileCompute {
       }
       const char* a_base = As + cur * A_STAGE + (wm * WTM + frag_row) * kPitch + frag_k;
       const char* b_base = Bs + cur * B_STAGE + (wn * WTN + frag_row) * kPitch + frag_k;
+      // Fragments are double-buffered in registers and the scheduler is asked (iglp_opt) to
+      // interleave the LDS reads of step ks+1 with the MFMAs of step ks; left alone it would sink
+      // every read next to its first use and expose the LDS latency four times per K step.
+      constexpr int KSTEPS = BK / Mfma<T>::KSTEP;
+      if constexpr (sizeof(T) == 2) __builtin_amdgcn_iglp_opt(1);
+      Frag fa[2][TM], fb[2][TN];
 #pragma unroll
-      for (int ks = 0; ks < BK / Mfma<T>::KSTEP; ++ks) {
-        Frag fa[TM], fb[TN];
-        const int koff = ks * Mfma<T>::KSTEP * (int)sizeof(T);
+      for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * kPitch);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * kPitch + koff);
+      for (int j = 0; j < TN; ++j) fb[0][j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * kPitch);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * kPitch + koff);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int cb = ks & 1, nb = cb ^ 1;
+        if (ks + 1 < KSTEPS) {
+          const int koff = (ks + 1) * Mfma<T>::KSTEP * (int)sizeof(T);
+#pragma unroll
+          for (int i = 0; i < TM; ++i) fa[nb][i] = *reinterpret_cast<const Frag*>(a_base + i * 32 * kPitch + koff);
+#pragma unroll
+          for (int j = 0; j < TN; ++j) fb[nb][j] = *reinterpret_cast<const Frag*>(b_base + j * 32 * kPitch + koff);
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::mma(fa[i], fb[j], acc[i][j]);
+          for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::mma(fa[cb][i], fb[cb][j], acc[i][j]);
       }
       if (more) {
         sa.store(As + (cur ^ 1) * A_STAGE, tid);
