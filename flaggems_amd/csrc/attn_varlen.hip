@@ -26,6 +26,7 @@
 // K/V tiles of 64 keys are gathered page by page (block_table -> page -> row), 16 bytes per lane,
 // zero-filled past the sequence end so stale cache contents can never reach the accumulators.
 // V is transposed on its way into LDS (8x8 register transposes with v_perm_b32).
+#include <stdlib.h>
 #include "fg_common.h"
 
 namespace {
@@ -56,6 +57,8 @@ struct AttnArgs {
   int right_off_w, left_off_w;  // window_right / window_left as used by the bounds
   float scale_log2;   // softmax_scale * log2(e)   (softcap == 0)
   float cap_in, cap_out_log2;  // softcap: t = cap_out_log2 * tanh(S * cap_in)
+  int page_shift;     // log2(page_size) when it is a power of two, else -1
+  int use_async;      // take the asynchronous-tile kernel (head dims 64, 96, 128, 192, 256)
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -285,9 +288,324 @@ __global__ __launch_bounds__(256) void attn_varlen_kernel(AttnArgs a) {
     }
 }
 
+// =============================================================================================
+// Fast path: asynchronous K/V tiles.
+//
+// Same work split and the same two transposed products as the kernel above; what changes is how
+// the tiles travel and how the waves overlap:
+//   * K and V tiles (64 keys x D) go from the paged cache straight into LDS with
+//     global_load_lds_dwordx4 (no staging registers, no LDS store instructions), two stages deep:
+//     the tile for step j+1 is in flight while step j computes; one s_waitcnt vmcnt + one barrier
+//     per step.  Keys past the sequence end are clamped to the last valid key: their scores are
+//     masked to -inf, so their probability is an exact zero and the duplicate rows never count.
+//   * LDS rows are RB = 2*D bytes rounded up to a power of two, with the 16-byte chunks of row
+//     `key` stored at position chunk ^ swz(key).  swz is a bit permutation of key & 15 chosen so
+//     that (a) the 16 keys a quarter-wave reads for one K fragment and (b) the 4 keys x 32 bytes a
+//     16-lane group reads for one transposed V fragment both fall into disjoint banks.
+//   * V stays in its natural [key][d] layout; the V^T MFMA operand (8 consecutive keys of one d
+//     per lane) is produced by ds_read_b64_tr_b16, which hands lane i of a 16-lane group the i-th
+//     16-bit column of the 4 rows x 64 bits the group addresses.
+//   * exp2 is the bare v_exp_f32; the softmax scale is folded into one fma per score; the output
+//     accumulator is rescaled only when a row maximum actually moved.
+//   * at most 256 VGPRs, so two workgroups share a CU and one workgroup's softmax (VALU) overlaps
+//     the other's MFMAs.
+// =============================================================================================
+#define FG_LDSP(p) ((__attribute__((address_space(3))) void*)(p))
+#define FG_GLBP(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FG_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (7 << 4) | (0xF << 8) | (((N) >> 4) << 14))
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int CPR>
+__device__ __forceinline__ int swz(int key) {
+  if constexpr (CPR >= 16) return (key & 8) | (((key >> 1) & 1) << 2) | ((key & 1) << 1) | ((key >> 2) & 1);
+  else return (((key >> 1) & 1) << 2) | (((key >> 2) & 1) << 1) | ((key >> 3) & 1);
+}
+
+// Two workgroups per CU when the tiles allow it (RB <= 256: 64 KB of LDS each); the wide-head
+// variants need 128 KB, run alone on a CU and may use the whole register file.
+template <typename T, int D, int RB>
+__global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_kernel(AttnArgs a) {
+  typedef typename AttnMfma<T>::Frag Frag;
+  constexpr int CPR = RB / 16;          // 16-byte chunks per LDS row
+  constexpr int VALID_C = D / 8;        // chunks that hold data
+  constexpr int KS = D / 16;            // MFMA k-steps over the head dim
+  constexpr int DT = (D + 31) / 32;     // 32-row output sub-tiles over the head dim
+  constexpr int OPB = kBN * RB;         // bytes of one operand tile
+  constexpr int STAGEB = 2 * OPB;       // K tile + V tile
+  constexpr int IPW = RB / 64;          // DMA instructions per wave per operand per tile
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const FgFlashParams& p = a.p;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, ql = lane & 31;
+  // long (late) row blocks first: they take the most steps under a causal mask
+  const int m_block = gridDim.x - 1 - blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+
+  const int q_bos = p.cu_seqlens_q[b];
+  const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
+  const int k_len = p.seqused_k[b];
+  const int block_row0 = m_block * a.rows_per_block;
+  if (block_row0 >= q_len) return;
+
+  const int waves_per_head = 4 / a.hpb;
+  const int head = hgroup * a.hpb + wave / waves_per_head;
+  const int row0 = block_row0 + (wave % waves_per_head) * kRW;
+  const int kv_head = head / (p.Hq / p.Hk);
+
+  const int shift = k_len - q_len;
+  int n_max = (k_len + kBN - 1) / kBN;
+  if (a.has_right) {
+    const int last = block_row0 + a.rows_per_block + shift + a.right_off_w;
+    const int lim = last <= 0 ? 0 : (last + kBN - 1) / kBN;
+    n_max = n_max < lim ? n_max : lim;
+  }
+  int n_min = 0;
+  if (a.has_left) {
+    const int first = block_row0 + shift - a.left_off_w;
+    n_min = first <= 0 ? 0 : first / kBN;
+  }
+
+  // ---- Q fragments ------------------------------------------------------------------------------
+  Frag qf[KS];
+  {
+    const int qrow = row0 + ql;
+    const bool row_ok = qrow < q_len;
+    const T* qp = (const T*)p.q + (int64_t)(q_bos + (row_ok ? qrow : 0)) * p.q_row_stride + (int64_t)head * p.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *reinterpret_cast<const u32x4*>(qp + ks * 16 + half * 8);
+      qf[ks] = __builtin_bit_cast(Frag, v);
+    }
+  }
+
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;  // running max (base-2 logits) and running sum
+
+  float slope = 0.f;
+  if (p.alibi_slopes != nullptr) slope = p.alibi_slopes[(int64_t)b * p.alibi_batch_stride + head] * 1.4426950408889634f;
+  const bool softcap = p.softcap > 0.f;
+
+  const int32_t* btab = p.block_table + (int64_t)b * p.block_table_stride;
+  const char* kbase = (const char*)((const T*)p.k_cache + (int64_t)kv_head * p.k_head_stride);
+  const char* vbase = (const char*)((const T*)p.v_cache + (int64_t)kv_head * p.v_head_stride);
+  const int page_size = p.page_size;
+  const int page_shift = a.page_shift;  // log2(page_size) or -1
+
+  // ---- DMA lane geometry (fixed per thread) -------------------------------------------------------
+  // instruction n = wave*IPW + j of an operand tile fills LDS bytes [n*1024, n*1024 + 1024); lane L
+  // lands at n*1024 + L*16 -> (key_l, position) and fetches the chunk that belongs there.
+  int dma_key[IPW], dma_coff[IPW];
+#pragma unroll
+  for (int j = 0; j < IPW; ++j) {
+    const int off = (wave * IPW + j) * 1024 + lane * 16;
+    const int key_l = off / RB, pos = (off % RB) / 16;
+    int c = pos ^ swz<CPR>(key_l);
+    if (c >= VALID_C) c = 0;  // padding region of the row: any finite data will do
+    dma_key[j] = key_l;
+    dma_coff[j] = c * 16;
+  }
+  auto issue_tile = [&](int nb, int stage) {
+    const int key0 = nb * kBN;
+    int64_t koff[IPW], voff[IPW];
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+      int key = key0 + dma_key[j];
+      key = key < k_len ? key : k_len - 1;
+      const int pg = page_shift >= 0 ? (key >> page_shift) : key / page_size;
+      const int64_t page = btab[pg];
+      const int slot = key - pg * page_size;
+      koff[j] = (page * p.k_page_stride + (int64_t)slot * p.k_row_stride) * (int64_t)sizeof(T) + dma_coff[j];
+      voff[j] = (page * p.v_page_stride + (int64_t)slot * p.v_row_stride) * (int64_t)sizeof(T) + dma_coff[j];
+    }
+    char* kdst = lds + stage * STAGEB + wave * IPW * 1024;
+    char* vdst = kdst + OPB;
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+      __builtin_amdgcn_global_load_lds(FG_GLBP(kbase + koff[j]), FG_LDSP(kdst + j * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(FG_GLBP(vbase + voff[j]), FG_LDSP(vdst + j * 1024), 16, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing (fixed per lane) ---------------------------------------------------------
+  // K fragment: row sigma(ql) of key sub-tile kt, chunk ks*2 + half  ->  ((ks*2) ^ kx) * 16 with kx = half ^ swz
+  const int k_row = sigma(ql);
+  const int k_lane = k_row * RB;
+  const int kx = half ^ swz<CPR>(k_row);
+  // V^T fragment via transposing reads: source lane s = lane%16 addresses key (s/4) of a group of 4 and the
+  // 8-byte piece (s%4) of the 32 bytes that hold d0 .. d0+15, d0 = dt*32 + 16*((lane/16)%2)
+  const int vs = lane & 15;
+  const int v_key0 = half * 8 + (vs >> 2);        // + t4*16 (+4 for the second read)
+  const int v_cc = 2 * ((lane >> 4) & 1) + ((vs & 3) >> 1);
+  const int v_byte = (vs & 1) * 8;
+  const int vx0 = v_cc ^ swz<CPR>(v_key0), vx1 = v_cc ^ swz<CPR>(v_key0 + 4);
+  const int v_lane0 = v_key0 * RB + v_byte, v_lane1 = (v_key0 + 4) * RB + v_byte;
+
+  const bool wave_rows_ok = row0 < q_len;
+  const int wave_row_last = (row0 + kRW - 1 < q_len ? row0 + kRW - 1 : q_len - 1);
+  const int qrow = row0 + ql;
+
+  if (n_min < n_max) issue_tile(n_min, 0);
+  for (int nb = n_min; nb < n_max; ++nb) {
+    const int stage = (nb - n_min) & 1;
+    const int key0 = nb * kBN;
+    FG_WAIT_VM(0);                   // this wave's share of tile nb has landed
+    __builtin_amdgcn_s_barrier();    // ... everybody's has, and nobody still reads the other stage
+    if (nb + 1 < n_max) issue_tile(nb + 1, stage ^ 1);
+
+    if (!wave_rows_ok) continue;
+    if (a.has_right && key0 > wave_row_last + shift + a.right_off_w) continue;
+    if (a.has_left && key0 + kBN - 1 < row0 + shift - a.left_off_w) continue;
+
+    const char* ks_base = lds + stage * STAGEB + k_lane;
+    const char* vs_base = lds + stage * STAGEB + OPB;
+
+    // ---- S^T = K . Q^T ----------------------------------------------------------------------------
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s_acc[kt][e] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const Frag kf = *reinterpret_cast<const Frag*>(ks_base + kt * 32 * RB + (((ks * 2) ^ kx) * 16));
+        s_acc[kt] = AttnMfma<T>::mma(kf, qf[ks], s_acc[kt]);
+      }
+    }
+
+    // ---- base-2 logits, masks, running max -----------------------------------------------------------
+    const bool need_mask = (key0 + kBN > k_len) || (a.has_right && key0 + kBN - 1 > row0 + shift + a.right_off_w) ||
+                           (a.has_left && key0 < wave_row_last + shift - a.left_off_w);
+    const bool plain = !softcap && p.alibi_slopes == nullptr;
+    float tmax = -INFINITY;
+    if (plain && !need_mask) {
+      // interior tile: raw scores; scale folded into the exponent below
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, s_acc[kt][e]);
+      tmax *= a.scale_log2;  // scale > 0, so max commutes with it
+    } else {
+      const int col_hi = a.has_right ? (qrow + shift + a.right_off_w < k_len - 1 ? qrow + shift + a.right_off_w : k_len - 1)
+                                     : k_len - 1;
+      const int col_lo = a.has_left ? qrow + shift - a.left_off_w : 0;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int col = key0 + kt * 32 + (e >> 3) * 16 + half * 8 + (e & 7);
+          float t = s_acc[kt][e];
+          if (softcap) t = a.cap_out_log2 * tanhf(t * a.cap_in);
+          else t = t * a.scale_log2;
+          if (p.alibi_slopes != nullptr) {
+            if (p.is_causal) t += slope * (float)(col - k_len + 1);
+            else t -= slope * fabsf((float)(col - shift - qrow));
+          }
+          if (col > col_hi || col < col_lo) t = -INFINITY;
+          s_acc[kt][e] = t;
+          tmax = fmaxf(tmax, t);
+        }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const bool moved = m_new != m_run;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float psum = 0.f;
+    Frag pf[4];
+    const float sc = (plain && !need_mask) ? a.scale_log2 : 1.0f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        T tmp[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float pv = __builtin_amdgcn_exp2f(fmaf(s_acc[kt][t2 * 8 + e], sc, -m_use));
+          psum += pv;
+          tmp[e] = (T)pv;
+        }
+        pf[kt * 2 + t2] = *reinterpret_cast<Frag*>(tmp);
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+
+    // ---- O^T = O^T * alpha + V^T . P^T  (rescale skipped while no row maximum of this wave moved) ---
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int o0 = ((dt * 4) ^ vx0) * 16, o1 = ((dt * 4) ^ vx1) * 16;
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(vs_base + v_lane0 + t4 * 16 * RB + o0));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(vs_base + v_lane1 + t4 * 16 * RB + o1));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o_acc[dt] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[t4], o_acc[dt]);
+      }
+    }
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------------------
+  if (qrow >= q_len) return;
+  const bool empty = l_run == 0.f || l_run != l_run;
+  const float inv = empty ? 1.f : 1.f / l_run;
+  if (p.lse != nullptr && half == 0) {
+    p.lse[(int64_t)head * p.total_q + q_bos + qrow] = empty ? INFINITY : m_run * 0.6931471805599453f + logf(l_run);
+  }
+  T* op = (T*)p.out + (int64_t)(q_bos + qrow) * p.o_row_stride + (int64_t)head * p.o_head_stride;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = dt * 32 + g * 8 + half * 4;
+      if (d < D) {
+        Pack<T, 4> o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.v[e] = (T)(o_acc[dt][g * 4 + e] * inv);
+        st_pack<T, 4>(op + d, o);
+      }
+    }
+}
+
+template <typename T, int D, int RB>
+int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
+  constexpr int LDS_BYTES = 2 * 2 * kBN * RB;
+  static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_varlen_async_kernel<T, D, RB>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+  if (attr_err != hipSuccess) {
+    fg_set_error("flash_attn_varlen_fwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(attr_err));
+    return FG_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((attn_varlen_async_kernel<T, D, RB>), grid, dim3(256), LDS_BYTES, st, a);
+  return fg_check_launch("flash_attn_varlen_fwd");
+}
+
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
+  if (a.use_async) {
+    switch (D) {
+      case 64: return launch_async<T, 64, 128>(a, grid, st);
+      case 96: return launch_async<T, 96, 256>(a, grid, st);
+      case 128: return launch_async<T, 128, 256>(a, grid, st);
+      case 192: return launch_async<T, 192, 512>(a, grid, st);
+      case 256: return launch_async<T, 256, 512>(a, grid, st);
+      default: break;
+    }
+  }
   if (D <= 64) hipLaunchKernelGGL((attn_varlen_kernel<T, 64>), grid, dim3(256), 0, st, a);
   else if (D <= 128) hipLaunchKernelGGL((attn_varlen_kernel<T, 128>), grid, dim3(256), 0, st, a);
   else if (D <= 192) hipLaunchKernelGGL((attn_varlen_kernel<T, 192>), grid, dim3(256), 0, st, a);
@@ -337,6 +655,13 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.scale_log2 = p.softmax_scale * log2e;
   a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
   a.cap_out_log2 = p.softcap * log2e;
+  a.page_shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == p.page_size) a.page_shift = sft;
+  {
+    const char* force = getenv("FG_ATTN_KERNEL");  // "sync" forces the register-staged kernel (debugging aid)
+    a.use_async = !(force != nullptr && force[0] == 's');
+  }
   dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
   hipStream_t st = (hipStream_t)stream;
   if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
