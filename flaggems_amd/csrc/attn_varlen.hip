@@ -34,6 +34,7 @@ namespace {
 constexpr int kBN = 64;        // keys per tile
 constexpr int kRW = 32;        // query rows per wave
 constexpr int kVtPitch = 144;  // V^T tile: row = 64 keys * 2 B + 16 B pad
+constexpr int kPageTabMaxBytes = 16384;  // LDS the asynchronous kernel may spend on block-table entries
 
 template <typename T> struct AttnMfma;
 template <> struct AttnMfma<bf16_t> {
@@ -59,6 +60,8 @@ struct AttnArgs {
   float cap_in, cap_out_log2;  // softcap: t = cap_out_log2 * tanh(S * cap_in)
   int page_shift;     // log2(page_size) when it is a power of two, else -1
   int use_async;      // take the asynchronous-tile kernel (head dims 64, 96, 128, 192, 256)
+  int nw, nst;        // waves per workgroup and LDS stages of the asynchronous kernel
+  int page_tab_entries;  // block-table entries the asynchronous kernel keeps in LDS (0: read them from global memory)
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -315,6 +318,34 @@ __global__ __launch_bounds__(256) void attn_varlen_kernel(AttnArgs a) {
 #define FG_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (7 << 4) | (0xF << 8) | (((N) >> 4) << 14))
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
+// ---- LDS reads the compiler must not reorder or guard ------------------------------------------------
+// The tile DMAs of later steps are still in flight while a step computes.  The compiler cannot tell
+// that they target other LDS stages and would wait for all of them (vmcnt(0)) before a transposing
+// LDS read; and left to itself it sinks every fragment read next to its first use.  So fragment
+// reads are issued through inline asm in groups, software-pipelined by hand: wait for group g (a full
+// lgkmcnt(0), tied to the group's registers), issue the reads of group g+1, then issue the MFMAs of
+// group g, which execute while the next reads are in flight.
+__device__ __forceinline__ uint32_t lds_off(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
+  return v;
+}
+__device__ __forceinline__ u32x2 lds_read_tr_b64(uint32_t addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr));
+  return v;
+}
+// Wait for every outstanding LDS read (and scalar load: they share the counter, and scalar loads
+// retire out of order, so a partial count can never be trusted here), tied to a group's registers.
+template <typename V>
+__device__ __forceinline__ void lds_wait_all(V (&r)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+}
+
 template <int CPR>
 __device__ __forceinline__ int swz(int key) {
   if constexpr (CPR >= 16) return (key & 8) | (((key >> 1) & 1) << 2) | ((key & 1) << 1) | ((key >> 2) & 1);
@@ -323,8 +354,8 @@ __device__ __forceinline__ int swz(int key) {
 
 // Two workgroups per CU when the tiles allow it (RB <= 256: 64 KB of LDS each); the wide-head
 // variants need 128 KB, run alone on a CU and may use the whole register file.
-template <typename T, int D, int RB>
-__global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_kernel(AttnArgs a) {
+template <typename T, int D, int RB, int NW, int NST, bool LP>
+__global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_async_kernel(AttnArgs a) {
   typedef typename AttnMfma<T>::Frag Frag;
   constexpr int CPR = RB / 16;          // 16-byte chunks per LDS row
   constexpr int VALID_C = D / 8;        // chunks that hold data
@@ -332,7 +363,7 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
   constexpr int DT = (D + 31) / 32;     // 32-row output sub-tiles over the head dim
   constexpr int OPB = kBN * RB;         // bytes of one operand tile
   constexpr int STAGEB = 2 * OPB;       // K tile + V tile
-  constexpr int IPW = RB / 64;          // DMA instructions per wave per operand per tile
+  constexpr int IPW = RB / 16 / NW;     // DMA instructions per wave per operand per tile
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   const FgFlashParams& p = a.p;
@@ -347,7 +378,7 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
   const int block_row0 = m_block * a.rows_per_block;
   if (block_row0 >= q_len) return;
 
-  const int waves_per_head = 4 / a.hpb;
+  const int waves_per_head = NW / a.hpb;
   const int head = hgroup * a.hpb + wave / waves_per_head;
   const int row0 = block_row0 + (wave % waves_per_head) * kRW;
   const int kv_head = head / (p.Hq / p.Hk);
@@ -365,7 +396,7 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
     n_min = first <= 0 ? 0 : first / kBN;
   }
 
-  // ---- Q fragments ------------------------------------------------------------------------------
+  // ---- Q fragments (async kernel) -----------------------------------------------------------------
   Frag qf[KS];
   {
     const int qrow = row0 + ql;
@@ -409,6 +440,39 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
     dma_key[j] = key_l;
     dma_coff[j] = c * 16;
   }
+  // Page ids.  The slice of the block table this workgroup walks is copied into LDS once, behind the
+  // tile stages, and every DMA lane looks its page up there: LDS reads retire on their own counter
+  // (lgkmcnt), so waiting for a page id never waits for a tile DMA (vmcnt), whereas a page id read
+  // from global memory after a DMA would, because memory operations retire in order.  When the
+  // slice does not fit the space reserved for it (LP == false) the ids are read from global memory.
+  int32_t* lds_pages = reinterpret_cast<int32_t*>(lds + NST * STAGEB);
+  const int pg_base = page_shift >= 0 ? ((n_min * kBN) >> page_shift) : (n_min * kBN) / page_size;
+  if constexpr (LP) {
+    const int last_key = (n_max * kBN < k_len ? n_max * kBN : k_len) - 1;
+    const int pg_last = last_key < 0 ? pg_base - 1 : (page_shift >= 0 ? (last_key >> page_shift) : last_key / page_size);
+    int count = pg_last - pg_base + 1;
+    count = count < a.page_tab_entries ? count : a.page_tab_entries;
+    for (int i = tid; i < count; i += NW * 64) lds_pages[i] = btab[pg_base + i];
+    __syncthreads();
+  }
+  int pg_id[IPW], pg_idx[IPW];
+  auto fetch_pages = [&](int nb) {
+    const int key0 = nb * kBN;
+#pragma unroll
+    for (int j = 0; j < IPW; ++j) {
+      int key = key0 + dma_key[j];
+      key = key < k_len ? key : k_len - 1;
+      const int pg = page_shift >= 0 ? (key >> page_shift) : key / page_size;
+      pg_idx[j] = pg;
+      if constexpr (LP) {
+        int rel = pg - pg_base;
+        rel = rel < a.page_tab_entries ? rel : a.page_tab_entries - 1;  // never read past the table
+        pg_id[j] = lds_pages[rel];
+      } else {
+        pg_id[j] = btab[pg];
+      }
+    }
+  };
   auto issue_tile = [&](int nb, int stage) {
     const int key0 = nb * kBN;
     int64_t koff[IPW], voff[IPW];
@@ -416,9 +480,8 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
     for (int j = 0; j < IPW; ++j) {
       int key = key0 + dma_key[j];
       key = key < k_len ? key : k_len - 1;
-      const int pg = page_shift >= 0 ? (key >> page_shift) : key / page_size;
-      const int64_t page = btab[pg];
-      const int slot = key - pg * page_size;
+      const int64_t page = pg_id[j];
+      const int slot = key - pg_idx[j] * page_size;
       koff[j] = (page * p.k_page_stride + (int64_t)slot * p.k_row_stride) * (int64_t)sizeof(T) + dma_coff[j];
       voff[j] = (page * p.v_page_stride + (int64_t)slot * p.v_row_stride) * (int64_t)sizeof(T) + dma_coff[j];
     }
@@ -449,31 +512,66 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
   const int wave_row_last = (row0 + kRW - 1 < q_len ? row0 + kRW - 1 : q_len - 1);
   const int qrow = row0 + ql;
 
-  if (n_min < n_max) issue_tile(n_min, 0);
+  // Prologue: NST-1 tiles in flight.  In the loop, tile nb has landed once at most NST-2 newer steps
+  // (2*IPW DMA instructions each, plus IPW page-id loads before them when those are global loads)
+  // are outstanding.
+  // vmcnt events per step: 2*IPW DMA, plus IPW page-id loads when those come from global memory
+  constexpr int PER_TILE = LP ? 2 * IPW : 3 * IPW;
+#pragma unroll
+  for (int s0 = 0; s0 < NST - 1; ++s0) {
+    if (n_min + s0 < n_max) {
+      fetch_pages(n_min + s0);
+      issue_tile(n_min + s0, s0);
+    }
+  }
   for (int nb = n_min; nb < n_max; ++nb) {
-    const int stage = (nb - n_min) & 1;
+    const int stage = (nb - n_min) % NST;
     const int key0 = nb * kBN;
-    FG_WAIT_VM(0);                   // this wave's share of tile nb has landed
-    __builtin_amdgcn_s_barrier();    // ... everybody's has, and nobody still reads the other stage
-    if (nb + 1 < n_max) issue_tile(nb + 1, stage ^ 1);
+    if (NST > 2 && nb + NST - 2 < n_max) {
+      FG_WAIT_VM((NST - 2) * PER_TILE);
+    } else {
+      FG_WAIT_VM(0);                 // this wave's share of tile nb has landed
+    }
+    __builtin_amdgcn_s_barrier();    // ... everybody's has, and nobody still reads the stage refilled next
+    if (nb + NST - 1 < n_max) {
+      fetch_pages(nb + NST - 1);
+      issue_tile(nb + NST - 1, (nb - n_min + NST - 1) % NST);
+    }
 
     if (!wave_rows_ok) continue;
     if (a.has_right && key0 > wave_row_last + shift + a.right_off_w) continue;
     if (a.has_left && key0 + kBN - 1 < row0 + shift - a.left_off_w) continue;
 
-    const char* ks_base = lds + stage * STAGEB + k_lane;
-    const char* vs_base = lds + stage * STAGEB + OPB;
+    const uint32_t ks_base = lds_off(lds) + stage * STAGEB + k_lane;
+    const uint32_t vs_base = lds_off(lds) + stage * STAGEB + OPB;
 
-    // ---- S^T = K . Q^T ----------------------------------------------------------------------------
+    // ---- S^T = K . Q^T : K fragments in groups of GS reads, one group ahead of the MFMAs ---------------
+    constexpr int GS = KS < 8 ? KS : 8;        // reads per group
+    constexpr int NGK = 2 * KS / GS;           // groups over both key sub-tiles
     f32x16 s_acc[2];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) s_acc[kt][e] = 0.f;
+    {
+      u32x4 kf[2][8];
+      auto issue_k = [&](int g, u32x4 (&dst)[8]) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const Frag kf = *reinterpret_cast<const Frag*>(ks_base + kt * 32 * RB + (((ks * 2) ^ kx) * 16));
-        s_acc[kt] = AttnMfma<T>::mma(kf, qf[ks], s_acc[kt]);
+        for (int r = 0; r < GS; ++r) {
+          const int idx = g * GS + r, kt = idx / KS, ks = idx % KS;
+          dst[r] = lds_read_b128(ks_base + kt * 32 * RB + (((ks * 2) ^ kx) * 16));
+        }
+      };
+      issue_k(0, kf[0]);
+#pragma unroll
+      for (int g = 0; g < NGK; ++g) {
+        lds_wait_all(kf[g & 1]);
+        if (g + 1 < NGK) issue_k(g + 1, kf[(g + 1) & 1]);
+#pragma unroll
+        for (int r = 0; r < GS; ++r) {
+          const int idx = g * GS + r, kt = idx / KS, ks = idx % KS;
+          s_acc[kt] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, kf[g & 1][r]), qf[ks], s_acc[kt]);
+        }
       }
     }
 
@@ -542,18 +640,27 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
 #pragma unroll
         for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
     }
+    {
+      // V^T fragments: per d sub-tile 8 transposing reads (4 key chunks x 2 halves), one sub-tile ahead
+      u32x2 vf[2][8];
+      auto issue_v = [&](int dt, u32x2 (&dst)[8]) {
+        const int o0 = ((dt * 4) ^ vx0) * 16, o1 = ((dt * 4) ^ vx1) * 16;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const int o0 = ((dt * 4) ^ vx0) * 16, o1 = ((dt * 4) ^ vx1) * 16;
+        for (int t4 = 0; t4 < 4; ++t4) {
+          dst[2 * t4] = lds_read_tr_b64(vs_base + v_lane0 + t4 * 16 * RB + o0);
+          dst[2 * t4 + 1] = lds_read_tr_b64(vs_base + v_lane1 + t4 * 16 * RB + o1);
+        }
+      };
+      issue_v(0, vf[0]);
 #pragma unroll
-      for (int t4 = 0; t4 < 4; ++t4) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4*)(vs_base + v_lane0 + t4 * 16 * RB + o0));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4*)(vs_base + v_lane1 + t4 * 16 * RB + o1));
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        o_acc[dt] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[t4], o_acc[dt]);
+      for (int dt = 0; dt < DT; ++dt) {
+        lds_wait_all(vf[dt & 1]);
+        if (dt + 1 < DT) issue_v(dt + 1, vf[(dt + 1) & 1]);
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) {
+          const u32x4 both = {vf[dt & 1][2 * t4][0], vf[dt & 1][2 * t4][1], vf[dt & 1][2 * t4 + 1][0], vf[dt & 1][2 * t4 + 1][1]};
+          o_acc[dt] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[t4], o_acc[dt]);
+        }
       }
     }
   }
@@ -580,30 +687,47 @@ __global__ __launch_bounds__(256, (RB <= 256 ? 2 : 1)) void attn_varlen_async_ke
     }
 }
 
-template <typename T, int D, int RB>
-int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
-  constexpr int LDS_BYTES = 2 * 2 * kBN * RB;
-  static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_varlen_async_kernel<T, D, RB>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+template <typename T, int D, int RB, int NW, int NST, bool LP>
+int launch_async_lp(const AttnArgs& a, dim3 grid, hipStream_t st) {
+  constexpr int STAGE_BYTES = NST * 2 * kBN * RB;
+  constexpr int MAX_LDS = STAGE_BYTES + kPageTabMaxBytes;
+  static hipError_t attr_err =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(attn_varlen_async_kernel<T, D, RB, NW, NST, LP>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS);
   if (attr_err != hipSuccess) {
-    fg_set_error("flash_attn_varlen_fwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(attr_err));
+    fg_set_error("flash_attn_varlen_fwd: cannot reserve %d bytes of LDS: %s", MAX_LDS, hipGetErrorString(attr_err));
     return FG_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((attn_varlen_async_kernel<T, D, RB>), grid, dim3(256), LDS_BYTES, st, a);
+  const int lds_bytes = STAGE_BYTES + (LP ? a.page_tab_entries * 4 : 0);
+  hipLaunchKernelGGL((attn_varlen_async_kernel<T, D, RB, NW, NST, LP>), grid, dim3(NW * 64), lds_bytes, st, a);
   return fg_check_launch("flash_attn_varlen_fwd");
+}
+template <typename T, int D, int RB, int NW, int NST>
+int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
+  if (a.page_tab_entries > 0) return launch_async_lp<T, D, RB, NW, NST, true>(a, grid, st);
+  return launch_async_lp<T, D, RB, NW, NST, false>(a, grid, st);
 }
 
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
   if (a.use_async) {
-    switch (D) {
-      case 64: return launch_async<T, 64, 128>(a, grid, st);
-      case 96: return launch_async<T, 96, 256>(a, grid, st);
-      case 128: return launch_async<T, 128, 256>(a, grid, st);
-      case 192: return launch_async<T, 192, 512>(a, grid, st);
-      case 256: return launch_async<T, 256, 512>(a, grid, st);
-      default: break;
+    if (a.nw == 8) {
+      switch (D) {
+        case 64: return a.nst == 3 ? launch_async<T, 64, 128, 8, 3>(a, grid, st) : launch_async<T, 64, 128, 8, 2>(a, grid, st);
+        case 96: return a.nst == 3 ? launch_async<T, 96, 256, 8, 3>(a, grid, st) : launch_async<T, 96, 256, 8, 2>(a, grid, st);
+        case 128: return a.nst == 3 ? launch_async<T, 128, 256, 8, 3>(a, grid, st) : launch_async<T, 128, 256, 8, 2>(a, grid, st);
+        default: break;
+      }
+    } else {
+      switch (D) {
+        case 64: return launch_async<T, 64, 128, 4, 2>(a, grid, st);
+        case 96: return launch_async<T, 96, 256, 4, 2>(a, grid, st);
+        case 128: return launch_async<T, 128, 256, 4, 2>(a, grid, st);
+        case 192: return launch_async<T, 192, 512, 4, 2>(a, grid, st);
+        case 256: return launch_async<T, 256, 512, 4, 2>(a, grid, st);
+        default: break;
+      }
     }
   }
   if (D <= 64) hipLaunchKernelGGL((attn_varlen_kernel<T, 64>), grid, dim3(256), 0, st, a);
@@ -642,7 +766,29 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.p = p;
   const int ratio = p.Hq / p.Hk;
   a.hpb = ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1);
-  a.rows_per_block = 128 / a.hpb;
+  a.page_shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == p.page_size) a.page_shift = sft;
+  // Kernel variant.  Head dims 64/96/128 take 8 waves sharing each K/V tile, three LDS stages deep;
+  // 192/256 take 4 waves and two stages; everything else the register-staged kernel.
+  // FG_ATTN_KERNEL = "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
+  a.use_async = (p.D == 64 || p.D == 96 || p.D == 128 || p.D == 192 || p.D == 256) ? 1 : 0;
+  a.nw = p.D <= 128 ? 8 : 4;
+  a.nst = p.D <= 128 ? 3 : 2;
+  if (const char* force = getenv("FG_ATTN_KERNEL")) {
+    if (force[0] == 's') a.use_async = 0;
+    if (force[0] == 'w' && p.D <= 128) {
+      a.nw = force[1] == '8' ? 8 : 4;
+      a.nst = (force[2] == 's' && force[3] == '3' && a.nw == 8) ? 3 : 2;
+    }
+  }
+  {
+    // LDS copy of the block-table slice: sized for the longest sequence, capped at kPageTabMaxBytes
+    const int64_t need = fg_cdiv(p.max_seqlen_k > 0 ? p.max_seqlen_k : 1, p.page_size) + 1;
+    a.page_tab_entries = need * 4 <= kPageTabMaxBytes ? (int)((need + 3) / 4 * 4) : 0;
+  }
+  const int waves = a.use_async ? a.nw : 4;
+  a.rows_per_block = waves * 32 / a.hpb;
   // Mask bounds (bottom-right aligned): keys col with col > row + shift + right or col < row + shift - left are
   // masked.  causal forces right = 0; a one-sided window leaves the other side open.
   int wl = p.window_left, wr = p.window_right;
@@ -655,13 +801,6 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.scale_log2 = p.softmax_scale * log2e;
   a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
   a.cap_out_log2 = p.softcap * log2e;
-  a.page_shift = -1;
-  for (int sft = 0; sft < 31; ++sft)
-    if ((1 << sft) == p.page_size) a.page_shift = sft;
-  {
-    const char* force = getenv("FG_ATTN_KERNEL");  // "sync" forces the register-staged kernel (debugging aid)
-    a.use_async = !(force != nullptr && force[0] == 's');
-  }
   dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
   hipStream_t st = (hipStream_t)stream;
   if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
