@@ -185,16 +185,20 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
       float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * kTileElems;
 #pragma unroll
       for (int j = 0; j < kEPT; ++j) st_coherent(slot + tid + kBlock * j, sum[j]);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      // The partial tile is written with device-coherent (write-through) stores, so no cache
+      // write-back is needed to publish it: it is enough that every store has completed
+      // (the workgroup-scope fence waits for that) before the ticket is drawn.  A device-scope
+      // release/acquire pair here would flush and invalidate the whole L2 and costs more than the
+      // rest of the kernel.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();  // every thread's slice of the partial tile is out
       const int w_first = worker_of(a.per, a.rem, tile_begin);
       const int w_last = worker_of(a.per, a.rem, tile_end - 1);
       if (tid == 0)
-        ticket_s = __hip_atomic_fetch_add(a.tickets + w_first, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        ticket_s = __hip_atomic_fetch_add(a.tickets + w_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       if (ticket_s == (unsigned)(w_last - w_first)) {
-        finish = true;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        finish = true;  // the loads below bypass the non-coherent caches (device-coherent loads)
 #pragma unroll
         for (int j = 0; j < kEPT; ++j) sum[j] = 0.f;
         for (int w2 = w_first; w2 <= w_last; ++w2) {

@@ -383,16 +383,17 @@ __global__ __launch_bounds__(kThreads) void gemm_streamk_kernel(GemmArgs g) {
           for (int e = 0; e < 16; ++e)
             __hip_atomic_store(slot + ((i * TC::TN + j) * 16 + e) * kThreads + tid, acc[i][j][e], __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      // device-coherent stores need no cache write-back to be visible; waiting for their completion
+      // (workgroup-scope fence) before the ticket is enough, and far cheaper than flushing L2
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();  // every thread's slice of the partial tile is out
       const int w_first = sk_worker_of(g.sk_per, g.sk_rem, tile_begin);
       const int w_last = sk_worker_of(g.sk_per, g.sk_rem, tile_end - 1);
       if (tid == 0)
-        ticket_s = __hip_atomic_fetch_add(g.tickets + w_first, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        ticket_s = __hip_atomic_fetch_add(g.tickets + w_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       if (ticket_s == (unsigned)(w_last - w_first)) {
-        finish = true;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        finish = true;  // the loads below are device-coherent: they bypass the non-coherent caches
 #pragma unroll
         for (int i = 0; i < TC::TM; ++i)
 #pragma unroll
