@@ -179,13 +179,15 @@ int softmax_dispatch(const TI* in, TO* out, int64_t M, int64_t N, int64_t K, hip
   } else if (packs <= 128) {
     FG_ROWS(2, 64);
   } else if (packs <= 256) {
-    FG_ROWS(4, 64);
+    // two packs per thread, two waves per row: 166.7 us on [131072, 2048] bf16 against 170.4 us
+    // (four packs, one wave) and 175.7 us (one pack, four waves) on MI355X
+    FG_ROWS(2, 128);
   } else if (packs <= 512) {
-    FG_ROWS(4, 128);
+    FG_ROWS(2, 256);
   } else if (packs <= 1024) {
-    FG_ROWS(4, 256);
+    FG_ROWS(2, 512);
   } else if (packs <= 2048) {
-    FG_ROWS(4, 512);
+    FG_ROWS(2, 1024);
   } else if (packs <= 4096) {
     FG_ROWS(4, 1024);
   } else {
