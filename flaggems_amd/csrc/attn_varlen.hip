@@ -338,6 +338,28 @@ __device__ __forceinline__ u32x2 lds_read_tr_b64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(addr));
   return v;
 }
+// Combine a value with the one held by lane ^ 32 without going through LDS: v_permlane32_swap
+// exchanges the upper half of its first register with the lower half of its second, so with both
+// holding v on entry the first ends as the lower-half value and the second as the upper-half value
+// of every lane position.  Written as asm because the builtin's second result is not usable with
+// this compiler; the no-ops cover the VALU-write -> permlane-read distance the compiler would
+// otherwise insert itself.
+__device__ __forceinline__ void xhalf_split(float v, float& lo, float& hi) {
+  lo = v;
+  hi = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float xhalf_max(float v) {
+  float lo, hi;
+  xhalf_split(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float xhalf_sum(float v) {
+  float lo, hi;
+  xhalf_split(v, lo, hi);
+  return lo + hi;
+}
+
 // Wait for every outstanding LDS read (and scalar load: they share the counter, and scalar loads
 // retire out of order, so a partial count can never be trusted here), tied to a group's registers.
 template <typename V>
@@ -346,14 +368,21 @@ __device__ __forceinline__ void lds_wait_all(V (&r)[8]) {
                : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
 }
 
+// Chunk swizzle: 16-byte chunk c of LDS row `key` is stored at position c ^ swz(key).
+// Written with key bits k3 k2 k1 k0:
+//   rows of 16 or 32 chunks: swz = (k1, k0, k3, k2).  The 16 keys of one K-fragment read get 16
+//     different values (a bit permutation), so a quarter-wave of ds_read_b128 covers all banks once.
+//     For a transposed V read the 32-byte pair index is swz >> 1 = (k1, k0, k3): the 4 consecutive keys
+//     of a 16-lane group land in pairs P ^ {0, 2, 4, 6} (+k3), and the neighbouring group, which
+//     reads pair P + 1 of the same keys in the same cycle, in (P + 1) ^ {0, 2, 4, 6}: disjoint.
+//   rows of 8 chunks (two rows per 256 bytes of banks, row parity = k0): swz = (k1, k2, k3); the
+//     same two properties hold with the row parity taking the place of the missing bit.
 template <int CPR>
 __device__ __forceinline__ int swz(int key) {
-  if constexpr (CPR >= 16) return (key & 8) | (((key >> 1) & 1) << 2) | ((key & 1) << 1) | ((key >> 2) & 1);
+  if constexpr (CPR >= 16) return ((key & 3) << 2) | (((key >> 3) & 1) << 1) | ((key >> 2) & 1);
   else return (((key >> 1) & 1) << 2) | (((key >> 2) & 1) << 1) | ((key >> 3) & 1);
 }
 
-// Two workgroups per CU when the tiles allow it (RB <= 256: 64 KB of LDS each); the wide-head
-// variants need 128 KB, run alone on a CU and may use the whole register file.
 template <typename T, int D, int RB, int NW, int NST, bool LP>
 __global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_async_kernel(AttnArgs a) {
   typedef typename AttnMfma<T>::Frag Frag;
@@ -608,11 +637,14 @@ __global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_asyn
           tmax = fmaxf(tmax, t);
         }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
+    tmax = xhalf_max(tmax);
+    // The reference maximum of a row moves only when the new maximum exceeds it by more than 2^8:
+    // any reference gives the same result as long as p and the running sum use the same one, and
+    // p <= 256 is harmless in bf16/fp16.  After the first steps almost no step has to rescale.
+    const bool moved = tmax > m_run + 8.0f;
+    const float m_new = moved ? tmax : m_run;
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const bool moved = m_new != m_run;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    const float alpha = moved ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.0f;
     float psum = 0.f;
     Frag pf[4];
     const float sc = (plain && !need_mask) ? a.scale_log2 : 1.0f;
@@ -629,11 +661,11 @@ __global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_asyn
         }
         pf[kt * 2 + t2] = *reinterpret_cast<Frag*>(tmp);
       }
-    psum += __shfl_xor(psum, 32, 64);
+    psum = xhalf_sum(psum);
     l_run = l_run * alpha + psum;
     m_run = m_new;
 
-    // ---- O^T = O^T * alpha + V^T . P^T  (rescale skipped while no row maximum of this wave moved) ---
+    // ---- O^T = O^T * alpha + V^T . P^T  (rescale skipped while no reference maximum of this wave moved) ---
     if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
@@ -769,12 +801,13 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.page_shift = -1;
   for (int sft = 0; sft < 31; ++sft)
     if ((1 << sft) == p.page_size) a.page_shift = sft;
-  // Kernel variant.  Head dims 64/96/128 take 8 waves sharing each K/V tile, three LDS stages deep;
-  // 192/256 take 4 waves and two stages; everything else the register-staged kernel.
+  // Kernel variant.  Head dims 64/96/128/192/256 take the asynchronous-tile kernel with 4 waves and
+  // two LDS stages (measured fastest; the 8-wave variants stay selectable for head dims <= 128);
+  // everything else the register-staged kernel.
   // FG_ATTN_KERNEL = "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
   a.use_async = (p.D == 64 || p.D == 96 || p.D == 128 || p.D == 192 || p.D == 256) ? 1 : 0;
-  a.nw = p.D <= 128 ? 8 : 4;
-  a.nst = p.D <= 128 ? 3 : 2;
+  a.nw = 4;
+  a.nst = 2;
   if (const char* force = getenv("FG_ATTN_KERNEL")) {
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && p.D <= 128) {
