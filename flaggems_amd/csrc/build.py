@@ -24,6 +24,7 @@ SOURCES = [
     "gemm.hip",
     "gemm_skinny.hip",
     "gemm_streamk.hip",
+    "gemm_dma.hip",
     "attn_varlen.hip",
 ]
 

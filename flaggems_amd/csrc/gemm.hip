@@ -1,5 +1,7 @@
 // Host side of fg_gemm: validation, load-mode and tile selection, schedule selection, launches.
+#include <cstdlib>
 #include <mutex>
+#include <type_traits>
 #include "gemm_tile.h"
 
 namespace fgk {
@@ -13,6 +15,10 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
 size_t streamk_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int num_cu);
 int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace, size_t workspace_bytes, int num_cu,
                    hipStream_t st);
+
+// implemented in gemm_dma.hip
+bool dma_supported(const GemmArgs& g, int elem_bytes);
+int dma_launch(const GemmArgs& g, int dtype, hipStream_t st);
 
 int num_cus(int device) {
   static std::mutex mu;
@@ -93,6 +99,9 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
     if (amode != LOAD_GEN && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
       set_tiles(g, 256, 256, BK);
+      // aligned operands with K a multiple of 64 take the direct-to-LDS kernel
+      if (dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr)
+        return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, st);
       return launch_dp_modes<T, 256, 256>(g, amode, bmode, st);
     }
   }

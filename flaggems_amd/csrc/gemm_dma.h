@@ -1,0 +1,286 @@
+// Direct-to-LDS MFMA GEMM for gfx950, 16-bit inputs: C[M,N] = alpha * A[M,K].B[K,N] + beta * bias.
+//
+// The large-matrix kernel.  A 256x256 output tile per workgroup, 4 waves in a 2x2 grid, each wave a
+// 128x128 sub-tile held as 4x4 MFMA 32x32 accumulators (256 accumulator registers per lane).
+//
+// Data movement.  Each K step covers 64 elements = one full 128-byte cache line per tile row.  The
+// operand tiles go from global memory straight into LDS with global_load_lds_dwordx4: no staging
+// registers, no LDS store instructions.  One such instruction writes 64 lanes x 16 bytes to 1 KB of
+// consecutive LDS, but every lane chooses its own global address, so the 16-byte chunks are laid
+// out swizzled: what the fragment reads below need to be free of bank conflicts without any row
+// padding.  LDS holds two stages (2 x 64 KB).
+//
+//   A (K contiguous), and B when it is K contiguous (B = W^T, "NT"):
+//     stage layout [row][128 B]; chunk c of row r sits at position c ^ ((r >> 1) & 7).  A fragment
+//     (8 consecutive k of one row per lane) is one ds_read_b128; the 16 rows a quarter-wave reads
+//     fall into 16 different 16-byte bank groups.
+//   B when it is N contiguous (row-major [K,N], "NN"):
+//     stage layout [k][512 B] (the 256 columns of the tile); chunk c of row k sits at position
+//     c ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)).  The fragment is produced by two
+//     ds_read_b64_tr_b16, which transpose 4 k-rows x 4 column groups among 16 lanes while reading.
+//
+// Schedule.  The K step is cut into four sub-steps of one MFMA K (16): sub-step s issues its 16
+// MFMAs on fragment set s&1 while the reads for sub-step s+1 fill the other set, one LDS read per
+// MFMA.  Sub-step 3 already reads the first fragments of the next stage, so the MFMA pipe does not
+// drain at a stage boundary.  One barrier per K step, after sub-step 2: by then this wave has issued
+// and completed every read of the current stage (the stage may be refilled) and every DMA it issued
+// for the next stage has landed (vmcnt(0)).  The refill for stage kb+2 is issued right behind that
+// barrier, spread over sub-step 3 and sub-step 0 of the next step (one DMA per MFMA), which leaves
+// it two to three sub-steps to land.  The compiler's own scheduling is pinned with sched_barrier
+// after every MFMA group; it keeps no counters for the DMA writes, hence the explicit waits.
+//
+// The MFMA operands are swapped (B fragment first), so a lane's accumulator registers hold 4
+// consecutive output columns of one output row; after packing to 16 bits, two v_permlane32_swap
+// give every lane 8 consecutive columns and the tile is written with 16-byte stores.
+//
+// Preconditions (checked on the host): 16-bit type; A K-contiguous; B K- or N-contiguous; K a
+// multiple of 64; N a multiple of 8; operand base pointers and row strides multiples of 16 bytes;
+// C with unit column stride and 16-byte aligned rows; a bias with unit column stride and 8-byte
+// aligned rows.  M and N are otherwise arbitrary: tile rows past the edge are clamped to the last
+// valid row (or 8-column chunk) on load and never stored.  Everything else runs on the
+// register-staged kernel.
+#pragma once
+#include "gemm_tile.h"
+
+namespace fgk {
+
+constexpr int kDmaRowB = 128;                 // bytes of K per stage per A row
+constexpr int kDmaOpB = 256 * kDmaRowB;       // one operand, one stage: 32 KB
+constexpr int kDmaStageB = 2 * kDmaOpB;
+constexpr int kDmaLdsBytes = 2 * kDmaStageB;  // 128 KB
+constexpr int kDmaBK = 64;
+
+#define FGK_LDSP(p) ((__attribute__((address_space(3))) void*)(p))
+#define FGK_GLBP(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FGK_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (7 << 4) | (0xF << 8) | (((N) >> 4) << 14))
+#define FGK_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F) /* vmcnt 63, expcnt 7, lgkmcnt 0 */
+
+template <int I> struct IntC { static constexpr int value = I; };
+template <int B, int E, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(IntC<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return v;
+}
+// Waits for every outstanding LDS read; tied to the registers the inline-asm reads wrote so that
+// nothing consuming them can be placed ahead of the wait.
+__device__ __forceinline__ void lds_wait_tied(u32x4 (&r)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+}
+// X.upper-half-lanes <-> Y.lower-half-lanes, for two register pairs at once
+__device__ __forceinline__ void swap_halves2(unsigned& x0, unsigned& y0, unsigned& x1, unsigned& y1) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+               : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
+}
+
+template <typename T, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs g) {
+  static_assert(sizeof(T) == 2, "16-bit element types");
+  typedef typename Mfma<T>::Frag Frag;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
+  const int row0 = tm * 256, col0 = tn * 256;
+  const int M = (int)g.M, N = (int)g.N;
+  const int nk = (int)(g.K / kDmaBK);
+
+  // ---- DMA source addresses.  Wave w issues instructions j = 0..7 per operand and stage; the LDS
+  // destination of instruction j is base + (j/4)*4096 (through M0) + (j%4)*1024 (immediate).  The
+  // hardware adds the immediate to the global address as well, so it is subtracted here.
+  const char* a_src[8];
+  const char* b_src[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    {
+      const int r = (wave * 8 + j) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
+      int ra = row0 + r;
+      ra = ra < M ? ra : M - 1;
+      a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024;
+    }
+    if constexpr (B_KC) {
+      const int r = (wave * 8 + j) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
+      int rb = col0 + r;
+      rb = rb < N ? rb : N - 1;
+      b_src[j] = (const char*)g.B + ((int64_t)rb * g.sbn + c * 8) * 2 - (j & 3) * 1024;
+    } else {
+      const int k = (wave * 8 + j) * 2 + (lane >> 5);
+      const int c = (lane & 31) ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1));
+      int cb = col0 + c * 8;
+      cb = cb + 8 <= N ? cb : N - 8;
+      b_src[j] = (const char*)g.B + ((int64_t)k * g.sbk + cb) * 2 - (j & 3) * 1024;
+    }
+  }
+  const int64_t b_step = B_KC ? (int64_t)kDmaRowB : g.sbk * (int64_t)(kDmaBK * 2);  // bytes per K step
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  char* const dma_base = lds + wave_s * 8192;
+  auto issue = [&](int kb, auto jc) {
+    constexpr int j = decltype(jc)::value;  // 0..15: the A instructions, then the B instructions
+    constexpr int jj = j & 7;
+    char* l = dma_base + (kb & 1) * kDmaStageB + (j < 8 ? 0 : kDmaOpB) + (jj >> 2) * 4096;
+    const char* gp = j < 8 ? a_src[jj] + (int64_t)kb * kDmaRowB : b_src[jj] + (int64_t)kb * b_step;
+    __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
+  };
+
+  // ---- fragment addresses
+  const int fr = lane & 31, fh = lane >> 5;
+  const int q = (fr >> 1) & 7;  // sub-tile rows start at multiples of 32, so (row >> 1) & 7 depends on fr only
+  const int a_lane = (wm * 128 + fr) * kDmaRowB;
+  int pos[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) pos[s] = ((2 * s + fh) ^ q) * 16;
+  int b_lane = 0;          // K-contiguous B: like A
+  uint32_t b_tr[4] = {0, 0, 0, 0};  // N-contiguous B: per sub-tile j, the lane's address within a stage
+  if constexpr (B_KC) {
+    b_lane = kDmaOpB + (wn * 128 + fr) * kDmaRowB;
+  } else {
+    const int m = (lane & 15) >> 2, hh = lane >> 5, b4 = (lane >> 4) & 1, b1 = (lane & 3) >> 1;
+    const int krow = 8 * hh + m;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int chunk = wn * 16 + ((j ^ m) << 2) + (((b4 ^ hh) << 1) | b1);
+      b_tr[j] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + kDmaOpB + krow * 512 + chunk * 16 +
+                (lane & 1) * 8;
+    }
+  }
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  Frag fa[2][4];
+  u32x4 fb[2][4];
+  // read x of fragment set `set` for sub-step S of `stage`: x < 4 -> A sub-tile x, else B sub-tile x-4
+  auto read_one = [&](int stage, auto sc, auto xc, int set) {
+    constexpr int S = decltype(sc)::value;
+    constexpr int x = decltype(xc)::value;
+    const int sb = (stage & 1) * kDmaStageB;
+    if constexpr (x < 4) {
+      fa[set][x] = *reinterpret_cast<const Frag*>(lds + sb + a_lane + x * 32 * kDmaRowB + pos[S]);
+    } else if constexpr (B_KC) {
+      fb[set][x - 4] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + (x - 4) * 32 * kDmaRowB + pos[S]);
+    } else {
+      const u32x2 lo = lds_read_tr16_b64<(16 * S) * 512>(b_tr[x - 4] + sb);
+      const u32x2 hi = lds_read_tr16_b64<(16 * S + 4) * 512>(b_tr[x - 4] + sb);
+      fb[set][x - 4] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
+  auto wait_reads = [&](int set) {
+    if constexpr (B_KC) FGK_WAIT_LGKM0();
+    else lds_wait_tied(fb[set]);
+  };
+
+  // ---- prologue: stage 0, and the head of stage 1 (the part sub-step 3 of the step before would issue)
+  static_for<0, 16>([&](auto jc) { issue(0, jc); });
+  if (nk > 1) {
+    static_for<0, 8>([&](auto jc) { issue(1, jc); });
+    FGK_WAIT_VM(8);
+  } else {
+    FGK_WAIT_VM(0);
+  }
+  __builtin_amdgcn_s_barrier();
+  static_for<0, 8>([&](auto xc) { read_one(0, IntC<0>{}, xc, 0); });
+  wait_reads(0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // One K step.  REFILL_TAIL: sub-steps 0 issue the second half of the DMAs of stage kb+1;
+  // REFILL_HEAD: sub-step 3 issues the first half of the DMAs of stage kb+2.
+  auto k_step = [&](int kb, auto tail_c, auto head_c) {
+    constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
+    constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
+    static_for<0, 4>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      constexpr int cur = s & 1, nxt = cur ^ 1;
+      static_for<0, 16>([&](auto xc) {
+        constexpr int x = decltype(xc)::value;
+        constexpr int i = x >> 2, j = x & 3;
+        acc[i][j] = Mfma<T>::mma(__builtin_bit_cast(Frag, fb[cur][j]), fa[cur][i], acc[i][j]);
+        if constexpr (x < 8) {
+          if constexpr (s < 3) read_one(kb, IntC<s + 1>{}, xc, nxt);
+          else read_one(kb + 1, IntC<0>{}, xc, nxt);
+        }
+        if constexpr (s == 3 && REFILL_HEAD && x < 8) issue(kb + 2, IntC<x>{});
+        if constexpr (s == 0 && REFILL_TAIL && x < 8) issue(kb + 1, IntC<8 + x>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if constexpr (s == 2) {
+        FGK_WAIT_VM(0);
+        wait_reads(nxt);
+        __builtin_amdgcn_s_barrier();
+      } else {
+        wait_reads(nxt);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  int kb = 0;
+  for (; kb < nk - 2; ++kb) k_step(kb, IntC<1>{}, IntC<1>{});
+  if (kb == nk - 2) {
+    k_step(kb, IntC<1>{}, IntC<0>{});
+    ++kb;
+  }
+  k_step(kb, IntC<0>{}, IntC<0>{});
+
+  // ---- epilogue (the host guarantees: C rows 16-byte aligned with unit column stride, N a multiple
+  // of 8, bias -- if any -- with unit column stride and 8-byte aligned rows)
+  T* C = (T*)g.C;
+  const T* bias = (const T*)g.bias;
+  const float alpha = g.alpha, beta = g.beta;
+  const bool scale = alpha != 1.0f;
+  const int lr = lane & 31, lh = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t r = row0 + wm * 128 + i * 32 + lr;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int cbase = col0 + wn * 128 + j * 32;
+      // element e of this lane: row r, column cbase + (e/4)*8 + lh*4 + e%4
+      if (bias != nullptr) {
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          const int c = cbase + gq * 8 + lh * 4;
+          typedef T T4 __attribute__((ext_vector_type(4)));
+          T4 t = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+#pragma unroll
+          for (int t4 = 0; t4 < 4; ++t4)
+            acc[i][j][gq * 4 + t4] = acc[i][j][gq * 4 + t4] * alpha + (float)t[t4] * beta;
+        }
+      } else if (scale) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] *= alpha;
+      }
+      unsigned pk[8];
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        typedef T T2 __attribute__((ext_vector_type(2)));
+        const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
+        pk[d] = __builtin_bit_cast(unsigned, t);
+      }
+#pragma unroll
+      for (int gp = 0; gp < 2; ++gp) {
+        // register groups 2gp (X) and 2gp+1 (Y): after X.upper <-> Y.lower the lower half-wave owns
+        // the 8 columns of group 2gp, the upper half-wave those of group 2gp+1
+        unsigned x0 = pk[4 * gp], x1 = pk[4 * gp + 1], y0 = pk[4 * gp + 2], y1 = pk[4 * gp + 3];
+        swap_halves2(x0, y0, x1, y1);
+        const int c = cbase + (2 * gp + lh) * 8;
+        if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
+      }
+    }
+  }
+}
+
+}  // namespace fgk
