@@ -125,6 +125,39 @@ def test_stream_k_needs_workspace(gpu):
     assert rc == -4 and "workspace" in _C.last_error()
 
 
+# Shapes with enough 256x256 tiles to take the direct-to-LDS kernel (first three), and neighbours that
+# miss one of its preconditions (K not a multiple of 64, N not a multiple of 8) and must take the
+# register-staged kernel instead; ragged M and N edges in both.
+LARGE_TILE_SHAPES = [(3857, 4104, 64), (4100, 4104, 256), (4096, 4096, 192), (4096, 4096, 72), (3900, 4100, 128)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", LARGE_TILE_SHAPES)
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_mm_addmm_large_tiles(gpu, M, N, K, dtype, b_col_major):
+    torch.manual_seed(M + K)
+    a = torch.randn(M, K, dtype=dtype, device=gpu)
+    b = _operand(K, N, dtype, gpu, b_col_major)
+    rows = torch.tensor([0, 1, 31, 32, 127, 128, 255, 256, 2047, 2048, M - 258, M - 257, M - 2, M - 1], device=gpu)
+    cols = torch.tensor([0, 7, 8, 63, 64, 255, 256, 257, N // 2, N - 257, N - 256, N - 9, N - 8, N - 1], device=gpu)
+    c = flag_gems.mm(a, b)
+    gems_assert_close(c[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
+    gems_assert_close(c[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
+    for bias in (torch.randn(N, dtype=dtype, device=gpu), torch.randn(M, N, dtype=dtype, device=gpu)):
+        d = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
+        brow = bias if bias.dim() == 1 else bias[rows]
+        bcol = bias[cols] if bias.dim() == 1 else bias[:, cols]
+        gems_assert_close(d[rows], O.addmm(brow, a[rows], b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+        gems_assert_close(d[:, cols], O.addmm(bcol, a, b[:, cols], alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+    # an output view whose row stride is not a multiple of 16 bytes (no vector stores possible)
+    wide = torch.empty(M, N + 3, dtype=dtype, device=gpu)
+    out = wide[:, :N]
+    with flag_gems.use_gems():
+        torch.mm(a, b, out=out)
+    gems_assert_close(out[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
+    gems_assert_close(out[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
+
+
 def test_mm_full_size_properties(gpu):
     """8192^3 bf16 (the benchmark shape): sampled rows against the oracle, plus linearity in A."""
     torch.manual_seed(3)
