@@ -62,6 +62,7 @@ struct AttnArgs {
   int use_async;      // take the asynchronous-tile kernel (head dims 64, 96, 128, 192, 256)
   int nw, nst;        // waves per workgroup and LDS stages of the asynchronous kernel
   int page_tab_entries;  // block-table entries the asynchronous kernel keeps in LDS (0: read them from global memory)
+  int use_fast;       // take the lean kernel (head dim 64/128, power-of-two pages, no ALiBi, no soft-cap)
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -740,9 +741,12 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
   return launch_async_lp<T, D, RB, NW, NST, false>(a, grid, st);
 }
 
+#include "attn_fast.h"
+
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
+  if (a.use_fast) return D == 64 ? launch_fast<T, 64>(a, grid, st) : launch_fast<T, 128>(a, grid, st);
   if (a.use_async) {
     if (a.nw == 8) {
       switch (D) {
@@ -804,11 +808,15 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   // Kernel variant.  Head dims 64/96/128/192/256 take the asynchronous-tile kernel with 4 waves and
   // two LDS stages (measured fastest; the 8-wave variants stay selectable for head dims <= 128);
   // everything else the register-staged kernel.
-  // FG_ATTN_KERNEL = "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
+  // FG_ATTN_KERNEL = "fast" | "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
   a.use_async = (p.D == 64 || p.D == 96 || p.D == 128 || p.D == 192 || p.D == 256) ? 1 : 0;
   a.nw = 4;
   a.nst = 2;
+  // The lean kernel needs every DMA instruction (1 KB = 4 rows of head dim 128, 8 of head dim 64) inside one page.
+  a.use_fast = ((p.D == 128 && a.page_shift >= 2) || (p.D == 64 && a.page_shift >= 3)) && p.alibi_slopes == nullptr &&
+               !(p.softcap > 0.f);
   if (const char* force = getenv("FG_ATTN_KERNEL")) {
+    a.use_fast = a.use_fast && force[0] == 'f';
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && p.D <= 128) {
       a.nw = force[1] == '8' ? 8 : 4;
