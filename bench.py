@@ -140,8 +140,8 @@ def main():
             O.softmax(sample, -1)
 
         # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
-        # read for a plain 512 MiB copy (profiles/softmax_c2_hbm_traffic.txt)
-        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=1073820700,
+        # read for a plain 512 MiB copy (profiles/hbm_traffic_softmax_mm_attention.txt)
+        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=1073780000,
                     workload="softmax dim=-1 [131072,2048] bf16, N(0,4) with 1% -inf (BASELINE.json configs[1])",
                     cpu=(cpu, 2 * 32768 * N * 2, "oracle softmax (torch CPU, fp64 upcast) on the first 32768 rows"))
 
@@ -191,6 +191,8 @@ def main():
             d = dict(run=run, work=work, bound=bound, dtype="bf16", workload=name,
                      cpu=(cpu, cw, "torch.mm on the host in fp32, first %d rows of A" % rows))
             d["post"] = lambda: {"schedule": {1: "data-parallel", 2: "stream-K"}.get(_gemm.last_schedule())}
+            if (M, N, K) == (8192, 8192, 8192) and not b_t and not bias:
+                d["traffic"] = 1770169000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
             return d
         return make
 
@@ -237,7 +239,7 @@ def main():
         def cpu():
             O.paged_attention(qc, kcc, vcc, [ls], [ls], btc, D ** -0.5, compute_dtype=torch.float32)
 
-        return dict(run=run, work=flops, bound="mfma", dtype="bf16",
+        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1824222000,
                     workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
                     cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
 
@@ -314,6 +316,26 @@ def main():
         return dict(run=run, work=2 * x.numel() * 2, bound="hbm", dtype="bf16",
                     workload="reference: torch copy of a [131072,2048] bf16 tensor (512 MiB read + 512 MiB written)", cpu=None)
 
+    def wl_mfma_ceiling(random_operands):
+        # calibration, not an operator: the rate the matrix cores sustain on nothing but MFMA 32x32x16
+        # bf16, with operand fragments of zeros or of N(0,1) values.  The chip is power-limited, so the
+        # second figure -- not the 2.5 PFLOP/s of the data sheet -- is what a real bf16 GEMM can approach.
+        import ctypes
+        from flaggems_amd import _C
+        src = (torch.randn(8 * 256 * 8, device=dev) if random_operands else torch.zeros(8 * 256 * 8, device=dev)).to(bf16)
+        blocks, iters = 1024, 4096
+        out = torch.empty(blocks * 256, device=dev)
+        flops = ctypes.c_double(0.0)
+
+        def run(i):
+            _C.check(_C.lib().fg_mfma_probe(src.data_ptr(), out.data_ptr(), blocks, iters, ctypes.byref(flops),
+                                            torch.cuda.current_stream().cuda_stream), "fg_mfma_probe")
+
+        run(0)
+        return dict(run=run, work=flops.value, bound="mfma", dtype="bf16",
+                    workload="calibration: MFMA-only loop, %s operands (sustained matrix-core rate under the power limit)"
+                    % ("N(0,1)" if random_operands else "all-zero"), cpu=None)
+
     workloads = {
         "softmax_c2": wl_softmax_c2,
         "fused_add_rms_norm_c1": wl_fused_add_rms_norm_c1,
@@ -323,6 +345,8 @@ def main():
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "decoder_layer_c5": wl_layer_c5,
+        "mfma_ceiling_random": lambda: wl_mfma_ceiling(True),
+        "mfma_ceiling_zeros": lambda: wl_mfma_ceiling(False),
         "copy_ref": wl_copy_ref,
     }
     if args.workload not in workloads:

@@ -72,6 +72,7 @@ _SIGNATURES = {
     "fg_last_error": (ctypes.c_char_p, []),
     "fg_abi_version": (c_int, []),
     "fg_device_info": (c_int, [c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
+    "fg_mfma_probe": (c_int, [c_vp, c_vp, c_int, c_int, ctypes.POINTER(ctypes.c_double), c_vp]),
     "fg_rms_norm": (c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_f32, c_int, c_vp]),
     "fg_fused_add_rms_norm": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_f32, c_int, c_vp]),
     "fg_softmax": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),

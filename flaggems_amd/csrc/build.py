@@ -26,6 +26,7 @@ SOURCES = [
     "gemm_streamk.hip",
     "gemm_dma.hip",
     "attn_varlen.hip",
+    "probe.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

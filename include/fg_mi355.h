@@ -45,6 +45,13 @@ int fg_abi_version(void);
  * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530). */
 int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
 
+/* Calibration of the matrix-core roofline (no counterpart in the reference; used by bench.py):
+ * every wave of `blocks` 256-thread workgroups issues 16 * iters MFMA 32x32x16 bf16 on operand
+ * fragments read once from `operands` (8 * 256 * 16 bytes).  `out` receives blocks * 256 floats;
+ * *flops the floating-point operations of the launch.  The sustained rate depends on the operand
+ * bits (power): random operands give the ceiling a real bf16 GEMM can approach on this part. */
+int fg_mfma_probe(const void* operands, float* out, int blocks, int iters, double* flops, void* stream);
+
 /* rms_norm forward.  y[m,:] = x[m,:] * rsqrt(mean(x[m,:]^2) + eps) * w, fp32 arithmetic,
  * one rounding on store; inv_rms[m] (fp32) is written when non-NULL; w may be NULL (= ones).
  * Replaces rms_norm_kernel, src/flag_gems/ops/rms_norm.py:15-51, and
