@@ -1,13 +1,13 @@
 // Paged varlen attention forward, lean variant of the asynchronous-tile kernel for the common case:
-// head dim 64 or 128, page size a power of two >= the keys one DMA instruction moves (8 / 4), no
-// ALiBi, no soft-cap.  Same work split, MFMA formulation, LDS layout and online softmax as
+// head dim 64 or 128, page size a power of two >= 16, at most 8192 keys per sequence, no ALiBi, no
+// soft-cap.  Same work split, MFMA formulation, LDS layout and online softmax as
 // attn_varlen_async_kernel (4 waves x 32 query rows, 64-key tiles, two LDS stages); what differs is
 // that nothing address-like is recomputed per tile on the vector ALU, which the general kernel
 // spends more time on than on the softmax itself:
-//   * One global_load_lds instruction moves 1 KB = KPI whole key rows, which lie in one page.  So
-//     the page id and the row base are wave-uniform: they are fetched with scalar loads one tile
-//     ahead and turned into a 64-bit scalar base; each lane adds a 32-bit offset fixed for the
-//     whole kernel (its row within the instruction and its swizzled chunk).
+//   * A wave moves 16 consecutive key rows of every tile, which lie in one page.  So the page id and
+//     the row base are wave-uniform: the ids of all tiles sit in two registers (a lane each), read
+//     once before the loop, and become a 64-bit scalar base; each lane adds a 32-bit offset fixed
+//     for the whole kernel (its row within the instruction and its swizzled chunk).
 //   * The tile loop is unrolled over the two LDS stages, so stage, sub-tile and k-step offsets of
 //     every fragment read are instruction immediates on top of 8 + 8 lane-constant registers.
 //   * Masking works on the raw scores with one compare and one select per element against a
@@ -114,27 +114,36 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_fast_kernel(AttnArgs a) {
     voff_k[j] = (uint32_t)(lane_key * (int)p.k_row_stride * 2 + c * 16);
     voff_v[j] = (uint32_t)(lane_key * (int)p.v_row_stride * 2 + c * 16);
   }
-  // page ids of the tile to be issued next (wave-uniform, scalar loads)
-  int page_next[IPW];
-  auto load_pages = [&](int nb) {
-#pragma unroll
-    for (int j = 0; j < IPW; ++j) {
-      const int key = nb * kBN + (wave_s * IPW + j) * KPI;
-      page_next[j] = btab[key >> page_shift];
-    }
-  };
-  // full tile: every key exists; scalar row bases
+  // A wave moves 16 consecutive key rows of every tile (IPW * KPI), which lie in one page (page size
+  // >= 16): one page id per wave and tile.  The ids of tiles n_min + l (pg_cache0) and n_min + 64 + l
+  // (pg_cache1) sit in lane l of two registers, loaded once, so that no load is left in the tile loop
+  // (it would be ordered behind the tile DMAs); the id of a tile is a v_readlane away.  The host routes
+  // key ranges of more than 128 tiles to the general kernel.
+  const int last_page = k_len > 0 ? (k_len - 1) >> page_shift : 0;
+  int pg_cache0, pg_cache1;
+  {
+    int pg0 = ((n_min + lane) * kBN + wave_s * (IPW * KPI)) >> page_shift;
+    int pg1 = ((n_min + 64 + lane) * kBN + wave_s * (IPW * KPI)) >> page_shift;
+    pg0 = pg0 < last_page ? pg0 : last_page;
+    pg1 = pg1 < last_page ? pg1 : last_page;
+    pg_cache0 = btab[pg0];
+    pg_cache1 = btab[pg1];
+  }
+  // full tile: every key exists; one scalar row base per tile and operand
   auto issue_full = [&](int nb, int stage) {
     char* kdst = lds + stage * STAGEB + wave_s * (IPW * 1024);
+    // (a caller whose max_seqlen_k understates seqused_k gets the page of tile 127 for later tiles: wrong
+    // numbers for a wrong argument, but always a page of this sequence)
+    const int tl = nb - n_min < 127 ? nb - n_min : 127;
+    const int64_t page = __builtin_amdgcn_readlane(tl < 64 ? pg_cache0 : pg_cache1, tl & 63);
+    const int key = nb * kBN + wave_s * (IPW * KPI);
+    const int slot = key & page_mask;
+    const char* kp = kbase + (page * p.k_page_stride + (int64_t)slot * p.k_row_stride) * 2;
+    const char* vp = vbase + (page * p.v_page_stride + (int64_t)slot * p.v_row_stride) * 2;
 #pragma unroll
     for (int j = 0; j < IPW; ++j) {
-      const int key = nb * kBN + (wave_s * IPW + j) * KPI;
-      const int64_t page = page_next[j];
-      const int slot = key & page_mask;
-      const char* kp = kbase + (page * p.k_page_stride + (int64_t)slot * p.k_row_stride) * 2;
-      const char* vp = vbase + (page * p.v_page_stride + (int64_t)slot * p.v_row_stride) * 2;
-      __builtin_amdgcn_global_load_lds(FG_GLBP(kp + voff_k[j]), FG_LDSP(kdst + j * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(FG_GLBP(vp + voff_v[j]), FG_LDSP(kdst + OPB + j * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(FG_GLBP(kp + (int64_t)j * KPI * p.k_row_stride * 2 + voff_k[j]), FG_LDSP(kdst + j * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(FG_GLBP(vp + (int64_t)j * KPI * p.v_row_stride * 2 + voff_v[j]), FG_LDSP(kdst + OPB + j * 1024), 16, 0, 0);
     }
   };
   // partial tile: keys past the end are clamped to the last one (their scores are masked)
@@ -154,7 +163,6 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_fast_kernel(AttnArgs a) {
   };
   auto issue_tile = [&](int nb, int stage) {
     if (nb * kBN + kBN <= k_len) {
-      load_pages(nb);
       issue_full(nb, stage);
     } else {
       issue_partial(nb, stage);

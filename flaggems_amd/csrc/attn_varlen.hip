@@ -812,8 +812,9 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.use_async = (p.D == 64 || p.D == 96 || p.D == 128 || p.D == 192 || p.D == 256) ? 1 : 0;
   a.nw = 4;
   a.nst = 2;
-  // The lean kernel needs every DMA instruction (1 KB = 4 rows of head dim 128, 8 of head dim 64) inside one page.
-  a.use_fast = ((p.D == 128 && a.page_shift >= 2) || (p.D == 64 && a.page_shift >= 3)) && p.alibi_slopes == nullptr &&
+  // The lean kernel needs the 16 key rows a wave moves per tile inside one page, and keeps the page ids of
+  // at most 128 tiles in registers.
+  a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.max_seqlen_k <= 128 * 64 && p.alibi_slopes == nullptr &&
                !(p.softcap > 0.f);
   if (const char* force = getenv("FG_ATTN_KERNEL")) {
     a.use_fast = a.use_fast && force[0] == 'f';
