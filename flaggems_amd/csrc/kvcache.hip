@@ -27,7 +27,16 @@ __global__ __launch_bounds__(256) void cache_scatter_kernel(const char* __restri
   const U* src = reinterpret_cast<const U*>(is_v ? value + tok * value_stride_b : key + tok * key_stride_b);
   U* dst = reinterpret_cast<U*>((is_v ? vc : kc) + blk * block_stride_b + off * row_bytes);
   const int64_t n = row_bytes / (int64_t)sizeof(U);
-  for (int64_t i = threadIdx.x & 63; i < n; i += 64) dst[i] = src[i];
+  // four pieces per lane in flight: the row is short, so the copy lives on memory-level parallelism
+  int64_t i = threadIdx.x & 63;
+  for (; i + 192 < n; i += 256) {
+    const U a = src[i], b = src[i + 64], c = src[i + 128], d = src[i + 192];
+    dst[i] = a;
+    dst[i + 64] = b;
+    dst[i + 128] = c;
+    dst[i + 192] = d;
+  }
+  for (; i < n; i += 64) dst[i] = src[i];
 }
 
 template <typename SLOT>

@@ -156,25 +156,29 @@ int rms_dispatch(const T* x, T* res, const T* w, T* y, float* inv_rms, int64_t M
   if (!vec_ok || packs > 1024 * 8) {
     hipLaunchKernelGGL((rms_looped_kernel<T, FUSED>), dim3((unsigned)M), dim3(256), 0, st, x, res, w, y, inv_rms, M,
                        N, xs, rs, ys, eps);
-  } else if (packs <= 64) {
-    // One pack per thread wherever a row fits 1024 threads: measured on MI355X this beats fewer
-    // threads holding several packs (16384 x 4096 bf16 fused: 84.8 us at 1 x 512 threads per row
-    // against 92.8 us at 4 x 128), the extra waves keeping more 16-byte requests in flight.
-    FG_ROWS(1, 64);
-  } else if (packs <= 128) {
-    FG_ROWS(1, 128);
-  } else if (packs <= 256) {
-    FG_ROWS(1, 256);
-  } else if (packs <= 512) {
-    FG_ROWS(1, 512);
-  } else if (packs <= 1024) {
-    FG_ROWS(1, 1024);
-  } else if (packs <= 2048) {
-    FG_ROWS(2, 1024);
-  } else if (packs <= 4096) {
-    FG_ROWS(4, 1024);
+  } else if (FUSED) {
+    // Two input streams: one pack per thread from each wherever a row fits 1024 threads.  Measured on
+    // MI355X this beats fewer threads holding several packs (16384 x 4096 bf16: 84.8 us at 1 x 512
+    // threads per row against 92.8 us at 4 x 128), the extra waves keeping more requests in flight.
+    if (packs <= 64) FG_ROWS(1, 64);
+    else if (packs <= 128) FG_ROWS(1, 128);
+    else if (packs <= 256) FG_ROWS(1, 256);
+    else if (packs <= 512) FG_ROWS(1, 512);
+    else if (packs <= 1024) FG_ROWS(1, 1024);
+    else if (packs <= 2048) FG_ROWS(2, 1024);
+    else if (packs <= 4096) FG_ROWS(4, 1024);
+    else FG_ROWS(8, 1024);
   } else {
-    FG_ROWS(8, 1024);
+    // One input stream: two packs per thread give the same two 16-byte requests in flight per thread
+    // (65536 x 4096 bf16: 171 us at 2 x 256 threads per row against 197 us at 1 x 512).
+    if (packs <= 64) FG_ROWS(1, 64);
+    else if (packs <= 128) FG_ROWS(2, 64);
+    else if (packs <= 256) FG_ROWS(2, 128);
+    else if (packs <= 512) FG_ROWS(2, 256);
+    else if (packs <= 1024) FG_ROWS(2, 512);
+    else if (packs <= 2048) FG_ROWS(2, 1024);
+    else if (packs <= 4096) FG_ROWS(4, 1024);
+    else FG_ROWS(8, 1024);
   }
 #undef FG_ROWS
   return fg_check_launch(FUSED ? "fused_add_rms_norm" : "rms_norm");
