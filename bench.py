@@ -243,6 +243,30 @@ def main():
                     workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
                     cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
 
+    def wl_decode():
+        # single-token queries over a paged cache (the decode side of configs[3]): a stream over K and V
+        B, S, Hq, Hk, D, bs = 64, 4096, 32, 8, 128, 16
+        torch.manual_seed(0)
+        nblk = B * (S // bs)
+        bt = torch.randperm(nblk, generator=torch.Generator().manual_seed(0)).int().view(B, -1).to(dev)
+        kc = torch.randn(nblk, bs, Hk, D, device=dev).to(bf16)
+        vc = torch.randn(nblk, bs, Hk, D, device=dev).to(bf16)
+        q = torch.randn(B, Hq, D, device=dev).to(bf16)
+        cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+        sk = torch.full((B,), S, dtype=torch.int32, device=dev)
+
+        def run(i):
+            flag_gems.flash_attn_varlen_func(q, kc, vc, 1, cu, S, seqused_k=sk, causal=True, block_table=bt)
+
+        qc, kcc, vcc, btc = q[:1].cpu(), kc.cpu(), vc.cpu(), bt[:1].cpu()
+
+        def cpu():
+            O.paged_attention(qc, kcc, vcc, [1], [S], btc, D ** -0.5, compute_dtype=torch.float32)
+
+        return dict(run=run, work=2 * B * S * Hk * D * 2 + 2 * B * Hq * D * 2, bound="hbm", dtype="bf16",
+                    workload="flash_attn_varlen_func decode: 64 seqs x 4096 keys, 1 query token each, 32q/8kv heads, D 128, page 16",
+                    cpu=(cpu, 2 * S * Hk * D * 2, "oracle paged attention (torch CPU fp32) on one sequence"))
+
     def wl_layer_c5():
         torch.manual_seed(0)
         Hd, H, D, F, bs, B, S = 4096, 32, 128, 11008, 16, 8, 2048
@@ -344,6 +368,7 @@ def main():
         "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
+        "flash_attn_decode": wl_decode,
         "decoder_layer_c5": wl_layer_c5,
         "mfma_ceiling_random": lambda: wl_mfma_ceiling(True),
         "mfma_ceiling_zeros": lambda: wl_mfma_ceiling(False),

@@ -65,6 +65,8 @@ class FgFlashParams(ctypes.Structure):
         ("softmax_scale", c_f32),
         ("softcap", c_f32),
         ("dtype", ctypes.c_int32),
+        ("workspace", c_vp),
+        ("workspace_bytes", c_i64),
     ]
 
 
@@ -98,6 +100,7 @@ _SIGNATURES = {
         [c_i64, c_i64, c_i64, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],
     ),
     "fg_flash_attn_varlen_fwd": (c_int, [ctypes.POINTER(FgFlashParams), c_vp]),
+    "fg_flash_attn_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(FgFlashParams), c_int]),
 }
 
 _lib = None

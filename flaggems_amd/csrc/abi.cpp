@@ -24,7 +24,7 @@ int fg_check_launch(const char* what) {
 
 extern "C" const char* fg_last_error(void) { return g_err; }
 
-extern "C" int fg_abi_version(void) { return 1; }
+extern "C" int fg_abi_version(void) { return 2; }
 
 extern "C" int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch) {
   hipDeviceProp_t p;

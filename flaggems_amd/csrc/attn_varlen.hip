@@ -26,6 +26,7 @@
 // K/V tiles of 64 keys are gathered page by page (block_table -> page -> row), 16 bytes per lane,
 // zero-filled past the sequence end so stale cache contents can never reach the accumulators.
 // V is transposed on its way into LDS (8x8 register transposes with v_perm_b32).
+#include <stdint.h>
 #include <stdlib.h>
 #include "fg_common.h"
 
@@ -742,6 +743,7 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
 }
 
 #include "attn_fast.h"
+#include "attn_decode.h"
 
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
@@ -775,6 +777,62 @@ int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
+namespace {
+int decode_num_cu() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  return n;
+}
+// Decides whether the single-token kernel takes these parameters and, if so, how the key ranges are cut.
+// Without a large enough workspace the ranges are not split beyond what the kernel itself requires.
+bool decode_setup(const FgFlashParams& p, DecodeArgs* d) {
+  if (p.max_seqlen_q != 1 || !(p.D == 64 || p.D == 128) || p.alibi_slopes != nullptr || p.softcap > 0.f) return false;
+  if (p.window_left >= 0 && p.window_left < p.max_seqlen_k) return false;
+  if (p.Hk <= 0 || p.Hq % p.Hk != 0 || p.Hq / p.Hk > 32) return false;
+  int shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == p.page_size) shift = sft;
+  if (shift < 4) return false;
+  if (const char* force = getenv("FG_ATTN_KERNEL")) {
+    if (force[0] != 'd') return false;
+  }
+  int splits = 1, tps = 4;
+  decode_plan(p, shift, decode_num_cu(), &splits, &tps);
+  if (splits > 1 && (p.workspace == nullptr || (size_t)p.workspace_bytes < decode_workspace_bytes(p, splits) ||
+                     !fg_aligned(p.workspace, 16))) {
+    // unsplit, if one range can hold the longest sequence
+    const int64_t tiles = fg_cdiv(p.max_seqlen_k > 0 ? p.max_seqlen_k : 1, kDecTile);
+    if (tiles * kDecTile > 4096) return false;
+    splits = 1;
+    tps = (int)((tiles + 3) / 4 * 4);
+  }
+  d->p = p;
+  d->scale_log2 = p.softmax_scale * 1.4426950408889634f;
+  d->page_shift = shift;
+  d->group = p.Hq / p.Hk;
+  d->splits = splits;
+  d->tiles_per_split = tps;
+  d->part_o = splits > 1 ? (float*)p.workspace : nullptr;
+  d->part_ml = splits > 1 ? (float*)p.workspace + (size_t)splits * p.batch * p.Hq * p.D : nullptr;
+  return true;
+}
+}  // namespace
+
+extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int device) {
+  if (pp == nullptr) return 0;
+  FgFlashParams p = *pp;
+  if (p.batch <= 0 || p.total_q <= 0) return 0;
+  // ask as if an unlimited workspace were offered
+  static char dummy_ws[16] __attribute__((aligned(16)));
+  p.workspace = dummy_ws;
+  p.workspace_bytes = INT64_MAX;
+  (void)device;
+  DecodeArgs d;
+  if (!decode_setup(p, &d)) return 0;
+  return decode_workspace_bytes(p, d.splits);
+}
+
 extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   FG_REQUIRE(pp != nullptr, FG_ERR_INVALID, "flash_attn_varlen_fwd: null params");
   const FgFlashParams& p = *pp;
@@ -798,6 +856,14 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
              "flash_attn_varlen_fwd: out rows must be 8-byte aligned");
   FG_REQUIRE(p.batch < 65536 && p.Hq < 65536, FG_ERR_UNSUPPORTED, "flash_attn_varlen_fwd: batch/heads exceed the grid");
 
+  hipStream_t st = (hipStream_t)stream;
+  {
+    DecodeArgs d;
+    if (decode_setup(p, &d)) {
+      if (p.dtype == FG_F16) return p.D == 64 ? launch_decode<f16_t, 64>(d, st) : launch_decode<f16_t, 128>(d, st);
+      return p.D == 64 ? launch_decode<bf16_t, 64>(d, st) : launch_decode<bf16_t, 128>(d, st);
+    }
+  }
   AttnArgs a;
   a.p = p;
   const int ratio = p.Hq / p.Hk;
@@ -844,7 +910,6 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
   a.cap_out_log2 = p.softcap * log2e;
   dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
-  hipStream_t st = (hipStream_t)stream;
   if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
   return attn_dispatch<bf16_t>(a, grid, st);
 }

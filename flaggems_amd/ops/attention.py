@@ -112,6 +112,12 @@ def mha_varlan_fwd(
             p.softmax_scale = float(softmax_scale)
             p.softcap = float(softcap)
             p.dtype = _C.dtype_id(q.dtype)
+            # single-token queries: scratch for the partial results of split key ranges (the reference's
+            # out_accum / softmax_lse_accum); the library says how much it wants, zero for prefill shapes
+            ws_bytes = _C.lib().fg_flash_attn_workspace_bytes(ctypes.byref(p), q.device.index or 0)
+            if ws_bytes > 0:
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+                p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes
             rc = _C.lib().fg_flash_attn_varlen_fwd(ctypes.byref(p), _C.current_stream(q.device))
             _C.check(rc, "fg_flash_attn_varlen_fwd")
         philox_args = torch.empty((2,), dtype=torch.int64, device=q.device)

@@ -161,6 +161,8 @@ typedef struct FgFlashParams {
   float softmax_scale;
   float softcap;            /* 0 = off */
   int32_t dtype;            /* FG_F16 or FG_BF16 */
+  void* workspace;          /* device scratch for split key ranges, may be NULL (see fg_flash_attn_workspace_bytes) */
+  int64_t workspace_bytes;
 } FgFlashParams;
 
 /* Forward of variable-length attention over a paged KV cache (FA2 semantics: bottom-right
@@ -169,6 +171,13 @@ typedef struct FgFlashParams {
  * half of mha_varlan_fwd (src/flag_gems/ops/flash_api.py:230-569,
  * lib/flash_attn_varlen_func.cpp:14-481). */
 int fg_flash_attn_varlen_fwd(const FgFlashParams* p /*host*/, void* stream);
+
+/* Scratch the forward would like for these parameters: non-zero only for single-token queries
+ * (max_seqlen_q == 1) whose key ranges are worth splitting over several workgroups; the partial
+ * results of the ranges go there (the role of the reference's out_accum / softmax_lse_accum,
+ * src/flag_gems/ops/flash_api.py:752-800).  The forward never needs it: without it (NULL or too
+ * small) it runs unsplit.  Uninitialised memory is fine; one stream at a time. */
+size_t fg_flash_attn_workspace_bytes(const FgFlashParams* p /*host*/, int device);
 
 #ifdef __cplusplus
 }

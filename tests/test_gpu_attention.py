@@ -85,6 +85,41 @@ def test_flash_attn_varlen_edges(gpu):
     check(gpu, [(1, 17), (1, 1000), (1, 1), (1, 4096)], 32, 8, 128, 16, 2048, torch.bfloat16)
 
 
+# Single-token queries: the streaming kernel with split key ranges (head dim 64/128, pages >= 16) and the
+# cases it must hand back to the general kernels (small pages, left window, ALiBi, other head dims).
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hk,D,block_size", [(32, 8, 128, 16), (8, 8, 64, 32), (16, 2, 64, 16), (32, 32, 128, 64),
+                                                 (4, 1, 128, 256), (8, 2, 128, 8), (8, 2, 96, 16)])
+def test_flash_attn_decode(gpu, dtype, Hq, Hk, D, block_size):
+    # ragged lengths around tile (32), page and range (4096) boundaries, an empty sequence, a long one that
+    # needs several key ranges by itself
+    check(gpu, [(1, 1), (1, 17), (1, 32), (1, 33), (1, 0), (1, 1000), (1, 4095), (1, 4097)], Hq, Hk, D, block_size, 1024, dtype)
+    check(gpu, [(1, 9001)], Hq, Hk, D, block_size, 1024, dtype)           # one sequence: split for parallelism
+    check(gpu, [(1, 100 + 37 * i) for i in range(70)], Hq, Hk, D, block_size, 1024, dtype)  # many short ones
+
+
+def test_flash_attn_decode_variants(gpu):
+    lens = [(1, 300), (1, 5000), (1, 64)]
+    check(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16, causal=False)
+    check(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16, window=(128, 0))     # left window: general kernel
+    check(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16, window=(-1, 5))
+    check(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16, alibi=True)          # ALiBi: general kernel
+    check(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16, softcap=30.0)
+    # a sequence with no query at all among single-token ones
+    check(gpu, [(1, 200), (0, 50), (1, 700)], 8, 2, 128, 16, 256, torch.float16)
+    # without a workspace the library must still be right (unsplit, or the prefill kernels for long ranges)
+    from flaggems_amd import _C
+    q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, [(1, 3000), (1, 6000)], 32, 8, 128, 16, 1024, torch.bfloat16)
+    orig = _C.lib().fg_flash_attn_workspace_bytes
+    try:
+        _C.lib().fg_flash_attn_workspace_bytes = lambda *a: 0
+        out = flag_gems.flash_attn_varlen_func(q, kc, vc, 1, cu, max(klens), seqused_k=sk, causal=True, block_table=bt)
+    finally:
+        _C.lib().fg_flash_attn_workspace_bytes = orig
+    ref = O.paged_attention(q, kc, vc, qlens, klens, bt, 128 ** -0.5, compute_dtype=torch.float32)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
+
+
 def test_flash_attn_varlen_out_argument_and_views(gpu):
     q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, [(40, 90), (17, 17)], 8, 2, 128, 16, 128, torch.bfloat16)
     out = torch.full_like(q, 7.0)

@@ -96,7 +96,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), f"{name} declared in include/fg_mi355.h but not exported"
     assert declared == set(_C.exported_symbols()), "python binding and header disagree"
-    assert _C.lib().fg_abi_version() == 1
+    assert _C.lib().fg_abi_version() == 2
 
 
 def test_struct_mirror_matches_header_order():
