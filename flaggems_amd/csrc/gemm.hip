@@ -18,7 +18,8 @@ int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace,
 
 // implemented in gemm_dma.hip
 bool dma_supported(const GemmArgs& g, int elem_bytes);
-int dma_launch(const GemmArgs& g, int dtype, hipStream_t st);
+void dma_pick_tile(int64_t M, int64_t N, int num_cu, int* bm, int* bn);
+int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st);
 
 int num_cus(int device) {
   static std::mutex mu;
@@ -95,13 +96,19 @@ template <typename T>
 int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
   constexpr int BK = kRowBytes / sizeof(T);
   if constexpr (sizeof(T) == 2) {
+    // Aligned operands with K a multiple of 64 take the direct-to-LDS kernel, on the tile size that fills
+    // the machine best, once there is at least half a round of the smallest tile.
+    if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr &&
+        fg_cdiv(g.M, 128) * fg_cdiv(g.N, 128) >= (int64_t)num_cu) {
+      int bm = 256, bn = 256;
+      dma_pick_tile(g.M, g.N, num_cu, &bm, &bn);
+      set_tiles(g, bm, bn, BK);
+      return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, st);
+    }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
     if (amode != LOAD_GEN && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
       set_tiles(g, 256, 256, BK);
-      // aligned operands with K a multiple of 64 take the direct-to-LDS kernel
-      if (dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr)
-        return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, st);
       return launch_dp_modes<T, 256, 256>(g, amode, bmode, st);
     }
   }

@@ -1,7 +1,9 @@
 // Direct-to-LDS MFMA GEMM for gfx950, 16-bit inputs: C[M,N] = alpha * A[M,K].B[K,N] + beta * bias.
 //
-// The large-matrix kernel.  A 256x256 output tile per workgroup, 4 waves in a 2x2 grid, each wave a
-// 128x128 sub-tile held as 4x4 MFMA 32x32 accumulators (256 accumulator registers per lane).
+// The kernel for aligned 16-bit problems.  A BM x BN output tile per workgroup (256x256, 256x128 or
+// 128x128, chosen on the host by how well the tile count fills the machine), 4 waves in a 2x2 grid,
+// each wave a (BM/2) x (BN/2) sub-tile held as MFMA 32x32 accumulators (256 accumulator registers per
+// lane for the largest tile).  The description below uses the 256x256 numbers.
 //
 // Data movement.  Each K step covers 64 elements = one full 128-byte cache line per tile row.  The
 // operand tiles go from global memory straight into LDS with global_load_lds_dwordx4: no staging
@@ -44,11 +46,9 @@
 
 namespace fgk {
 
-constexpr int kDmaRowB = 128;                 // bytes of K per stage per A row
-constexpr int kDmaOpB = 256 * kDmaRowB;       // one operand, one stage: 32 KB
-constexpr int kDmaStageB = 2 * kDmaOpB;
-constexpr int kDmaLdsBytes = 2 * kDmaStageB;  // 128 KB
+constexpr int kDmaRowB = 128;   // bytes of K per stage per A row
 constexpr int kDmaBK = 64;
+constexpr int dma_lds_bytes(int bm, int bn) { return 2 * (bm + bn) * kDmaRowB; }  // two stages of (A tile + B tile)
 
 #define FGK_LDSP(p) ((__attribute__((address_space(3))) void*)(p))
 #define FGK_GLBP(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -79,42 +79,55 @@ __device__ __forceinline__ void swap_halves2(unsigned& x0, unsigned& y0, unsigne
                : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
 }
 
-template <typename T, bool B_KC>
-__global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs g) {
+template <typename T, bool B_KC, int BM, int BN>
+__global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
   static_assert(sizeof(T) == 2, "16-bit element types");
   typedef typename Mfma<T>::Frag Frag;
+  constexpr int TM = BM / 64, TN = BN / 64;        // MFMA sub-tiles per wave
+  constexpr int WTM = BM / 2, WTN = BN / 2;        // wave tile
+  constexpr int A_OPB = BM * kDmaRowB;             // A tile, one stage
+  constexpr int B_OPB = BN * kDmaRowB;             // B tile, one stage (64 k-rows of BN*2 bytes when N-contiguous)
+  constexpr int STAGEB = A_OPB + B_OPB;
+  constexpr int NA = BM / 32, NB = BN / 32;        // DMA instructions per wave, operand and stage
+  constexpr int NDMA = NA + NB, HALF = NDMA / 2;
+  constexpr int NMF = TM * TN, NRD = TM + TN;      // MFMAs and fragment reads per sub-step
+  constexpr int RBB = BN * 2;                      // N-contiguous B: bytes per k-row of the tile
+  constexpr int CPRB = RBB / 16, RPI = 1024 / RBB; // ... chunks per k-row, k-rows per DMA instruction
+  static_assert(HALF <= NMF && NRD <= NMF, "one LDS read or DMA per MFMA");
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
-  const int row0 = tm * 256, col0 = tn * 256;
+  const int row0 = tm * BM, col0 = tn * BN;
   const int M = (int)g.M, N = (int)g.N;
   const int nk = (int)(g.K / kDmaBK);
 
-  // ---- DMA source addresses.  Wave w issues instructions j = 0..7 per operand and stage; the LDS
-  // destination of instruction j is base + (j/4)*4096 (through M0) + (j%4)*1024 (immediate).  The
-  // hardware adds the immediate to the global address as well, so it is subtracted here.
-  const char* a_src[8];
-  const char* b_src[8];
+  // ---- DMA source addresses.  Wave w issues NA (NB) instructions per stage for A (B); instruction j
+  // lands at operand base + (w*NA + j) * 1024, split into a part that goes through M0 ((j/4)*4096)
+  // and an instruction immediate ((j%4)*1024).  The hardware adds the immediate to the global address
+  // as well, so it is subtracted here.
+  const char* a_src[NA];
+  const char* b_src[NB];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    {
-      const int r = (wave * 8 + j) * 8 + (lane >> 3);
-      const int c = (lane & 7) ^ ((r >> 1) & 7);
-      int ra = row0 + r;
-      ra = ra < M ? ra : M - 1;
-      a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024;
-    }
+  for (int j = 0; j < NA; ++j) {
+    const int r = (wave * NA + j) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ ((r >> 1) & 7);
+    int ra = row0 + r;
+    ra = ra < M ? ra : M - 1;
+    a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024;
+  }
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
     if constexpr (B_KC) {
-      const int r = (wave * 8 + j) * 8 + (lane >> 3);
+      const int r = (wave * NB + j) * 8 + (lane >> 3);
       const int c = (lane & 7) ^ ((r >> 1) & 7);
       int rb = col0 + r;
       rb = rb < N ? rb : N - 1;
       b_src[j] = (const char*)g.B + ((int64_t)rb * g.sbn + c * 8) * 2 - (j & 3) * 1024;
     } else {
-      const int k = (wave * 8 + j) * 2 + (lane >> 5);
-      const int c = (lane & 31) ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1));
+      const int k = (wave * NB + j) * RPI + lane / CPRB;
+      const int c = (lane % CPRB) ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1));
       int cb = col0 + c * 8;
       cb = cb + 8 <= N ? cb : N - 8;
       b_src[j] = (const char*)g.B + ((int64_t)k * g.sbk + cb) * 2 - (j & 3) * 1024;
@@ -122,81 +135,92 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs g) {
   }
   const int64_t b_step = B_KC ? (int64_t)kDmaRowB : g.sbk * (int64_t)(kDmaBK * 2);  // bytes per K step
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-  char* const dma_base = lds + wave_s * 8192;
+  char* const dma_a = lds + wave_s * (NA * 1024);
+  char* const dma_b = lds + A_OPB + wave_s * (NB * 1024);
   auto issue = [&](int kb, auto jc) {
-    constexpr int j = decltype(jc)::value;  // 0..15: the A instructions, then the B instructions
-    constexpr int jj = j & 7;
-    char* l = dma_base + (kb & 1) * kDmaStageB + (j < 8 ? 0 : kDmaOpB) + (jj >> 2) * 4096;
-    const char* gp = j < 8 ? a_src[jj] + (int64_t)kb * kDmaRowB : b_src[jj] + (int64_t)kb * b_step;
+    constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
+    constexpr bool IS_A = j < NA;
+    constexpr int jj = IS_A ? j : j - NA;
+    char* l = (IS_A ? dma_a : dma_b) + (kb & 1) * STAGEB + (jj >> 2) * 4096;
+    const char* gp = IS_A ? a_src[jj] + (int64_t)kb * kDmaRowB : b_src[jj] + (int64_t)kb * b_step;
     __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
   };
 
   // ---- fragment addresses
   const int fr = lane & 31, fh = lane >> 5;
   const int q = (fr >> 1) & 7;  // sub-tile rows start at multiples of 32, so (row >> 1) & 7 depends on fr only
-  const int a_lane = (wm * 128 + fr) * kDmaRowB;
+  const int a_lane = (wm * WTM + fr) * kDmaRowB;
   int pos[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) pos[s] = ((2 * s + fh) ^ q) * 16;
-  int b_lane = 0;          // K-contiguous B: like A
-  uint32_t b_tr[4] = {0, 0, 0, 0};  // N-contiguous B: per sub-tile j, the lane's address within a stage
+  int b_lane = 0;      // K-contiguous B: like A
+  uint32_t b_tr[TN];   // N-contiguous B: per sub-tile j, the lane's address within a stage
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b_tr[j] = 0;
   if constexpr (B_KC) {
-    b_lane = kDmaOpB + (wn * 128 + fr) * kDmaRowB;
+    b_lane = A_OPB + (wn * WTN + fr) * kDmaRowB;
   } else {
+    // lane -> k-row 8*hh + m (+ 16*sub-step, +4 for the second read), columns 16*b4 + 4*(lane&3) .. +3 of sub-tile j
     const int m = (lane & 15) >> 2, hh = lane >> 5, b4 = (lane >> 4) & 1, b1 = (lane & 3) >> 1;
     const int krow = 8 * hh + m;
+    const int sw = (m << 2) | (hh << 1);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int chunk = wn * 16 + ((j ^ m) << 2) + (((b4 ^ hh) << 1) | b1);
-      b_tr[j] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + kDmaOpB + krow * 512 + chunk * 16 +
+    for (int j = 0; j < TN; ++j) {
+      const int chunk = (wn * (WTN / 8) + j * 4 + ((b4 << 1) | b1)) ^ sw;
+      b_tr[j] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + A_OPB + krow * RBB + chunk * 16 +
                 (lane & 1) * 8;
     }
   }
 
-  f32x16 acc[4][4];
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  Frag fa[2][4];
+  Frag fa[2][TM];
   u32x4 fb[2][4];
-  // read x of fragment set `set` for sub-step S of `stage`: x < 4 -> A sub-tile x, else B sub-tile x-4
+  // read x of fragment set `set` for sub-step S of `stage`: x < TM -> A sub-tile x, else B sub-tile x-TM
   auto read_one = [&](int stage, auto sc, auto xc, int set) {
     constexpr int S = decltype(sc)::value;
     constexpr int x = decltype(xc)::value;
-    const int sb = (stage & 1) * kDmaStageB;
-    if constexpr (x < 4) {
+    const int sb = (stage & 1) * STAGEB;
+    if constexpr (x < TM) {
       fa[set][x] = *reinterpret_cast<const Frag*>(lds + sb + a_lane + x * 32 * kDmaRowB + pos[S]);
     } else if constexpr (B_KC) {
-      fb[set][x - 4] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + (x - 4) * 32 * kDmaRowB + pos[S]);
+      fb[set][x - TM] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + (x - TM) * 32 * kDmaRowB + pos[S]);
     } else {
-      const u32x2 lo = lds_read_tr16_b64<(16 * S) * 512>(b_tr[x - 4] + sb);
-      const u32x2 hi = lds_read_tr16_b64<(16 * S + 4) * 512>(b_tr[x - 4] + sb);
-      fb[set][x - 4] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      const u32x2 lo = lds_read_tr16_b64<(16 * S) * RBB>(b_tr[x - TM] + sb);
+      const u32x2 hi = lds_read_tr16_b64<(16 * S + 4) * RBB>(b_tr[x - TM] + sb);
+      fb[set][x - TM] = u32x4{lo[0], lo[1], hi[0], hi[1]};
     }
   };
   auto wait_reads = [&](int set) {
     if constexpr (B_KC) FGK_WAIT_LGKM0();
     else lds_wait_tied(fb[set]);
   };
+  if constexpr (!B_KC && TN < 4) {
+    // the tied wait names four registers per set; give the unused ones a value
+#pragma unroll
+    for (int j = TN; j < 4; ++j) fb[0][j] = fb[1][j] = u32x4{0u, 0u, 0u, 0u};
+  }
 
   // ---- prologue: stage 0, and the head of stage 1 (the part sub-step 3 of the step before would issue)
-  static_for<0, 16>([&](auto jc) { issue(0, jc); });
+  static_for<0, NDMA>([&](auto jc) { issue(0, jc); });
   if (nk > 1) {
-    static_for<0, 8>([&](auto jc) { issue(1, jc); });
-    FGK_WAIT_VM(8);
+    static_for<0, HALF>([&](auto jc) { issue(1, jc); });
+    FGK_WAIT_VM(HALF);
   } else {
     FGK_WAIT_VM(0);
   }
   __builtin_amdgcn_s_barrier();
-  static_for<0, 8>([&](auto xc) { read_one(0, IntC<0>{}, xc, 0); });
+  static_for<0, NRD>([&](auto xc) { read_one(0, IntC<0>{}, xc, 0); });
   wait_reads(0);
   __builtin_amdgcn_sched_barrier(0);
 
-  // One K step.  REFILL_TAIL: sub-steps 0 issue the second half of the DMAs of stage kb+1;
+  // One K step.  REFILL_TAIL: sub-step 0 issues the second half of the DMAs of stage kb+1;
   // REFILL_HEAD: sub-step 3 issues the first half of the DMAs of stage kb+2.
   auto k_step = [&](int kb, auto tail_c, auto head_c) {
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
@@ -204,16 +228,16 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs g) {
     static_for<0, 4>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
       constexpr int cur = s & 1, nxt = cur ^ 1;
-      static_for<0, 16>([&](auto xc) {
+      static_for<0, NMF>([&](auto xc) {
         constexpr int x = decltype(xc)::value;
-        constexpr int i = x >> 2, j = x & 3;
+        constexpr int i = x / TN, j = x % TN;
         acc[i][j] = Mfma<T>::mma(__builtin_bit_cast(Frag, fb[cur][j]), fa[cur][i], acc[i][j]);
-        if constexpr (x < 8) {
+        if constexpr (x < NRD) {
           if constexpr (s < 3) read_one(kb, IntC<s + 1>{}, xc, nxt);
           else read_one(kb + 1, IntC<0>{}, xc, nxt);
         }
-        if constexpr (s == 3 && REFILL_HEAD && x < 8) issue(kb + 2, IntC<x>{});
-        if constexpr (s == 0 && REFILL_TAIL && x < 8) issue(kb + 1, IntC<8 + x>{});
+        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + 2, IntC<x>{});
+        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + 1, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       if constexpr (s == 2) {
@@ -242,11 +266,11 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmArgs g) {
   const bool scale = alpha != 1.0f;
   const int lr = lane & 31, lh = lane >> 5;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int64_t r = row0 + wm * 128 + i * 32 + lr;
+  for (int i = 0; i < TM; ++i) {
+    const int64_t r = row0 + wm * WTM + i * 32 + lr;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int cbase = col0 + wn * 128 + j * 32;
+    for (int j = 0; j < TN; ++j) {
+      const int cbase = col0 + wn * WTN + j * 32;
       // element e of this lane: row r, column cbase + (e/4)*8 + lh*4 + e%4
       if (bias != nullptr) {
 #pragma unroll

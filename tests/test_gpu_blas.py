@@ -158,6 +158,35 @@ def test_mm_addmm_large_tiles(gpu, M, N, K, dtype, b_col_major):
     gems_assert_close(out[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
 
 
+# The direct-to-LDS kernel exists for three tile sizes; the library picks by how the tile count fills the
+# machine.  Each is forced in turn on ragged shapes (edge tiles in M and N, one to several K steps) and, with
+# no forcing, on shapes whose automatic choice is the 128x128 and the 256x128 tile.
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tile", ["256x256", "256x128", "128x128", None])
+@pytest.mark.parametrize("M,N,K", [(1024, 4096, 128), (1100, 4104, 64), (2040, 4104, 256), (1537, 2824, 192)])
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_mm_addmm_tile_sizes(gpu, monkeypatch, M, N, K, dtype, tile, b_col_major):
+    if tile is None:
+        monkeypatch.delenv("FG_GEMM_TILE", raising=False)
+    else:
+        monkeypatch.setenv("FG_GEMM_TILE", tile)
+    torch.manual_seed(M + K)
+    a = torch.randn(M, K, dtype=dtype, device=gpu)
+    b = _operand(K, N, dtype, gpu, b_col_major)
+    rows = torch.tensor([0, 1, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, M // 2, M - 130, M - 129, M - 2, M - 1], device=gpu)
+    cols = torch.tensor([0, 7, 8, 63, 64, 127, 128, 255, 256, 257, N // 2, N - 137, N - 129, N - 9, N - 8, N - 1], device=gpu)
+    c = flag_gems.mm(a, b)
+    gems_assert_close(c[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
+    gems_assert_close(c[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
+    bias = torch.randn(N, dtype=dtype, device=gpu)
+    d = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
+    gems_assert_close(d[rows], O.addmm(bias, a[rows], b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+    gems_assert_close(d[:, cols], O.addmm(bias[cols], a, b[:, cols], alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+    # every tile size accumulates each output element over K in the same order: identical bits
+    monkeypatch.setenv("FG_GEMM_TILE", "256x256")
+    assert torch.equal(flag_gems.mm(a, b), c)
+
+
 def test_mm_full_size_properties(gpu):
     """8192^3 bf16 (the benchmark shape): sampled rows against the oracle, plus linearity in A."""
     torch.manual_seed(3)
