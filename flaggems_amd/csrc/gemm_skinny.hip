@@ -24,7 +24,8 @@
 //     columns n0 + 16*c + slot.
 #include <atomic>
 #include <stdlib.h>
-#include "gemm_tile.h"
+#include <mutex>
+#include "gemm_dma.h"
 
 namespace fgk {
 
@@ -109,8 +110,11 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int c = 0; c < 8; ++c) acc[c] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
-    u32x4 bv[8], bn[8];
-    u32x4 av, an;
+    // a ring of kDepth k-steps in flight per wave: a wave's share is only a handful of steps, so the
+    // depth of the ring decides how quickly the stream of B reaches full bandwidth
+    constexpr int kDepth = 4;
+    u32x4 bv[kDepth][8];
+    u32x4 av[kDepth];
     auto load_step = [&](int ks, u32x4 (&bd)[8], u32x4& ad) {
       const int k0 = ks * kStepK;
       const int ka = k0 + grp * 8;
@@ -151,14 +155,17 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
         acc[c] = Mfma16<T>::mma(__builtin_bit_cast(Frag, o), af, acc[c]);
       }
     };
-    if (my0 < my1) {
-      load_step(my0, bv, av);
-      for (int ks = my0; ks < my1; ks += 2) {
-        if (ks + 1 < my1) load_step(ks + 1, bn, an);
-        compute(bv, av);
-        if (ks + 1 < my1) {
-          if (ks + 2 < my1) load_step(ks + 2, bv, av);
-          compute(bn, an);
+    const int nmine = my1 - my0;
+#pragma unroll
+    for (int p = 0; p < kDepth - 1; ++p)
+      if (p < nmine) load_step(my0 + p, bv[p], av[p]);
+    for (int i = 0; i < nmine; i += kDepth) {
+#pragma unroll
+      for (int p = 0; p < kDepth; ++p) {
+        if (i + p < nmine) {
+          if (i + p + kDepth - 1 < nmine)
+            load_step(my0 + i + p + kDepth - 1, bv[(p + kDepth - 1) % kDepth], av[(p + kDepth - 1) % kDepth]);
+          compute(bv[p], av[p]);
         }
       }
     }
@@ -201,11 +208,25 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
         finish = true;  // the loads below bypass the non-coherent caches (device-coherent loads)
 #pragma unroll
         for (int j = 0; j < kEPT; ++j) sum[j] = 0.f;
-        for (int w2 = w_first; w2 <= w_last; ++w2) {
-          const float* src =
-              a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * kTileElems;
+        // contributors in groups of kGroup: all loads of a group are issued before the first add, so a
+        // group costs one memory round trip; the adds keep workgroup order
+        constexpr int kGroup = 8;
+        for (int wb = w_first; wb <= w_last; wb += kGroup) {
+          float part[kGroup][kEPT];
 #pragma unroll
-          for (int j = 0; j < kEPT; ++j) sum[j] += ld_coherent(src + tid + kBlock * j);
+          for (int q = 0; q < kGroup; ++q) {
+            const int w2 = wb + q <= w_last ? wb + q : w_last;
+            const float* src =
+                a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * kTileElems;
+#pragma unroll
+            for (int j = 0; j < kEPT; ++j) part[q][j] = ld_coherent(src + tid + kBlock * j);
+          }
+#pragma unroll
+          for (int q = 0; q < kGroup; ++q)
+            if (wb + q <= w_last) {
+#pragma unroll
+              for (int j = 0; j < kEPT; ++j) sum[j] += part[q][j];
+            }
         }
         if (tid == 0) __hip_atomic_store(a.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -232,6 +253,188 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
   }
 }
 
+// ---- K-contiguous B (B = W^T with W [N, K]: the layout of a linear layer's weight) -------------
+//
+// Read straight into MFMA fragments, this layout gives every load instruction 16 rows x 64 bytes: half
+// cache lines, and only as many bytes in flight as registers can hold.  Here the rows go to LDS by
+// asynchronous copies (global_load_lds) instead, 8 rows x 128 bytes per instruction, into a private
+// ring of kcRing slots per wave, issued kcRing-1 steps ahead of their use; fragments are read back
+// from LDS (the 16-byte pieces of a row are permuted by the row number on the way in, so that the
+// sixteen lanes of a fragment read hit different banks).  The output tile is 16 rows x 16 columns:
+// with that few columns a workgroup's range usually covers whole tiles (N = 4096 gives exactly one
+// tile per CU of a 256-CU part) and there is nothing to fix up between workgroups; split tiles use
+// the same ticket scheme as above.  Requires K % 64 == 0.
+constexpr int kcTileN = 16, kcStepK = 64, kcRing = 8;
+constexpr int kcSlotB = kcTileN * kcStepK * 2;            // bytes of one ring slot
+constexpr int kcLdsBytes = kWaves * kcRing * kcSlotB;     // 128 KB
+constexpr int kcTileElems = 16 * kcTileN;
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
+  typedef typename Mfma16<T>::Frag Frag;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  __shared__ float red[kWaves][kcTileElems];
+  __shared__ unsigned ticket_s;
+  const GemmArgs& g = a.g;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, grp = lane >> 4;
+  const int w = blockIdx.x;
+  const int M = (int)g.M, N = (int)g.N;
+  const char* A = (const char*)g.A;
+  const char* B = (const char*)g.B;
+  char* const ring = lds + __builtin_amdgcn_readfirstlane(wave) * (kcRing * kcSlotB);
+  // fragment of MFMA h: row m of the slot, 16-byte piece 4h + grp, stored at position piece ^ (row & 7)
+  int rd[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) rd[h] = m * 128 + (((4 * h + grp) ^ (m & 7)) << 4);
+  const int arow = m < M ? m : M - 1;  // rows beyond M are computed on a copy of the last row and never stored
+
+  const int64_t u_begin = range_begin(a.per, a.rem, w);
+  const int64_t u_end = range_begin(a.per, a.rem, w + 1);
+  int64_t u = u_begin;
+  while (u < u_end) {
+    const int tile = (int)(u / a.ksteps);
+    const int64_t tile_begin = (int64_t)tile * a.ksteps;
+    const int64_t tile_end = tile_begin + a.ksteps;
+    const int ks0 = (int)(u - tile_begin);
+    const int ks1 = (int)((u_end < tile_end ? u_end : tile_end) - tile_begin);
+    const int n0 = tile * kcTileN;
+
+    const int nsteps = ks1 - ks0;
+    const int share = (nsteps + kWaves - 1) / kWaves;
+    const int my0 = ks0 + wave * share;
+    const int my1 = (my0 + share < ks1) ? my0 + share : ks1;
+    const int nmine = my1 - my0;
+
+    f32x4v acc = f32x4v{0.f, 0.f, 0.f, 0.f};
+    if (nmine > 0) {
+      // copy instruction i of a step: slot rows 8i + lane/8, the lane's piece chosen so that it lands permuted
+      const char* bsrc[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int r = 8 * i + (lane >> 3);
+        const int c = (lane & 7) ^ (r & 7);
+        int n = n0 + r;
+        n = n < N ? n : N - 1;
+        bsrc[i] = B + ((int64_t)n * g.sbn + c * 8) * 2 - i * 1024;  // the instruction offset moves both addresses
+      }
+      const char* asrc[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) asrc[h] = A + ((int64_t)arow * g.sam + (4 * h + grp) * 8) * 2;
+      u32x4 af[kcRing][2];
+      // Every step issues the same four memory operations, so the count to wait for is a constant; steps
+      // past the end of the share re-read the last one (served by the caches) and are not computed.
+      auto issue = [&](int step, auto pc) {
+        constexpr int p = decltype(pc)::value;
+        const int sidx = step < nmine ? step : nmine - 1;
+        const int64_t koff = (int64_t)(my0 + sidx) * (kcStepK * 2);
+        char* slot = ring + p * kcSlotB;
+        __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[0] + koff), FGK_LDSP(slot), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[1] + koff), FGK_LDSP(slot), 16, 1024, 0);
+        af[p][0] = *reinterpret_cast<const u32x4*>(asrc[0] + koff);
+        af[p][1] = *reinterpret_cast<const u32x4*>(asrc[1] + koff);
+      };
+      auto compute = [&](auto pc) {
+        constexpr int p = decltype(pc)::value;
+        const char* slot = ring + p * kcSlotB;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const Frag bf = *reinterpret_cast<const Frag*>(slot + rd[h]);
+          acc = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, af[p][h]), acc);
+        }
+      };
+      static_for<0, kcRing - 1>([&](auto pc) {
+        issue(decltype(pc)::value, pc);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // whole rounds of the ring: issue, wait for the step issued kcRing-1 steps ago, compute -- no branches,
+      // so the number of operations in flight at every wait is known
+      int i = 0;
+      for (; i + kcRing <= nmine; i += kcRing) {
+        static_for<0, kcRing>([&](auto pc) {
+          constexpr int p = decltype(pc)::value;
+          issue(i + p + kcRing - 1, IntC<(p + kcRing - 1) % kcRing>{});
+          FGK_WAIT_VM(4 * (kcRing - 1));
+          compute(pc);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
+      // the rest (fewer than kcRing steps) is already on its way
+      FGK_WAIT_VM(0);
+      const int rest = nmine - i;
+      static_for<0, kcRing - 1>([&](auto pc) {
+        if (decltype(pc)::value < rest) compute(pc);
+      });
+    }
+
+    // ---- add the 8 waves' accumulators through LDS; thread t < 256 ends up with element t ----------
+    __syncthreads();  // red[] of the previous segment is no longer read
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][i * 64 + lane] = acc[i];
+    __syncthreads();
+    float sum = 0.f;
+    if (tid < kcTileElems) {
+#pragma unroll
+      for (int v = 0; v < kWaves; ++v) sum += red[v][tid];
+    }
+
+    bool finish = (ks0 == 0 && ks1 == a.ksteps);
+    if (!finish) {
+      float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * kcTileElems;
+      if (tid < kcTileElems) st_coherent(slot + tid, sum);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      const int w_first = worker_of(a.per, a.rem, tile_begin);
+      const int w_last = worker_of(a.per, a.rem, tile_end - 1);
+      if (tid == 0)
+        ticket_s = __hip_atomic_fetch_add(a.tickets + w_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (ticket_s == (unsigned)(w_last - w_first)) {
+        finish = true;
+        sum = 0.f;
+        if (tid < kcTileElems) {
+          for (int w2 = w_first; w2 <= w_last; ++w2) {
+            const float* src =
+                a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * kcTileElems;
+            sum += ld_coherent(src + tid);
+          }
+        }
+        if (tid == 0) __hip_atomic_store(a.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (finish && tid < kcTileElems) {
+      T* C = (T*)g.C;
+      const T* bias = (const T*)g.bias;
+      const int el = tid & 63, i = tid >> 6;
+      const int em = el & 15, eg = el >> 4;
+      const int n = n0 + 4 * eg + i;
+      if (em < M && n < N) {
+        float v = sum;
+        if (bias != nullptr) v = v * g.alpha + (float)bias[(int64_t)em * g.sim + (int64_t)n * g.sin] * g.beta;
+        else if (g.alpha != 1.0f) v = v * g.alpha;
+        C[(int64_t)em * g.scm + (int64_t)n * g.scn] = (T)v;
+      }
+    }
+    u = tile_begin + ks1;
+  }
+}
+
+template <typename T>
+int launch_kc(const SkinnyArgs& a, hipStream_t st) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto kern = gemm_skinny_kc_kernel<T>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kcLdsBytes);
+  });
+  if (attr_err != hipSuccess) {
+    fg_set_error("gemm(stream-K, skinny): cannot reserve %d bytes of LDS: %s", kcLdsBytes, hipGetErrorString(attr_err));
+    return FG_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)a.workers), dim3(kBlock), kcLdsBytes, st, a);
+  return fg_check_launch("gemm(stream-K, skinny)");
+}
+
 }  // namespace
 
 // 0: not a case for this kernel; 1: B row-major (N contiguous); 2: B = W^T (K contiguous)
@@ -256,8 +459,10 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   FG_REQUIRE(fg_aligned(workspace, 256), FG_ERR_WORKSPACE, "gemm(stream-K): workspace must be 256-byte aligned");
   SkinnyArgs a;
   a.g = g;
-  a.tiles_n = (int)fg_cdiv(g.N, kTileN);
-  a.ksteps = (int)fg_cdiv(g.K, kStepK);
+  // K-contiguous B with K a multiple of 64: the kernel that stages B through LDS, on 16-column tiles
+  const bool kc = b_kind == 2 && g.K % kcStepK == 0 && getenv("FG_SKINNY_NO_LDS") == nullptr;
+  a.tiles_n = (int)fg_cdiv(g.N, kc ? kcTileN : kTileN);
+  a.ksteps = (int)fg_cdiv(g.K, kc ? kcStepK : kStepK);
   const int64_t units = (int64_t)a.tiles_n * a.ksteps;
   if (num_cu > kMaxWorkers) num_cu = kMaxWorkers;
   a.workers = (int)(units < num_cu ? units : num_cu);
@@ -266,6 +471,7 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   char* ws = (char*)workspace;
   a.tickets = (unsigned*)(ws + kTicketOffset);
   a.partials = (float*)(ws + kPartialOffset);
+  if (kc) return dtype == FG_BF16 ? launch_kc<bf16_t>(a, st) : launch_kc<f16_t>(a, st);
   dim3 grid((unsigned)a.workers), block(kBlock);
   if (dtype == FG_BF16) {
     if (b_kind == 1) hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, true>), grid, block, 0, st, a);

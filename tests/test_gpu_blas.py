@@ -87,6 +87,10 @@ SK_CASES = [
     # (M, N, K, schedule)               skinny stream-K kernel (M <= 16) ...
     (16, 4096, 14336, _C.SCHED_AUTO), (1, 4096, 4096, _C.SCHED_AUTO), (7, 1000, 2048, _C.SCHED_AUTO),
     (16, 152, 1024, _C.SCHED_AUTO), (3, 11008, 4096, _C.SCHED_STREAM_K), (13, 128, 40960, _C.SCHED_AUTO),
+    # ... few columns (every tile split between many workgroups), ragged N with several tiles per workgroup,
+    # K a multiple of 8 but not of 64, K an odd multiple of 64
+    (16, 24, 2048, _C.SCHED_AUTO), (2, 8200, 1024, _C.SCHED_AUTO), (5, 1000, 1032, _C.SCHED_AUTO),
+    (9, 4096, 1088, _C.SCHED_AUTO),
     # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
     (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
