@@ -58,6 +58,11 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_fast_kernel(AttnArgs a) {
   const int k_len = p.seqused_k[b];
   const int block_row0 = m_block * a.rows_per_block;
   if (block_row0 >= q_len) return;
+  // As the second pass behind the head-pair kernel: only blocks that kernel has marked (its blocks hold two
+  // of these in the row direction).
+  if (a.redo_rows != 0 &&
+      a.redo_flags[((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * a.redo_grid_x + (m_block >> 1)] == 0)
+    return;
 
   const int waves_per_head = 4 / a.hpb;
   const int head = hgroup * a.hpb + wave / waves_per_head;

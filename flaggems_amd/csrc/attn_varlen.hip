@@ -64,6 +64,10 @@ struct AttnArgs {
   int nw, nst;        // waves per workgroup and LDS stages of the asynchronous kernel
   int page_tab_entries;  // block-table entries the asynchronous kernel keeps in LDS (0: read them from global memory)
   int use_fast;       // take the lean kernel (head dim 64/128, power-of-two pages, no ALiBi, no soft-cap)
+  int use_pair;       // take the head-pair kernel (lean kernel's conditions, head dim 128, even GQA ratio)
+  int* redo_flags;    // head-pair kernel: one flag per workgroup, set when the block has to be redone by the lean kernel
+  int redo_rows;      // lean kernel as the second pass: query rows per flagged block (0: ordinary launch)
+  int redo_grid_x;    // ... and the first grid dimension of the flagging launch
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -743,11 +747,13 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
 }
 
 #include "attn_fast.h"
+#include "attn_pair.h"
 #include "attn_decode.h"
 
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
+  if (a.use_pair) return launch_pair<T, 128>(a, grid, st);
   if (a.use_fast) return D == 64 ? launch_fast<T, 64>(a, grid, st) : launch_fast<T, 128>(a, grid, st);
   if (a.use_async) {
     if (a.nw == 8) {
@@ -817,6 +823,24 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d) {
   d->part_ml = splits > 1 ? (float*)p.workspace + (size_t)splits * p.batch * p.Hq * p.D : nullptr;
   return true;
 }
+// Head-pair kernel: applicable?  If so, its block shape and the size of its flag array.
+bool pair_plan(const FgFlashParams& p, int* hpb, int* rows, size_t* flag_bytes) {
+  if (p.Hk <= 0 || p.Hq % p.Hk != 0) return false;
+  const int ratio = p.Hq / p.Hk;
+  int page_shift = -1;
+  for (int sft = 4; sft < 31; ++sft)
+    if ((1 << sft) == p.page_size) page_shift = sft;
+  if (p.D != 128 || ratio % 2 != 0 || page_shift < 0 || p.max_seqlen_k > 128 * 64 || p.max_seqlen_q < 2 ||
+      p.alibi_slopes != nullptr || p.softcap > 0.f)
+    return false;
+  // Measured on MI355X the lean kernel is still ahead (see the header of attn_pair.h): opt-in for now.
+  const char* force = getenv("FG_ATTN_KERNEL");
+  if (force == nullptr || force[0] != 'p') return false;
+  *hpb = ratio % 4 == 0 ? 4 : 2;
+  *rows = (8 / *hpb) * 32;
+  *flag_bytes = (size_t)fg_cdiv(p.max_seqlen_q, *rows) * (size_t)p.batch * (size_t)(p.Hq / *hpb) * sizeof(int);
+  return true;
+}
 }  // namespace
 
 extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int device) {
@@ -829,8 +853,11 @@ extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int dev
   p.workspace_bytes = INT64_MAX;
   (void)device;
   DecodeArgs d;
-  if (!decode_setup(p, &d)) return 0;
-  return decode_workspace_bytes(p, d.splits);
+  if (decode_setup(p, &d)) return decode_workspace_bytes(p, d.splits);
+  int hpb = 0, rows = 0;
+  size_t flag_bytes = 0;
+  if (pair_plan(p, &hpb, &rows, &flag_bytes)) return flag_bytes;
+  return 0;
 }
 
 extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
@@ -882,8 +909,12 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   // at most 128 tiles in registers.
   a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.max_seqlen_k <= 128 * 64 && p.alibi_slopes == nullptr &&
                !(p.softcap > 0.f);
+  a.use_pair = 0;
+  a.redo_flags = nullptr;
+  a.redo_rows = 0;
+  a.redo_grid_x = 0;
   if (const char* force = getenv("FG_ATTN_KERNEL")) {
-    a.use_fast = a.use_fast && force[0] == 'f';
+    a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p');
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && p.D <= 128) {
       a.nw = force[1] == '8' ? 8 : 4;
@@ -910,6 +941,25 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
   a.cap_out_log2 = p.softcap * log2e;
   dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
+  {
+    // The head-pair kernel first, where it applies and the caller brought room for its flags; the lean kernel
+    // then runs as a second pass over the blocks it marked (normally none).
+    int hpb = 0, rows = 0;
+    size_t flag_bytes = 0;
+    if (a.use_fast && pair_plan(p, &hpb, &rows, &flag_bytes) && hpb == a.hpb && rows == 2 * a.rows_per_block &&
+        p.workspace != nullptr && p.workspace_bytes >= (int64_t)flag_bytes && fg_aligned(p.workspace, 4)) {
+      AttnArgs ap = a;
+      ap.use_pair = 1;
+      ap.rows_per_block = rows;
+      ap.redo_flags = (int*)p.workspace;
+      dim3 grid_p((unsigned)fg_cdiv(p.max_seqlen_q, rows), (unsigned)p.batch, (unsigned)(p.Hq / hpb));
+      const int rc = p.dtype == FG_F16 ? attn_dispatch<f16_t>(ap, grid_p, st) : attn_dispatch<bf16_t>(ap, grid_p, st);
+      if (rc != FG_OK) return rc;
+      a.redo_flags = (int*)p.workspace;
+      a.redo_rows = rows;
+      a.redo_grid_x = (int)grid_p.x;
+    }
+  }
   if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
   return attn_dispatch<bf16_t>(a, grid, st);
 }

@@ -142,7 +142,9 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
     char* l = (IS_A ? dma_a : dma_b) + (kb & 1) * STAGEB + (jj >> 2) * 4096;
-    const char* gp = IS_A ? a_src[jj] + (int64_t)kb * kDmaRowB : b_src[jj] + (int64_t)kb * b_step;
+    const char* gp;
+    if constexpr (IS_A) gp = a_src[jj] + (int64_t)kb * kDmaRowB;
+    else gp = b_src[jj] + (int64_t)kb * b_step;
     __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
   };
 

@@ -85,6 +85,48 @@ def test_flash_attn_varlen_edges(gpu):
     check(gpu, [(1, 17), (1, 1000), (1, 1), (1, 4096)], 32, 8, 128, 16, 2048, torch.bfloat16)
 
 
+# The head-pair kernel (two heads of a KV group per wave, software-pipelined tiles; opt-in through the
+# environment): same oracle, same tolerances.  The last case feeds scores that keep growing along the keys, so
+# that rows leave the exponent headroom above their fixed softmax reference and the blocks are handed to the
+# lean kernel by the second pass.
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hk", [(8, 2), (4, 2), (6, 3)])
+def test_flash_attn_head_pair_kernel(gpu, monkeypatch, dtype, Hq, Hk):
+    monkeypatch.setenv("FG_ATTN_KERNEL", "pair")
+    check(gpu, [(1, 1328), (5, 18), (129, 463), (70, 70)], Hq, Hk, 128, 16, 512, dtype)
+    check(gpu, [(200, 200), (64, 64), (65, 65), (300, 1000)], Hq, Hk, 128, 32, 1024, dtype)
+    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=False)
+    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=True, window=(50, 0))
+    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=False, window=(20, 30))
+    check(gpu, [(300, 200), (130, 130), (64, 5)], Hq, Hk, 128, 16, 512, dtype)
+    check(gpu, [(2000, 2000), (100, 3000)], Hq, Hk, 128, 16, 1024, dtype)
+
+
+@pytest.mark.parametrize("dtype,grow", [(torch.bfloat16, 0.02), (torch.float16, 0.004), (torch.bfloat16, 0.05)])
+def test_flash_attn_head_pair_second_pass(gpu, monkeypatch, dtype, grow):
+    monkeypatch.setenv("FG_ATTN_KERNEL", "pair")
+    dev, Hq, Hk, D, bs, nblk = gpu, 8, 2, 128, 16, 512
+    qlens, klens = [300, 64], [300, 700]
+    torch.manual_seed(5)
+    q = torch.ones(sum(qlens), Hq, D, dtype=dtype, device=dev)
+    kc = torch.zeros(nblk, bs, Hk, D, dtype=dtype, device=dev)
+    vc = torch.randn(nblk, bs, Hk, D, dtype=dtype, device=dev)
+    pages = (max(klens) + bs - 1) // bs
+    bt = torch.randperm(nblk)[:2 * pages].reshape(2, pages).to(torch.int32).to(dev)
+    for b in range(2):
+        for j in range(pages):
+            pos = (j * bs + torch.arange(bs, device=dev)).float()
+            kc[bt[b, j].long()] = (pos * grow).to(dtype)[:, None, None].expand(bs, Hk, D)
+    cu = torch.tensor([0] + qlens, dtype=torch.int32, device=dev).cumsum(0, dtype=torch.int32)
+    sk = torch.tensor(klens, dtype=torch.int32, device=dev)
+    scale = D ** -0.5
+    out, lse = flag_gems.ops.flash_attn_varlen_func(q, kc, vc, max(qlens), cu, max(klens), seqused_k=sk, softmax_scale=scale,
+                                                    causal=True, block_table=bt, return_softmax_lse=True)
+    ref, rlse = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, compute_dtype=torch.float32, return_lse=True)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
+    torch.testing.assert_close(lse.cpu(), rlse, atol=1e-2, rtol=1e-3)
+
+
 # Single-token queries: the streaming kernel with split key ranges (head dim 64/128, pages >= 16) and the
 # cases it must hand back to the general kernels (small pages, left window, ALiBi, other head dims).
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
