@@ -192,7 +192,7 @@ def main():
                      cpu=(cpu, cw, "torch.mm on the host in fp32, first %d rows of A" % rows))
             d["post"] = lambda: {"schedule": {1: "data-parallel", 2: "stream-K"}.get(_gemm.last_schedule())}
             if (M, N, K) == (8192, 8192, 8192) and not b_t and not bias:
-                d["traffic"] = 1770169000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
+                d["traffic"] = 1764196000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
             return d
         return make
 
@@ -239,7 +239,7 @@ def main():
         def cpu():
             O.paged_attention(qc, kcc, vcc, [ls], [ls], btc, D ** -0.5, compute_dtype=torch.float32)
 
-        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1824222000,
+        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1835372000,
                     workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
                     cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
 
@@ -366,6 +366,8 @@ def main():
         "mm_c3a_8192": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B row-major (configs[2]a)"),
         "mm_c3a_8192_nt": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B = W^T column-major (configs[2]a, weight layout)", b_t=True),
         "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),
+        "mm_c3b_skinny_nt": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, B = W^T of a [N, K] weight, stream-K",
+                                  b_t=True, bound="hbm"),
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "flash_attn_decode": wl_decode,
