@@ -163,7 +163,32 @@ def supported_dtype(dtype):
 
 
 def current_stream(device):
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on `device` (the launches of this library go there)."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device):
+    """Context that makes `device` current for the library call.  Switching devices costs several
+    microseconds per call, as much as a small kernel runs; when the device is current already (the
+    usual case) nothing is switched."""
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 _dev_info = {}

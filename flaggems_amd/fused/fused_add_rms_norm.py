@@ -27,7 +27,7 @@ def fused_add_rms_norm(x, residual, normalized_shape, weight, eps=1e-5):
     weight = weight.contiguous()
     if M == 0 or N == 0:
         return x, residual
-    with torch.cuda.device(x.device):
+    with _C.device_guard(x.device):
         rc = _C.lib().fg_fused_add_rms_norm(
             x.data_ptr(), residual.data_ptr(), weight.data_ptr(), M, N, N, N, eps,
             _C.dtype_id(x.dtype), _C.current_stream(x.device),

@@ -33,7 +33,7 @@ def reshape_and_cache_flash(
     assert slot_mapping.stride(0) == 1 or num_tokens <= 1, "slot_mapping must be contiguous"
     if num_tokens == 0:
         return
-    with torch.cuda.device(key.device):
+    with _C.device_guard(key.device):
         rc = _C.lib().fg_reshape_and_cache_flash(
             key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
             slot_mapping.data_ptr(), 1 if slot_mapping.dtype == torch.int64 else 0,

@@ -70,7 +70,7 @@ def apply_rotary_pos_emb(
 
     if n_tokens > 0 and head_dim > 0:
         I3 = _C.I64x3
-        with torch.cuda.device(q.device):
+        with _C.device_guard(q.device):
             rc = _C.lib().fg_rope(
                 q_embed.data_ptr(), k_embed.data_ptr(), q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                 position_ids.data_ptr() if position_ids is not None else None,

@@ -42,7 +42,7 @@ def _launch(A, B, out):
     rows, cols, _ = vo
     if rows * cols == 0:
         return out
-    with torch.cuda.device(out.device):
+    with _C.device_guard(out.device):
         rc = _C.lib().fg_silu_and_mul(
             A.data_ptr(), B.data_ptr(), out.data_ptr(), rows, cols, va[2], vb[2], vo[2],
             _C.dtype_id(out.dtype), _C.current_stream(out.device),

@@ -52,7 +52,7 @@ def gemm(a, b, bias, c, alpha=1.0, beta=0.0, schedule=_C.SCHED_AUTO):
     N = b.shape[1]
     lib = _C.lib()
     dev = c.device
-    with torch.cuda.device(dev):
+    with _C.device_guard(dev):
         stream = _C.current_stream(dev)
         ab = _C.dtype_id(a.dtype)
         ws_bytes = lib.fg_gemm_workspace_bytes(M, N, K, ab, schedule, dev.index)

@@ -84,7 +84,7 @@ def mha_varlan_fwd(
     else:
         alibi_batch_stride = 0
 
-    with torch.cuda.device(q.device):
+    with _C.device_guard(q.device):
         if out is None:
             out = torch.empty_like(q, dtype=v.dtype)
         lse = torch.empty((num_heads, total_q), dtype=torch.float, device=q.device)

@@ -46,7 +46,7 @@ def rms_norm(x, normalized_shape, weight=None, eps=1e-5):
     y = torch.empty_like(x)
     if M == 0 or N == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _C.device_guard(x.device):
         rc = _C.lib().fg_rms_norm(
             x.data_ptr(), w.data_ptr() if w is not None else None, y.data_ptr(), None,
             M, N, N, N, eps, _C.dtype_id(x.dtype), _C.current_stream(x.device),

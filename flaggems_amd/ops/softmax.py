@@ -26,7 +26,7 @@ def softmax(self, dim, half_to_float=False):
     if self.numel() == 0:
         return out
     K = self.numel() // M // N
-    with torch.cuda.device(self.device):
+    with _C.device_guard(self.device):
         rc = _C.lib().fg_softmax(
             self.data_ptr(), out.data_ptr(), M, N, K, _C.dtype_id(self.dtype), _C.dtype_id(dtype),
             _C.current_stream(self.device),
