@@ -20,6 +20,7 @@ int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace,
 bool dma_supported(const GemmArgs& g, int elem_bytes);
 void dma_pick_tile(int64_t M, int64_t N, int num_cu, int* bm, int* bn);
 int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st);
+int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st);
 
 int num_cus(int device) {
   static std::mutex mu;
@@ -97,9 +98,8 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
   constexpr int BK = kRowBytes / sizeof(T);
   if constexpr (sizeof(T) == 2) {
     // Aligned operands with K a multiple of 64 take the direct-to-LDS kernel, on the tile size that fills
-    // the machine best, once there is at least half a round of the smallest tile.
-    if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr &&
-        fg_cdiv(g.M, 128) * fg_cdiv(g.N, 128) >= (int64_t)num_cu) {
+    // the machine best (even a lone 128x128 workgroup per CU runs twice as fast as the register-staged kernel).
+    if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr) {
       int bm = 256, bn = 256;
       dma_pick_tile(g.M, g.N, num_cu, &bm, &bn);
       set_tiles(g, bm, bn, BK);
@@ -197,11 +197,13 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
         if (schedule == FG_SCHED_STREAM_K) {
           use_streamk = true;
         } else {
-          // auto: stream-K when the tiles cannot fill half the machine and K is deep enough to hand
-          // every workgroup at least four K steps; fuller grids run data-parallel.
+          // auto: stream-K when the tiles cannot fill the machine and K is deep enough to hand every workgroup
+          // at least four K steps; fuller grids run data-parallel.  The direct-to-LDS main loop is worth
+          // sharing up to 0.9 waves of tiles, the register-staged one up to half a wave.
           const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
           const int64_t iters = fg_cdiv(K, 64);
-          use_streamk = tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;
+          const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && getenv("FG_GEMM_NO_DMA") == nullptr;
+          use_streamk = (dma ? tiles * 10 <= (int64_t)cu * 9 : tiles * 2 <= (int64_t)cu) && tiles * iters >= 4 * (int64_t)cu;
         }
       }
     }
@@ -217,6 +219,8 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
   }
   if (use_streamk) {
     if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;
+    if (amode != LOAD_GEN && dma_supported(g, eb) && getenv("FG_GEMM_NO_DMA") == nullptr)
+      return dma_streamk_launch(g, ab_dtype, workspace, workspace_bytes, cu, st);
     return streamk_launch(g, ab_dtype, amode, bmode, workspace, workspace_bytes, cu, st);
   }
   switch (ab_dtype) {

@@ -79,8 +79,66 @@ __device__ __forceinline__ void swap_halves2(unsigned& x0, unsigned& y0, unsigne
                : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
 }
 
-template <typename T, bool B_KC, int BM, int BN>
-__global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
+// Epilogue of one tile (the host guarantees: C rows 16-byte aligned with unit column stride, N a multiple
+// of 8, bias -- if any -- with unit column stride and 8-byte aligned rows).  acc is in the layout the
+// main loop leaves: operands swapped, so a lane owns 4 consecutive output columns per register group.
+template <typename T, int BM, int BN>
+__device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int tn, f32x16 (&acc)[BM / 64][BN / 64]) {
+  constexpr int TM = BM / 64, TN = BN / 64, WTM = BM / 2, WTN = BN / 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int row0 = tm * BM, col0 = tn * BN;
+  const int M = (int)g.M, N = (int)g.N;
+  T* C = (T*)g.C;
+  const T* bias = (const T*)g.bias;
+  const float alpha = g.alpha, beta = g.beta;
+  const bool scale = alpha != 1.0f;
+  const int lr = lane & 31, lh = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int64_t r = row0 + wm * WTM + i * 32 + lr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int cbase = col0 + wn * WTN + j * 32;
+      // element e of this lane: row r, column cbase + (e/4)*8 + lh*4 + e%4
+      if (bias != nullptr) {
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          const int c = cbase + gq * 8 + lh * 4;
+          typedef T T4 __attribute__((ext_vector_type(4)));
+          T4 t = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+#pragma unroll
+          for (int t4 = 0; t4 < 4; ++t4)
+            acc[i][j][gq * 4 + t4] = acc[i][j][gq * 4 + t4] * alpha + (float)t[t4] * beta;
+        }
+      } else if (scale) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] *= alpha;
+      }
+      unsigned pk[8];
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        typedef T T2 __attribute__((ext_vector_type(2)));
+        const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
+        pk[d] = __builtin_bit_cast(unsigned, t);
+      }
+#pragma unroll
+      for (int gp = 0; gp < 2; ++gp) {
+        // register groups 2gp (X) and 2gp+1 (Y): after X.upper <-> Y.lower the lower half-wave owns
+        // the 8 columns of group 2gp, the upper half-wave those of group 2gp+1
+        unsigned x0 = pk[4 * gp], x1 = pk[4 * gp + 1], y0 = pk[4 * gp + 2], y1 = pk[4 * gp + 3];
+        swap_halves2(x0, y0, x1, y1);
+        const int c = cbase + (2 * gp + lh) * 8;
+        if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
+      }
+    }
+  }
+}
+
+// Main loop over the K steps [kb0, kb0 + nk) of tile (tm, tn); `finish` receives the accumulators.
+template <typename T, bool B_KC, int BM, int BN, typename F>
+__device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish) {
   static_assert(sizeof(T) == 2, "16-bit element types");
   typedef typename Mfma<T>::Frag Frag;
   constexpr int TM = BM / 64, TN = BN / 64;        // MFMA sub-tiles per wave
@@ -94,14 +152,11 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
   constexpr int RBB = BN * 2;                      // N-contiguous B: bytes per k-row of the tile
   constexpr int CPRB = RBB / 16, RPI = 1024 / RBB; // ... chunks per k-row, k-rows per DMA instruction
   static_assert(HALF <= NMF && NRD <= NMF, "one LDS read or DMA per MFMA");
-  extern __shared__ __attribute__((aligned(16))) char lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  int tm, tn;
-  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
   const int row0 = tm * BM, col0 = tn * BN;
   const int M = (int)g.M, N = (int)g.N;
-  const int nk = (int)(g.K / kDmaBK);
+  const int64_t b_step = B_KC ? (int64_t)kDmaRowB : g.sbk * (int64_t)(kDmaBK * 2);  // bytes per K step
 
   // ---- DMA source addresses.  Wave w issues NA (NB) instructions per stage for A (B); instruction j
   // lands at operand base + (w*NA + j) * 1024, split into a part that goes through M0 ((j/4)*4096)
@@ -115,7 +170,7 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
     const int c = (lane & 7) ^ ((r >> 1) & 7);
     int ra = row0 + r;
     ra = ra < M ? ra : M - 1;
-    a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024;
+    a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024 + (int64_t)kb0 * kDmaRowB;
   }
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
@@ -124,16 +179,15 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
       const int c = (lane & 7) ^ ((r >> 1) & 7);
       int rb = col0 + r;
       rb = rb < N ? rb : N - 1;
-      b_src[j] = (const char*)g.B + ((int64_t)rb * g.sbn + c * 8) * 2 - (j & 3) * 1024;
+      b_src[j] = (const char*)g.B + ((int64_t)rb * g.sbn + c * 8) * 2 - (j & 3) * 1024 + kb0 * b_step;
     } else {
       const int k = (wave * NB + j) * RPI + lane / CPRB;
       const int c = (lane % CPRB) ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1));
       int cb = col0 + c * 8;
       cb = cb + 8 <= N ? cb : N - 8;
-      b_src[j] = (const char*)g.B + ((int64_t)k * g.sbk + cb) * 2 - (j & 3) * 1024;
+      b_src[j] = (const char*)g.B + ((int64_t)k * g.sbk + cb) * 2 - (j & 3) * 1024 + kb0 * b_step;
     }
   }
-  const int64_t b_step = B_KC ? (int64_t)kDmaRowB : g.sbk * (int64_t)(kDmaBK * 2);  // bytes per K step
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   char* const dma_a = lds + wave_s * (NA * 1024);
   char* const dma_b = lds + A_OPB + wave_s * (NB * 1024);
@@ -260,52 +314,87 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
   }
   k_step(kb, IntC<0>{}, IntC<0>{});
 
-  // ---- epilogue (the host guarantees: C rows 16-byte aligned with unit column stride, N a multiple
-  // of 8, bias -- if any -- with unit column stride and 8-byte aligned rows)
-  T* C = (T*)g.C;
-  const T* bias = (const T*)g.bias;
-  const float alpha = g.alpha, beta = g.beta;
-  const bool scale = alpha != 1.0f;
-  const int lr = lane & 31, lh = lane >> 5;
+  finish(acc);
+}
+
+template <typename T, bool B_KC, int BM, int BN>
+__global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  int tm, tn;
+  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
+  dma_tile_mainloop<T, B_KC, BM, BN>(g, lds, tm, tn, 0, (int)(g.K / kDmaBK),
+                                     [&](f32x16 (&acc)[BM / 64][BN / 64]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); });
+}
+
+// Stream-K over 128x128 tiles with the main loop above: the (tile, K step) units, tile-major, are dealt
+// in equal contiguous ranges to the workgroups; a tile split between workgroups is finished by whichever
+// of them arrives last (ticket per tile, fp32 partial tiles in the workspace, added in workgroup order so
+// the result does not depend on who finishes).  Same scheme as gemm_streamk_kernel in gemm_tile.h.
+template <typename T, bool B_KC>
+__global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
+  constexpr int BM = 128, BN = 128, TM = 2, TN = 2;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  __shared__ unsigned ticket_s;
+  const int w = blockIdx.x, tid = threadIdx.x;
+  const int64_t u_begin = sk_begin(g.sk_per, g.sk_rem, w);
+  const int64_t u_end = sk_begin(g.sk_per, g.sk_rem, w + 1);
+  int64_t u = u_begin;
+  while (u < u_end) {
+    const int tile = (int)(u / g.iters_per_tile);
+    const int64_t tile_begin = (int64_t)tile * g.iters_per_tile;
+    const int64_t tile_end = tile_begin + g.iters_per_tile;
+    const int it0 = (int)(u - tile_begin);
+    const int it1 = (int)((u_end < tile_end ? u_end : tile_end) - tile_begin);
+    int tm, tn;
+    tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
+    __syncthreads();  // the LDS stages of the previous segment are no longer read
+    dma_tile_mainloop<T, B_KC, BM, BN>(g, lds, tm, tn, it0, it1 - it0, [&](f32x16 (&acc)[TM][TN]) {
+      bool finish = (it0 == 0 && it1 == g.iters_per_tile);
+      if (!finish) {
+        // slot 0 of a workgroup: the tile it starts in; slot 1: a tile it enters from the left
+        float* slot = g.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * (BM * BN);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int64_t r = row0 + wm * WTM + i * 32 + lr;
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int cbase = col0 + wn * WTN + j * 32;
-      // element e of this lane: row r, column cbase + (e/4)*8 + lh*4 + e%4
-      if (bias != nullptr) {
+          for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          const int c = cbase + gq * 8 + lh * 4;
-          typedef T T4 __attribute__((ext_vector_type(4)));
-          T4 t = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-          if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+            for (int e = 0; e < 16; ++e)
+              __hip_atomic_store(slot + ((i * TN + j) * 16 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+        // device-coherent stores: waiting for their completion before the ticket publishes them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        const int w_first = sk_worker_of(g.sk_per, g.sk_rem, tile_begin);
+        const int w_last = sk_worker_of(g.sk_per, g.sk_rem, tile_end - 1);
+        if (tid == 0)
+          ticket_s = __hip_atomic_fetch_add(g.tickets + w_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket_s == (unsigned)(w_last - w_first)) {
+          finish = true;
 #pragma unroll
-          for (int t4 = 0; t4 < 4; ++t4)
-            acc[i][j][gq * 4 + t4] = acc[i][j][gq * 4 + t4] * alpha + (float)t[t4] * beta;
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+          for (int w2 = w_first; w2 <= w_last; ++w2) {
+            const float* src =
+                g.partials + ((int64_t)w2 * 2 + (sk_begin(g.sk_per, g.sk_rem, w2) < tile_begin ? 1 : 0)) * (BM * BN);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                  acc[i][j][e] += __hip_atomic_load(src + ((i * TN + j) * 16 + e) * 256 + tid, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+          }
+          if (tid == 0) __hip_atomic_store(g.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-      } else if (scale) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] *= alpha;
       }
-      unsigned pk[8];
-#pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        typedef T T2 __attribute__((ext_vector_type(2)));
-        const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
-        pk[d] = __builtin_bit_cast(unsigned, t);
-      }
-#pragma unroll
-      for (int gp = 0; gp < 2; ++gp) {
-        // register groups 2gp (X) and 2gp+1 (Y): after X.upper <-> Y.lower the lower half-wave owns
-        // the 8 columns of group 2gp, the upper half-wave those of group 2gp+1
-        unsigned x0 = pk[4 * gp], x1 = pk[4 * gp + 1], y0 = pk[4 * gp + 2], y1 = pk[4 * gp + 3];
-        swap_halves2(x0, y0, x1, y1);
-        const int c = cbase + (2 * gp + lh) * 8;
-        if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
-      }
-    }
+      if (finish) dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc);
+    });
+    u = tile_begin + it1;
   }
 }
 

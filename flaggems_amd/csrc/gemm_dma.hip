@@ -72,4 +72,61 @@ int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st) {
 #undef FG_DMA
 }
 
+
+// Stream-K on the direct-to-LDS main loop, 128x128 tiles: the tiles of the ragged last wave (all tiles, when there
+// is less than a wave of them) are shared K step by K step between one workgroup per CU; full waves in front of
+// them run data-parallel.  `g` must satisfy dma_supported(); the workspace is the one streamk_workspace_bytes()
+// sizes (tickets + two partial tiles per workgroup).
+template <typename T, bool B_KC>
+static int launch_dma_streamk_t(const GemmArgs& g, int dp_tiles, hipStream_t st) {
+  constexpr int LDS = dma_lds_bytes(128, 128);
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  auto dp = gemm_dma_kernel<T, B_KC, 128, 128>;
+  auto sk = gemm_dma_streamk_kernel<T, B_KC>;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(dp), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (attr_err == hipSuccess)
+      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(sk), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  });
+  if (attr_err != hipSuccess) {
+    fg_set_error("gemm(stream-K): cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
+    return FG_ERR_LAUNCH;
+  }
+  if (dp_tiles > 0) hipLaunchKernelGGL(dp, dim3((unsigned)dp_tiles), dim3(256), LDS, st, g);
+  if (g.sk_tiles > 0) hipLaunchKernelGGL(sk, dim3((unsigned)g.sk_workers), dim3(256), LDS, st, g);
+  return fg_check_launch("gemm(stream-K)");
+}
+
+int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st) {
+  FG_REQUIRE(workspace != nullptr && fg_aligned(workspace, 256), FG_ERR_WORKSPACE,
+             "gemm(stream-K): workspace must be 256-byte aligned");
+  FG_REQUIRE(num_cu <= kMaxWorkers, FG_ERR_UNSUPPORTED, "gemm(stream-K): more CUs than ticket counters");
+  FG_REQUIRE(workspace_bytes >= kPartialOffset + (size_t)num_cu * 2 * 128 * 128 * sizeof(float), FG_ERR_WORKSPACE,
+             "gemm(stream-K): workspace too small");
+  g.tiles_m = (int)fg_cdiv(g.M, 128);
+  g.tiles_n = (int)fg_cdiv(g.N, 128);
+  g.iters_per_tile = (int)(g.K / kDmaBK);
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  FG_REQUIRE(tiles < ((int64_t)1 << 30), FG_ERR_UNSUPPORTED, "gemm(stream-K): too many tiles");
+  int64_t sk_tiles = 0;
+  fg_streamk_partition(tiles, g.iters_per_tile, num_cu, &sk_tiles, nullptr, nullptr);
+  const int64_t total_iters = sk_tiles * g.iters_per_tile;
+  int workers = num_cu;
+  if (total_iters < workers) workers = (int)total_iters;
+  g.sk_tiles = (int)sk_tiles;
+  g.sk_workers = workers;
+  g.sk_per = workers > 0 ? total_iters / workers : 0;
+  g.sk_rem = workers > 0 ? total_iters % workers : 0;
+  g.tile_base = (int)sk_tiles;
+  char* ws = (char*)workspace;
+  g.tickets = (unsigned*)(ws + kTicketOffset);
+  g.partials = (float*)(ws + kPartialOffset);
+  const int dp_tiles = (int)(tiles - sk_tiles);
+  const bool kc = g.sbk == 1;
+  if (dtype == FG_BF16)
+    return kc ? launch_dma_streamk_t<bf16_t, true>(g, dp_tiles, st) : launch_dma_streamk_t<bf16_t, false>(g, dp_tiles, st);
+  return kc ? launch_dma_streamk_t<f16_t, true>(g, dp_tiles, st) : launch_dma_streamk_t<f16_t, false>(g, dp_tiles, st);
+}
+
 }  // namespace fgk

@@ -94,6 +94,10 @@ SK_CASES = [
     # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
     (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
+    # ... and the same schedule on the direct-to-LDS main loop (aligned operands, K a multiple of 64): less than
+    # a wave of tiles (chosen automatically), ragged edges with bias, full waves in front of the shared tiles
+    (512, 4096, 4096, _C.SCHED_AUTO), (256, 4096, 1024, _C.SCHED_AUTO), (1000, 1304, 2048, _C.SCHED_STREAM_K),
+    (3000, 4104, 1024, _C.SCHED_STREAM_K), (130, 136, 64, _C.SCHED_STREAM_K),
 ]
 
 
