@@ -267,6 +267,28 @@ def main():
                     workload="flash_attn_varlen_func decode: 64 seqs x 4096 keys, 1 query token each, 32q/8kv heads, D 128, page 16",
                     cpu=(cpu, 2 * S * Hk * D * 2, "oracle paged attention (torch CPU fp32) on one sequence"))
 
+    def wl_sdpa():
+        # dense causal attention through scaled_dot_product_attention (the caller's (batch, heads, seq, d) tensors
+        # are used in place as a virtual paged cache)
+        B, H, Hk, S, D = 8, 32, 8, 4096, 128
+        torch.manual_seed(0)
+        q = torch.randn(B, H, S, D, device=dev).to(bf16)
+        k = torch.randn(B, Hk, S, D, device=dev).to(bf16)
+        v = torch.randn(B, Hk, S, D, device=dev).to(bf16)
+
+        def run(i):
+            flag_gems.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+
+        rows = 64
+        qc, kc_, vc_ = q[:1, :, S - rows:].transpose(1, 2).cpu(), k[:1].transpose(1, 2).cpu(), v[:1].transpose(1, 2).cpu()
+
+        def cpu():
+            O.dense_attention(qc, kc_, vc_, D ** -0.5, causal=True)
+
+        return dict(run=run, work=4 * D * H * B * S * (S + 1) // 2, bound="mfma", dtype="bf16",
+                    workload="scaled_dot_product_attention causal, batch 8 x 4096 tokens, 32q/8kv heads, D 128",
+                    cpu=(cpu, 4 * D * H * rows * S, "oracle dense attention (torch CPU fp32), last %d query rows of one sequence" % rows))
+
     def wl_layer_c5():
         torch.manual_seed(0)
         Hd, H, D, F, bs, B, S = 4096, 32, 128, 11008, 16, 8, 2048
@@ -371,6 +393,7 @@ def main():
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "flash_attn_decode": wl_decode,
+        "sdpa_dense": wl_sdpa,
         "decoder_layer_c5": wl_layer_c5,
         "mfma_ceiling_random": lambda: wl_mfma_ceiling(True),
         "mfma_ceiling_zeros": lambda: wl_mfma_ceiling(False),

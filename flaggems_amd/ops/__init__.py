@@ -1,7 +1,10 @@
 from .addmm import addmm, addmm_out
-from .attention import flash_attn_varlen_func
+from .attention import flash_attention_forward, flash_attn_varlen_func, scaled_dot_product_attention
 from .mm import mm, mm_out
 from .rms_norm import rms_norm
 from .softmax import softmax
 
-__all__ = ["addmm", "addmm_out", "flash_attn_varlen_func", "mm", "mm_out", "rms_norm", "softmax"]
+__all__ = [
+    "addmm", "addmm_out", "flash_attention_forward", "flash_attn_varlen_func", "mm", "mm_out", "rms_norm",
+    "scaled_dot_product_attention", "softmax",
+]

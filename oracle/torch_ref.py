@@ -183,6 +183,42 @@ def paged_attention(query, key_cache, value_cache, query_lens, kv_lens, block_ta
     return out
 
 
+def dense_attention(q, k, v, scale, causal=False, window_size=(-1, -1), softcap=0.0, return_lse=False):
+    """tests/test_attention_ops.py:53-198 (construct_local_mask + attention_ref, the FlashAttention test
+    reference): q (batch, seqlen_q, heads, d), k / v (batch, seqlen_k, heads_k, d); fp32 arithmetic; GQA
+    by repeat_interleave; scores = scale * q . k^T, optional soft cap; keys col with
+    col > row + seqlen_k - seqlen_q + right or col < row + seqlen_k - seqlen_q - left are masked
+    (causal means right = 0: the mask is aligned to the bottom right corner); softmax; rows with no
+    visible key give zeros.  `return_lse` adds the log-sum-exp of the masked scores, (batch, heads, seqlen_q)."""
+    q, k, v = (to_reference(t).float() for t in (q, k, v))
+    left, right = window_size
+    if causal:
+        right = 0
+    seqlen_q, seqlen_k = q.shape[1], k.shape[1]
+    g = q.shape[2] // k.shape[2]
+    k = k.repeat_interleave(g, dim=2)
+    v = v.repeat_interleave(g, dim=2)
+    scores = torch.einsum("bthd,bshd->bhts", q * scale, k)
+    if softcap > 0:
+        scores = torch.tanh(scores / softcap) * softcap
+    if left >= 0 or right >= 0:
+        row = torch.arange(seqlen_q)[:, None]
+        col = torch.arange(seqlen_k)[None, :]
+        shift = seqlen_k - seqlen_q
+        if left < 0:
+            masked = col > row + shift + right
+        else:
+            hi = torch.minimum(row + shift + right, torch.tensor(seqlen_k)) if right >= 0 else torch.full_like(row, seqlen_k)
+            masked = (col > hi) | (col < row + shift - left)
+        scores = scores.masked_fill(masked, float("-inf"))
+    lse = torch.logsumexp(scores, dim=-1)
+    probs = torch.nan_to_num(torch.softmax(scores, dim=-1), nan=0.0)
+    out = torch.einsum("bhts,bshd->bthd", probs, v)
+    if return_lse:
+        return out, lse
+    return out
+
+
 def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping):
     """tests/test_attention_ops.py:1459-1467: python loop scatter.  Returns updated clones."""
     key, value = to_reference(key), to_reference(value)

@@ -162,6 +162,81 @@ def test_flash_attn_decode_variants(gpu):
     torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
 
 
+# Dense attention through the same kernel: aten::_flash_attention_forward and scaled_dot_product_attention
+# (reference: tests/test_attention_ops.py:540-575 test_flash_fwd_nonsquare_qk, :578-640 GQA and alibi, :296-330 sdpa).
+def _dense_inputs(dev, batch, heads, heads_k, sq, sk, d, dtype):
+    torch.manual_seed(1234567890)
+    q = torch.empty(batch, heads, sq, d, dtype=dtype, device=dev).uniform_(-0.05, 0.05)
+    k = torch.empty(batch, heads_k, sk, d, dtype=dtype, device=dev).uniform_(-0.05, 0.05)
+    v = torch.empty(batch, heads_k, sk, d, dtype=dtype, device=dev).uniform_(-0.05, 0.05)
+    return q, k, v
+
+
+@pytest.mark.parametrize("batch,heads,sq,sk", [(1, 1, 128, 2048), (4, 8, 1024, 128), (4, 8, 17, 1030)])
+@pytest.mark.parametrize("d", [64, 128, 192, 256])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_flash_attention_forward_nonsquare(gpu, batch, heads, sq, sk, d, causal, dtype):
+    q, k, v = _dense_inputs(gpu, batch, heads, heads, sq, sk, d, dtype)
+    scale = float(1.0 / np.sqrt(d))
+    # the caller holds (batch, heads, seq, d) tensors and passes transposed views, as torch's SDPA front end does
+    out, lse, *_ = flag_gems.ops.flash_attention_forward(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, None,
+                                                         sq, sk, 0, causal, False, scale=scale)
+    ref, rlse = O.dense_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), scale, causal=causal, return_lse=True)
+    atol, rtol = O.gems_tolerance(dtype)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=max(atol, 2e-3 if dtype == torch.bfloat16 else 2e-4), rtol=rtol)
+    fin = torch.isfinite(rlse)
+    torch.testing.assert_close(lse.cpu()[fin], rlse[fin], atol=1e-3, rtol=1e-4)
+    assert (lse.cpu()[~fin] == float("inf")).all()
+
+
+@pytest.mark.parametrize("heads,heads_k", [(8, 2), (6, 3), (4, 1)])
+@pytest.mark.parametrize("layout", ["bshd", "bhsd"])
+@pytest.mark.parametrize("window,softcap", [((-1, -1), 0.0), ((64, 0), 0.0), ((30, 20), 0.0), ((-1, -1), 15.0)])
+def test_flash_attention_forward_gqa_layouts_windows(gpu, heads, heads_k, layout, window, softcap):
+    batch, sq, sk, d, dtype = 3, 200, 384, 128, torch.bfloat16
+    q, k, v = _dense_inputs(gpu, batch, heads, heads_k, sq, sk, d, dtype)
+    if layout == "bshd":
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    else:
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))
+    causal = window == (-1, -1)
+    out, lse, *_ = flag_gems.ops.flash_attention_forward(q, k, v, None, None, sq, sk, 0, causal, False, scale=0.11, softcap=softcap,
+                                                         window_size_left=window[0], window_size_right=window[1])
+    ref, rlse = O.dense_attention(q, k, v, 0.11, causal=causal, window_size=window, softcap=softcap, return_lse=True)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=2e-3, rtol=1.6e-2)
+    torch.testing.assert_close(lse.cpu(), rlse, atol=1e-3, rtol=1e-4)
+
+
+def test_flash_attention_forward_dispatch_and_sdpa(gpu):
+    dtype = torch.bfloat16
+    q, k, v = _dense_inputs(gpu, 2, 8, 8, 256, 256, 128, dtype)
+    ref = O.dense_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), 128 ** -0.5, causal=True)
+    # the ATen operator, overridden inside use_gems()
+    with flag_gems.use_gems():
+        out, lse, *_ = torch.ops.aten._flash_attention_forward(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, None,
+                                                               256, 256, 0.0, True, False, scale=128 ** -0.5)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=2e-3, rtol=1.6e-2)
+    assert lse.shape == (2, 8, 256) and lse.dtype == torch.float32
+    # scaled_dot_product_attention: (batch, heads, seq, d) in and out, with and without GQA
+    o = flag_gems.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert o.shape == q.shape
+    torch.testing.assert_close(o.transpose(1, 2).float().cpu(), ref, atol=2e-3, rtol=1.6e-2)
+    qg, kg, vg = _dense_inputs(gpu, 2, 8, 2, 100, 333, 64, torch.float16)
+    o = flag_gems.scaled_dot_product_attention(qg, kg, vg, scale=0.2, enable_gqa=True)
+    refg = O.dense_attention(qg.transpose(1, 2), kg.transpose(1, 2), vg.transpose(1, 2), 0.2)
+    torch.testing.assert_close(o.transpose(1, 2).float().cpu(), refg, atol=2e-4, rtol=1e-3)
+    # what the kernel does not cover goes to torch's own implementation: an attention mask, a gradient
+    mask = torch.rand(2, 8, 256, 256, device=gpu) > 0.5
+    o = flag_gems.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    torch.testing.assert_close(o, torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask))
+    qr = q.clone().requires_grad_()
+    flag_gems.scaled_dot_product_attention(qr, k, v, is_causal=True).sum().backward()
+    assert qr.grad is not None and torch.isfinite(qr.grad).all()
+    with pytest.raises(AssertionError):
+        flag_gems.scaled_dot_product_attention(qg, kg, vg)  # different head counts need enable_gqa
+
+
 def test_flash_attn_varlen_out_argument_and_views(gpu):
     q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, [(40, 90), (17, 17)], 8, 2, 128, 16, 128, torch.bfloat16)
     out = torch.full_like(q, 7.0)

@@ -249,6 +249,48 @@ def test_paged_attention_special_cases():
     assert torch.allclose(o1, o2)
 
 
+@pytest.mark.parametrize("causal,window,softcap", [
+    (False, (-1, -1), 0.0), (True, (-1, -1), 0.0), (True, (2, 0), 0.0), (False, (1, 2), 0.0), (True, (-1, -1), 5.0),
+    (False, (3, -1), 0.0),
+])
+@pytest.mark.parametrize("sq,sk", [(5, 8), (8, 8), (7, 4)])
+def test_dense_attention_vs_brute_force(causal, window, softcap, sq, sk):
+    """The dense oracle against the scalar loops above, by presenting the batch as a paged cache (page = 4 rows)."""
+    g = torch.Generator().manual_seed(sq * 10 + sk)
+    B, H, Hk, D, bs = 2, 4, 2, 8, 4
+    q = torch.randn(B, sq, H, D, generator=g); k = torch.randn(B, sk, Hk, D, generator=g); v = torch.randn(B, sk, Hk, D, generator=g)
+    pages = (sk + bs - 1) // bs
+    kc = torch.zeros(B * pages, bs, Hk, D); vc = torch.zeros_like(kc)
+    for b in range(B):
+        for r in range(sk):
+            kc[b * pages + r // bs, r % bs] = k[b, r]; vc[b * pages + r // bs, r % bs] = v[b, r]
+    bt = torch.arange(B * pages, dtype=torch.int32).reshape(B, pages)
+    win = None if window == (-1, -1) else window
+    ref, rlse = brute_attention(q.reshape(B * sq, H, D), kc, vc, [sq] * B, [sk] * B, bt, 0.3, causal, win, softcap or None, None)
+    out, lse = O.dense_attention(q, k, v, 0.3, causal=causal, window_size=window, softcap=softcap, return_lse=True)
+    assert torch.allclose(out.double().reshape(B * sq, H, D), ref, atol=1e-5)
+    lse_flat = lse.permute(1, 0, 2).reshape(H, B * sq).double()
+    fin = torch.isfinite(rlse)
+    assert torch.allclose(lse_flat[fin], rlse[fin], atol=1e-4)
+    assert (lse_flat[~fin] == -math.inf).all()
+
+
+def test_dense_attention_special_cases():
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(1, 3, 2, 8, generator=g); k = torch.randn(1, 5, 2, 8, generator=g); v = torch.randn(1, 5, 2, 8, generator=g)
+    # one key: the output is that key's value row
+    out = O.dense_attention(q, k[:, :1], v[:, :1], 1.0)
+    assert torch.allclose(out, v[:, :1].expand(1, 3, 2, 8))
+    # zero queries: uniform weights, the mean of the visible values (causal, bottom-right: row r sees keys 0..r+2)
+    out = O.dense_attention(torch.zeros_like(q), k, v, 1.0, causal=True)
+    for r in range(3):
+        assert torch.allclose(out[0, r], v[0, : r + 3].mean(0), atol=1e-6)
+    # softmax is shift-invariant: adding a constant vector to every key direction of q . k changes nothing
+    out1 = O.dense_attention(q, k, v, 0.7)
+    out2 = O.dense_attention(q, k, v, 0.7, window_size=(100, 100))  # a window wider than the sequence masks nothing
+    assert torch.allclose(out1, out2)
+
+
 # ---------------------------------------------------------------------------------------------
 # byte / integer work: the C restatements
 # ---------------------------------------------------------------------------------------------
