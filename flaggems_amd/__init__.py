@@ -14,6 +14,7 @@ from . import config  # noqa: F401
 from . import runtime  # noqa: F401
 from . import testing  # noqa: F401
 from . import fused, ops  # noqa: F401
+from . import modules  # noqa: F401
 from .fused import *  # noqa: F401,F403
 from .logging_utils import setup_flaggems_logging
 from .ops import *  # noqa: F401,F403
