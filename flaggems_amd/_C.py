@@ -78,6 +78,7 @@ _SIGNATURES = {
     "fg_rms_norm": (c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_f32, c_int, c_vp]),
     "fg_fused_add_rms_norm": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_f32, c_int, c_vp]),
     "fg_softmax": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),
+    "fg_log_softmax": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),
     "fg_rope": (
         c_int,
         [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_int, c_i64, c_i64, c_int, c_int, c_int,

@@ -1,4 +1,4 @@
-// softmax forward for gfx950.
+// softmax and log_softmax forward for gfx950 (LOG selects out = (x - max) - log(sum) instead of e / sum).
 //
 // Inner axis (K == 1): the row lives in registers as fp32 (TPR threads per row, ITERS packs of VEC
 // elements per thread, same column interleave as the norm kernels), so HBM is read once and
@@ -36,7 +36,7 @@ __device__ __forceinline__ float row_reduce(float v, float* smem, int row_in_blo
   return v;
 }
 
-template <typename TI, typename TO, int VEC, int ITERS, int TPR>
+template <typename TI, typename TO, int VEC, int ITERS, int TPR, bool LOG>
 __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(const TI* __restrict__ in,
                                                                               TO* __restrict__ out, int64_t M,
                                                                               int N) {
@@ -75,13 +75,19 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
   for (int j = 0; j < ITERS; ++j) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      v[j][e] = fast_exp<sizeof(TI) == 4>(v[j][e] - m);
-      s += v[j][e];
+      if constexpr (LOG) {
+        v[j][e] -= m;
+        s += fast_exp<sizeof(TI) == 4>(v[j][e]);
+      } else {
+        v[j][e] = fast_exp<sizeof(TI) == 4>(v[j][e] - m);
+        s += v[j][e];
+      }
     }
   }
   s = row_reduce<TPR>(s, smem, row_in_block, t, OpSum(), 0.f);
   if (!row_ok) return;
   const float inv = 1.0f / s;
+  const float log_s = LOG ? logf(s) : 0.f;
   TO* yr = out + row * (int64_t)N;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
@@ -91,7 +97,8 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         // 16-bit results hide the last fp32 ulp, so the reciprocal multiply is exact enough there.
-        if constexpr (sizeof(TO) == 4) po.v[e] = (TO)(v[j][e] / s);
+        if constexpr (LOG) po.v[e] = (TO)(v[j][e] - log_s);
+        else if constexpr (sizeof(TO) == 4) po.v[e] = (TO)(v[j][e] / s);
         else po.v[e] = (TO)(v[j][e] * inv);
       }
       st_pack_nt<TO, VEC>(yr + col, po);
@@ -100,7 +107,7 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
 }
 
 // Any N: one block per row, online (max, sum) then a second sweep.
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool LOG>
 __global__ __launch_bounds__(256) void softmax_looped_kernel(const TI* __restrict__ in, TO* __restrict__ out,
                                                             int64_t M, int64_t N) {
   __shared__ float smem[4];
@@ -120,14 +127,15 @@ __global__ __launch_bounds__(256) void softmax_looped_kernel(const TI* __restric
   float zz = (m == -INFINITY) ? 0.f : z * __expf(m - mr);
   if (z != z) zz = z;
   const float s = row_reduce<256>(zz, smem, 0, threadIdx.x, OpSum(), 0.f);
+  const float log_s = LOG ? logf(s) : 0.f;
   for (int64_t c = threadIdx.x; c < N; c += 256) {
-    const float e = __expf((float)xr[c] - mr);
-    yr[c] = (TO)(e / s);
+    const float d = (float)xr[c] - mr;
+    yr[c] = LOG ? (TO)(d - log_s) : (TO)(__expf(d) / s);
   }
 }
 
 // Middle axis: in viewed as [M, N, K], K contiguous.  Thread = one (m, k) column.
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool LOG>
 __global__ __launch_bounds__(256) void softmax_non_inner_kernel(const TI* __restrict__ in, TO* __restrict__ out,
                                                                int64_t M, int64_t N, int64_t K) {
   const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -143,26 +151,27 @@ __global__ __launch_bounds__(256) void softmax_non_inner_kernel(const TI* __rest
     if (v != v) z = v;
     m = mn;
   }
+  const float log_z = LOG ? logf(z) : 0.f;
   for (int64_t n = 0; n < N; ++n) {
-    const float e = __expf((float)x[n * K] - m);
-    y[n * K] = (TO)(e / z);
+    const float d = (float)x[n * K] - m;
+    y[n * K] = LOG ? (TO)(d - log_z) : (TO)(__expf(d) / z);
   }
 }
 
-template <typename TI, typename TO, int VEC, int ITERS, int TPR>
+template <typename TI, typename TO, int VEC, int ITERS, int TPR, bool LOG>
 void launch_rows(const TI* in, TO* out, int64_t M, int N, hipStream_t st) {
   constexpr int BLOCK = TPR < 256 ? 256 : TPR;
   constexpr int RPB = BLOCK / TPR;
-  hipLaunchKernelGGL((softmax_rows_kernel<TI, TO, VEC, ITERS, TPR>), dim3((unsigned)fg_cdiv(M, RPB)), dim3(BLOCK), 0,
+  hipLaunchKernelGGL((softmax_rows_kernel<TI, TO, VEC, ITERS, TPR, LOG>), dim3((unsigned)fg_cdiv(M, RPB)), dim3(BLOCK), 0,
                      st, in, out, M, N);
 }
 
-template <typename TI, typename TO>
+template <typename TI, typename TO, bool LOG>
 int softmax_dispatch(const TI* in, TO* out, int64_t M, int64_t N, int64_t K, hipStream_t st) {
   if (K > 1) {
     FG_REQUIRE(M < 65536, FG_ERR_UNSUPPORTED, "softmax: leading extent %lld too large for the middle-axis kernel",
                (long long)M);
-    hipLaunchKernelGGL((softmax_non_inner_kernel<TI, TO>), dim3((unsigned)fg_cdiv(K, 256), (unsigned)M), dim3(256), 0,
+    hipLaunchKernelGGL((softmax_non_inner_kernel<TI, TO, LOG>), dim3((unsigned)fg_cdiv(K, 256), (unsigned)M), dim3(256), 0,
                        st, in, out, M, N, K);
     return fg_check_launch("softmax(non-inner)");
   }
@@ -171,9 +180,9 @@ int softmax_dispatch(const TI* in, TO* out, int64_t M, int64_t N, int64_t K, hip
   constexpr int VEC = 16 / sizeof(TI);
   const bool vec_ok = (N % VEC == 0) && fg_aligned(in, 16) && fg_aligned(out, sizeof(TO) * VEC);
   const int64_t packs = vec_ok ? N / VEC : 0;
-#define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR>(in, out, M, (int)N, st)
+#define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, LOG>(in, out, M, (int)N, st)
   if (!vec_ok || packs > 1024 * 8) {
-    hipLaunchKernelGGL((softmax_looped_kernel<TI, TO>), dim3((unsigned)M), dim3(256), 0, st, in, out, M, N);
+    hipLaunchKernelGGL((softmax_looped_kernel<TI, TO, LOG>), dim3((unsigned)M), dim3(256), 0, st, in, out, M, N);
   } else if (packs <= 64) {
     FG_ROWS(1, 64);
   } else if (packs <= 128) {
@@ -197,22 +206,33 @@ int softmax_dispatch(const TI* in, TO* out, int64_t M, int64_t N, int64_t K, hip
   return fg_check_launch("softmax");
 }
 
+template <bool LOG>
+int softmax_entry(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype, void* stream) {
+  const char* name = LOG ? "log_softmax" : "softmax";
+  FG_REQUIRE(M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "%s: negative size", name);
+  if (M == 0 || N == 0 || K == 0) return FG_OK;
+  FG_REQUIRE(in && out, FG_ERR_INVALID, "%s: null pointer", name);
+  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "%s: N=%lld too large", name, (long long)N);
+  FG_REQUIRE(out_dtype == in_dtype || out_dtype == FG_F32, FG_ERR_INVALID,
+             "%s: out dtype %d must equal in dtype %d or be fp32", name, out_dtype, in_dtype);
+  hipStream_t st = (hipStream_t)stream;
+  if (in_dtype == FG_F16 && out_dtype == FG_F16) return softmax_dispatch<f16_t, f16_t, LOG>((const f16_t*)in, (f16_t*)out, M, N, K, st);
+  if (in_dtype == FG_F16 && out_dtype == FG_F32) return softmax_dispatch<f16_t, float, LOG>((const f16_t*)in, (float*)out, M, N, K, st);
+  if (in_dtype == FG_BF16 && out_dtype == FG_BF16) return softmax_dispatch<bf16_t, bf16_t, LOG>((const bf16_t*)in, (bf16_t*)out, M, N, K, st);
+  if (in_dtype == FG_BF16 && out_dtype == FG_F32) return softmax_dispatch<bf16_t, float, LOG>((const bf16_t*)in, (float*)out, M, N, K, st);
+  if (in_dtype == FG_F32 && out_dtype == FG_F32) return softmax_dispatch<float, float, LOG>((const float*)in, (float*)out, M, N, K, st);
+  fg_set_error("%s: unsupported dtype pair (%d, %d)", name, in_dtype, out_dtype);
+  return FG_ERR_INVALID;
+}
+
 }  // namespace
 
 extern "C" int fg_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
                           void* stream) {
-  FG_REQUIRE(M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "softmax: negative size");
-  if (M == 0 || N == 0 || K == 0) return FG_OK;
-  FG_REQUIRE(in && out, FG_ERR_INVALID, "softmax: null pointer");
-  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "softmax: N=%lld too large", (long long)N);
-  FG_REQUIRE(out_dtype == in_dtype || out_dtype == FG_F32, FG_ERR_INVALID,
-             "softmax: out dtype %d must equal in dtype %d or be fp32", out_dtype, in_dtype);
-  hipStream_t st = (hipStream_t)stream;
-  if (in_dtype == FG_F16 && out_dtype == FG_F16) return softmax_dispatch((const f16_t*)in, (f16_t*)out, M, N, K, st);
-  if (in_dtype == FG_F16 && out_dtype == FG_F32) return softmax_dispatch((const f16_t*)in, (float*)out, M, N, K, st);
-  if (in_dtype == FG_BF16 && out_dtype == FG_BF16) return softmax_dispatch((const bf16_t*)in, (bf16_t*)out, M, N, K, st);
-  if (in_dtype == FG_BF16 && out_dtype == FG_F32) return softmax_dispatch((const bf16_t*)in, (float*)out, M, N, K, st);
-  if (in_dtype == FG_F32 && out_dtype == FG_F32) return softmax_dispatch((const float*)in, (float*)out, M, N, K, st);
-  fg_set_error("softmax: unsupported dtype pair (%d, %d)", in_dtype, out_dtype);
-  return FG_ERR_INVALID;
+  return softmax_entry<false>(in, out, M, N, K, in_dtype, out_dtype, stream);
+}
+
+extern "C" int fg_log_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype, int out_dtype,
+                              void* stream) {
+  return softmax_entry<true>(in, out, M, N, K, in_dtype, out_dtype, stream);
 }

@@ -74,6 +74,12 @@ int fg_fused_add_rms_norm(void* x, void* residual, const void* w, int64_t M, int
 int fg_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype,
                int out_dtype, void* stream);
 
+/* log_softmax over the middle axis of a contiguous [M, N, K] view: (x - max) - log(sum exp(x - max)), fp32
+ * arithmetic, out_dtype == in_dtype or FG_F32.  Same kernels as fg_softmax with a different last step.
+ * Replaces log_softmax_kernel, src/flag_gems/ops/log_softmax.py:15-58,98-128. */
+int fg_log_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype,
+               int out_dtype, void* stream);
+
 /* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
  * {token, head, dim}); cos/sin [max_pos, D/2] with unit inner stride.  pos == NULL means
  * position = token_index % seq_len.  q_out/k_out may alias q/k (in-place).

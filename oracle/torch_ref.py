@@ -41,6 +41,11 @@ def softmax(x, dim):
     return F.softmax(to_reference(x, True), dim=dim)
 
 
+def log_softmax(x, dim):
+    """tests/test_reduction_ops.py:466-480: F.log_softmax on an fp64 copy."""
+    return torch.nn.functional.log_softmax(to_reference(x, True), dim=dim)
+
+
 def rms_norm(x, weight, eps):
     """tests/test_norm_ops.py:539-544: fp32 normalisation, cast to the input dtype, then the weight
     multiply (the test does not widen to fp64 for this operator)."""

@@ -87,6 +87,33 @@ def test_softmax(gpu, shape, dtype, neg_inf):
         gems_assert_close(res, O.softmax(x, -1), torch.float32, equal_nan=True)
 
 
+# log_softmax: the same kernels with (x - max) - log(sum) as the last step (reference test:
+# tests/test_reduction_ops.py:466-480); vocabulary-sized rows included, -inf entries stay -inf.
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES + [(16, 2048), (7, 40999), (5, 33), (3, 70000), (8, 32000), (2, 151936)])
+def test_log_softmax(gpu, shape, dtype):
+    torch.manual_seed(0)
+    for dim in range(len(shape)):
+        x = torch.randn(shape, dtype=dtype, device=gpu)
+        ref = O.log_softmax(x, dim)
+        with flag_gems.use_gems():
+            res = torch.nn.functional.log_softmax(x, dim=dim)
+        gems_assert_close(res, ref, dtype)
+    xm = torch.where(x < -1.0, float("-inf"), x)
+    res = flag_gems.log_softmax(xm, -1)
+    fin = torch.isfinite(xm)
+    live = fin.any(-1, keepdim=True)  # a row of nothing but -inf is NaN (-inf - -inf), as in torch
+    assert (res[(~fin) & live] == float("-inf")).all()
+    gems_assert_close(res[fin], O.log_softmax(xm, -1)[fin.cpu()], dtype)
+    assert torch.isnan(res[(~live).expand_as(res)]).all()
+    if dtype != torch.float32:  # half_to_float
+        res = flag_gems.log_softmax(x, -1, True)
+        assert res.dtype == torch.float32
+        gems_assert_close(res, O.log_softmax(x, -1), torch.float32)
+    # exp(log_softmax) is softmax
+    torch.testing.assert_close(flag_gems.log_softmax(x, -1).double().exp().cpu(), O.softmax(x, -1), atol=1e-3, rtol=2e-2)
+
+
 def test_softmax_full_size_properties(gpu):
     """[131072, 2048] bf16 with 1 % -inf (the benchmark input): rows sum to 1, masked entries are exact
     zeros, sampled rows match the oracle, and adding a constant to a row changes nothing."""

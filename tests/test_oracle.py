@@ -90,6 +90,29 @@ def test_fused_add_rms_norm_both_outputs():
 # ---------------------------------------------------------------------------------------------
 # softmax
 # ---------------------------------------------------------------------------------------------
+def test_log_softmax_pinned():
+    """Closed forms and a scalar loop: log_softmax(x) = x - log(sum(exp(x))); uniform rows give -log(N)."""
+    import math
+    x = torch.tensor([[0.0, math.log(2.0), math.log(5.0)], [3.0, 3.0, 3.0]], dtype=torch.float32)
+    y = O.log_softmax(x, -1)
+    assert torch.allclose(y[0], torch.tensor([-math.log(8.0), math.log(2.0 / 8.0), math.log(5.0 / 8.0)], dtype=torch.float64))
+    assert torch.allclose(y[1], torch.full((3,), -math.log(3.0), dtype=torch.float64))
+    g = torch.Generator().manual_seed(3)
+    z = torch.randn(4, 5, 6, generator=g)
+    for dim in range(3):
+        got = O.log_softmax(z, dim)
+        zz = z.double().movedim(dim, -1).contiguous()
+        rows = []
+        for row in zz.reshape(-1, zz.shape[-1]):
+            lse = math.log(sum(math.exp(float(v)) for v in row))
+            rows.append([float(v) - lse for v in row])
+        want = torch.tensor(rows, dtype=torch.float64).reshape(zz.shape)
+        assert torch.allclose(got, want.movedim(-1, dim), atol=1e-12)
+        assert torch.allclose(got.exp(), O.softmax(z, dim), atol=1e-12)
+    w = torch.tensor([[1.0, float("-inf"), 2.0]])
+    assert O.log_softmax(w, -1)[0, 1] == float("-inf")
+
+
 def test_softmax_invariants():
     x = torch.randn(6, 11, generator=torch.Generator().manual_seed(2))
     x[0, 3] = float("-inf"); x[2] = float("-inf")
