@@ -96,6 +96,11 @@ _SIGNATURES = {
         [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
          c_f32, c_f32, c_int, c_int, c_int, c_int, c_vp, ctypes.c_size_t, ctypes.POINTER(c_int), c_vp],
     ),
+    "fg_bmm": (
+        c_int,
+        [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+         c_int, c_vp],
+    ),
     "fg_streamk_partition": (
         c_int,
         [c_i64, c_i64, c_i64, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],

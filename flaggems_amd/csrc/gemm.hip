@@ -229,3 +229,23 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
     default: return run_dp<float>(g, amode, bmode, cu, st);
   }
 }
+
+extern "C" int fg_bmm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                      int64_t sab, int64_t sam, int64_t sak, int64_t sbb, int64_t sbk, int64_t sbn, int64_t scb,
+                      int64_t scm, int64_t scn, int dtype, void* stream) {
+  FG_REQUIRE(batch >= 0 && M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "bmm: negative size");
+  FG_REQUIRE(dtype == FG_F16 || dtype == FG_BF16 || dtype == FG_F32, FG_ERR_INVALID, "bmm: bad dtype %d", dtype);
+  if (batch == 0 || M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(K > 0, FG_ERR_INVALID, "bmm: K must be positive (the caller handles K == 0)");
+  FG_REQUIRE(A && B && C, FG_ERR_INVALID, "bmm: null pointer");
+  // One data-parallel 2-D launch per matrix, back to back on the stream: every matrix takes the kernel and
+  // tile size its own pointers and strides qualify for.
+  const int64_t eb = dtype == FG_F32 ? 4 : 2;
+  for (int64_t z = 0; z < batch; ++z) {
+    const int rc = fg_gemm((const char*)A + z * sab * eb, (const char*)B + z * sbb * eb, nullptr,
+                           (char*)C + z * scb * eb, M, N, K, sam, sak, sbk, sbn, 0, 0, scm, scn, 1.0f, 0.0f, dtype,
+                           dtype, dtype, FG_SCHED_DATA_PARALLEL, nullptr, 0, nullptr, stream);
+    if (rc != FG_OK) return rc;
+  }
+  return FG_OK;
+}

@@ -24,8 +24,9 @@ def _kernel_covers(a, b):
 
 
 def _vendor_mm(a, b, out=None):
-    # bmm is a separate ATen kernel, so this cannot re-enter the override
-    r = torch.bmm(a.unsqueeze(0), b.unsqueeze(0)).squeeze(0)
+    # bmm.out is a separate ATen kernel that is never overridden, so this cannot re-enter
+    r = torch.empty((1, a.shape[0], b.shape[1]), dtype=torch.result_type(a, b), device=a.device)
+    r = torch.ops.aten.bmm.out(a.unsqueeze(0), b.unsqueeze(0), out=r).squeeze(0)
     if out is None:
         return r
     out.copy_(r)

@@ -132,6 +132,14 @@ int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, 
             int c_dtype, int bias_dtype, int schedule, void* workspace, size_t workspace_bytes,
             int* schedule_used, void* stream);
 
+/* C[b] = A[b] . B[b] for b in [0, batch), fp32 accumulate, every operand addressed through
+ * (matrix, row, col) element strides (a matrix stride of 0 broadcasts one operand).  Matrix b is
+ * one data-parallel fg_gemm launch; the launches follow each other on the stream.
+ * Replaces bmm_kernel (src/flag_gems/ops/bmm.py:15-136) and its C++ twin lib/bmm.cpp. */
+int fg_bmm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
+           int64_t sab, int64_t sam, int64_t sak, int64_t sbb, int64_t sbk, int64_t sbn,
+           int64_t scb, int64_t scm, int64_t scn, int dtype, void* stream);
+
 /* Host-side stream-K partition (pure integer function; also used by the tests).
  * Given `tiles` output tiles of `iters_per_tile` K-iterations each and `workers` persistent
  * workgroups, worker w owns the half-open range [begin[w], end[w]) of the tile-major iteration

@@ -36,6 +36,11 @@ def addmm(bias, a, b, alpha=1, beta=1):
     return torch.addmm(to_reference(bias, True), to_reference(a, True), to_reference(b, True), alpha=alpha, beta=beta)
 
 
+def bmm(a, b):
+    """tests/test_blas_ops.py:95-110: torch.bmm on fp64 copies."""
+    return torch.bmm(to_reference(a, True), to_reference(b, True))
+
+
 def softmax(x, dim):
     """tests/test_reduction_ops.py:507-523: F.softmax on an fp64 copy."""
     return F.softmax(to_reference(x, True), dim=dim)

@@ -59,6 +59,65 @@ def test_addmm(gpu, M, N, K, scalar, dtype, b_col_major):
     gems_assert_close(out, ref, dtype, reduce_dim=K)
 
 
+BMM_LAYOUTS = ["contiguous", "b_transposed", "a_transposed", "broadcast_b", "batch_inner"]
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("M,N,K", MNK_SHAPES + EXTRA_SHAPES[:3] + [(256, 512, 128), (77, 40, 24)])
+@pytest.mark.parametrize("layout", BMM_LAYOUTS)
+def test_bmm(gpu, M, N, K, dtype, layout):
+    """tests/test_blas_ops.py:95-110 of the reference (batch 4), plus operand layouts the kernels take
+    without a copy: transposed matrices, one matrix broadcast over the batch, batch as the middle dim."""
+    torch.manual_seed(0)
+    batch = 4
+    a = torch.randn(batch, M, K, dtype=dtype, device=gpu)
+    b = torch.randn(batch, K, N, dtype=dtype, device=gpu)
+    if layout == "b_transposed":
+        b = torch.randn(batch, N, K, dtype=dtype, device=gpu).transpose(1, 2)
+    elif layout == "a_transposed":
+        a = torch.randn(batch, K, M, dtype=dtype, device=gpu).transpose(1, 2)
+    elif layout == "broadcast_b":
+        b = torch.randn(K, N, dtype=dtype, device=gpu).expand(batch, K, N)
+    elif layout == "batch_inner":
+        a = torch.randn(M, batch, K, dtype=dtype, device=gpu).transpose(0, 1)
+        b = torch.randn(K, batch, N, dtype=dtype, device=gpu).transpose(0, 1)
+    ref = O.bmm(a, b)
+    with flag_gems.use_gems():
+        res = torch.bmm(a, b)
+    assert res.shape == (batch, M, N) and res.is_contiguous()
+    gems_assert_close(res, ref, dtype, reduce_dim=K)
+
+
+def test_bmm_special_cases(gpu):
+    torch.manual_seed(2)
+    a = torch.randn(3, 33, 40, device=gpu); b = torch.randn(3, 40, 17, device=gpu)
+    # every matrix of the batch equals the 2-D product of its operands, bit for bit (same kernel, same order)
+    res = flag_gems.bmm(a, b)
+    for z in range(3):
+        assert torch.equal(res[z], flag_gems.mm(a[z], b[z]))
+    # batch of one, empty extents, K == 0
+    gems_assert_close(flag_gems.bmm(a[:1], b[:1]), O.bmm(a[:1], b[:1]), torch.float32, reduce_dim=40)
+    assert flag_gems.bmm(a[:0], b[:0]).shape == (0, 33, 17)
+    assert flag_gems.bmm(a[:, :0], b).shape == (3, 0, 17)
+    z = flag_gems.bmm(a[:, :, :0], b[:, :0])
+    assert z.shape == (3, 33, 17) and not z.any()
+    # dtypes the kernels do not cover stay on the vendor library, also under the override
+    with flag_gems.use_gems():
+        d = torch.bmm(a.double(), b.double())
+        m = torch.mm(a[0].double(), b[0].double())
+    assert d.dtype == torch.float64 and torch.allclose(d.cpu(), O.bmm(a, b), atol=1e-10)
+    assert torch.allclose(m.cpu(), O.mm(a[0], b[0]), atol=1e-10)
+    with pytest.raises(AssertionError):
+        flag_gems.bmm(a, b[:2])
+    # a large aligned batch on the direct-to-LDS kernels (attention-like shapes), against the oracle
+    q = torch.randn(16, 512, 128, device=gpu, dtype=torch.bfloat16)
+    k = torch.randn(16, 512, 128, device=gpu, dtype=torch.bfloat16)
+    s = flag_gems.bmm(q, k.transpose(1, 2))
+    gems_assert_close(s, O.bmm(q, k.transpose(1, 2)), torch.bfloat16, reduce_dim=128)
+    v = torch.randn(16, 512, 128, device=gpu, dtype=torch.bfloat16)
+    gems_assert_close(flag_gems.bmm(s, v), O.bmm(s, v), torch.bfloat16, reduce_dim=512)
+
+
 def test_addmm_special_cases(gpu):
     torch.manual_seed(1)
     a = torch.randn(33, 40, device=gpu); b = torch.randn(40, 17, device=gpu); bias = torch.randn(17, device=gpu)

@@ -140,6 +140,24 @@ def test_mm_addmm_roles():
     assert torch.equal(O.addmm(bias, a, b, alpha=0, beta=1), bias.double().expand(3, 4))
 
 
+def test_bmm_pinned():
+    """Scalar triple loop per matrix; matrix b of the result depends on matrix b of the inputs only."""
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(3, 4, 5, generator=g); b = torch.randn(3, 5, 2, generator=g)
+    got = O.bmm(a, b)
+    assert got.dtype == torch.float64 and got.shape == (3, 4, 2)
+    for z in range(3):
+        for i in range(4):
+            for j in range(2):
+                want = sum(float(a[z, i, k]) * float(b[z, k, j]) for k in range(5))
+                assert abs(float(got[z, i, j]) - want) < 1e-12
+        assert torch.equal(got[z], O.mm(a[z], b[z]))
+    # (A.B)^T = B^T.A^T per matrix; permuting the batch permutes the result
+    assert torch.allclose(O.bmm(b.transpose(1, 2), a.transpose(1, 2)), got.transpose(1, 2), atol=1e-12)
+    perm = torch.tensor([2, 0, 1])
+    assert torch.equal(O.bmm(a[perm], b[perm]), got[perm])
+
+
 # ---------------------------------------------------------------------------------------------
 # rope
 # ---------------------------------------------------------------------------------------------
