@@ -15,9 +15,11 @@ from . import runtime  # noqa: F401
 from . import testing  # noqa: F401
 from . import fused, ops  # noqa: F401
 from . import modules  # noqa: F401
+from . import patches  # noqa: F401
 from .fused import *  # noqa: F401,F403
 from .logging_utils import setup_flaggems_logging
 from .ops import *  # noqa: F401,F403
+from .patches import apply_gems_patches_to_vllm  # noqa: F401
 from .runtime.register import Register
 
 __version__ = "3.0"
@@ -92,4 +94,4 @@ def all_ops():
     return current_work_registrar.get_all_ops()
 
 
-__all__ = ["enable", "use_gems", "all_ops"] + list(ops.__all__) + list(fused.__all__)
+__all__ = ["enable", "use_gems", "all_ops", "apply_gems_patches_to_vllm"] + list(ops.__all__) + list(fused.__all__)
