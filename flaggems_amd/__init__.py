@@ -32,11 +32,13 @@ current_work_registrar = None
 
 def _aten_table():
     """(aten overload, python kernel) rows of the reference's table that lie on this path
-    (src/flag_gems/__init__.py:38-39,41,55-56,89,213-214,275)."""
+    (src/flag_gems/__init__.py:38-42,55-56,89,213-214,275)."""
     return (
         ("_flash_attention_forward", flash_attention_forward),  # noqa: F405
         ("_log_softmax", log_softmax),  # noqa: F405
+        ("_log_softmax_backward_data", log_softmax_backward),  # noqa: F405
         ("_softmax", softmax),  # noqa: F405
+        ("_softmax_backward_data", softmax_backward),  # noqa: F405
         ("addmm", addmm),  # noqa: F405
         ("addmm.out", addmm_out),  # noqa: F405
         ("bmm", bmm),  # noqa: F405

@@ -1,0 +1,301 @@
+// Row-wise backward passes for gfx950: softmax, log_softmax and rms_norm.
+//
+// All three have the shape of their forward kernels: two inputs in the forward's row layout, one
+// fp32 sum per row, one output.
+//   softmax:      dx = y * (dy - sum(y * dy))
+//   log_softmax:  dx = dy - exp(y) * sum(dy)
+//   rms_norm:     g = dy * w, xh = x * inv_rms, dx = (g - xh * sum(xh * g) / N) * inv_rms
+// Inner axis (K == 1): the two rows live in registers as fp32 (TPR threads per row, ITERS packs of
+// VEC elements per thread), so HBM is read once per input and written once.  Rows that do not fit,
+// or that defeat 16-byte access, use a looped kernel that reads the row twice (the second time from
+// L2).  Middle axis (softmax only, K > 1): one thread per (m, k) column, walking N with stride K.
+// The weight gradient of rms_norm is a column sum over all rows: a first kernel leaves one fp32
+// partial row per block of rows, the caller adds the partial rows up.
+#include "fg_common.h"
+
+namespace {
+
+enum { BWD_SOFTMAX = 0, BWD_LOG_SOFTMAX = 1, BWD_RMS = 2 };
+
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* smem, int row_in_block, int t) {
+  v = wave_sum(v);
+  if constexpr (TPR > 64) {
+    constexpr int WPR = TPR / 64;  // waves per row
+    __syncthreads();
+    if ((t & 63) == 0) smem[row_in_block * WPR + (t >> 6)] = v;
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) s += smem[row_in_block * WPR + i];
+    v = s;
+  }
+  return v;
+}
+
+template <typename T> __device__ __forceinline__ float exp_like_forward(float x) {
+  if constexpr (sizeof(T) == 4) return expf(x);
+  else return __expf(x);
+}
+
+// a: y (softmax modes) or x (rms); g: dy.  w and inv_rms are read in the rms mode only (w may be null).
+template <typename TI, typename TO, int VEC, int ITERS, int TPR, int MODE>
+__global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const TI* __restrict__ a,
+                                                                          const TI* __restrict__ g,
+                                                                          const TI* __restrict__ w,
+                                                                          const float* __restrict__ inv_rms,
+                                                                          TO* __restrict__ out, int64_t M, int N) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ float smem[BLOCK / 64];
+  const int tid = threadIdx.x;
+  const int row_in_block = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + row_in_block;
+  const bool row_ok = row < M;
+  const TI* ar = a + row * (int64_t)N;
+  const TI* gr = g + row * (int64_t)N;
+  float inv = 1.0f;
+  if constexpr (MODE == BWD_RMS) {
+    if (row_ok) inv = inv_rms[row];
+  }
+
+  float va[ITERS][VEC], vg[ITERS][VEC];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    if (row_ok && col < N) {
+      const Pack<TI, VEC> pa = ld_pack_nt<TI, VEC>(ar + col);
+      const Pack<TI, VEC> pg = ld_pack_nt<TI, VEC>(gr + col);
+      if constexpr (MODE == BWD_RMS) {
+        Pack<TI, VEC> pw;
+        if (w != nullptr) pw = ld_pack<TI, VEC>(w + col);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          va[j][e] = (float)pa.v[e] * inv;
+          vg[j][e] = w != nullptr ? (float)pg.v[e] * (float)pw.v[e] : (float)pg.v[e];
+          s += va[j][e] * vg[j][e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          va[j][e] = (float)pa.v[e];
+          vg[j][e] = (float)pg.v[e];
+          s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) va[j][e] = vg[j][e] = 0.f;
+    }
+  }
+  s = row_sum<TPR>(s, smem, row_in_block, t);
+  if (!row_ok) return;
+  const float mean = s / (float)N;
+  TO* orow = out + row * (int64_t)N;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    if (col < N) {
+      Pack<TO, VEC> po;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float r;
+        if constexpr (MODE == BWD_SOFTMAX) r = va[j][e] * (vg[j][e] - s);
+        else if constexpr (MODE == BWD_LOG_SOFTMAX) r = vg[j][e] - exp_like_forward<TI>(va[j][e]) * s;
+        else r = (vg[j][e] - va[j][e] * mean) * inv;
+        po.v[e] = (TO)r;
+      }
+      st_pack_nt<TO, VEC>(orow + col, po);
+    }
+  }
+}
+
+// Any N, any alignment: one 256-thread block per row, element-wise access, two sweeps.
+template <typename TI, typename TO, int MODE>
+__global__ __launch_bounds__(256) void bwd_looped_kernel(const TI* __restrict__ a, const TI* __restrict__ g,
+                                                        const TI* __restrict__ w, const float* __restrict__ inv_rms,
+                                                        TO* __restrict__ out, int64_t M, int64_t N) {
+  __shared__ float smem[4];
+  const int64_t row = blockIdx.x;
+  const TI* ar = a + row * N;
+  const TI* gr = g + row * N;
+  TO* orow = out + row * N;
+  const float inv = MODE == BWD_RMS ? inv_rms[row] : 1.0f;
+  float s = 0.f;
+  for (int64_t c = threadIdx.x; c < N; c += 256) {
+    const float x = (float)ar[c], d = (float)gr[c];
+    if constexpr (MODE == BWD_SOFTMAX) s += x * d;
+    else if constexpr (MODE == BWD_LOG_SOFTMAX) s += d;
+    else s += x * inv * d * (w != nullptr ? (float)w[c] : 1.0f);
+  }
+  s = row_sum<256>(s, smem, 0, threadIdx.x);
+  const float mean = s / (float)N;
+  for (int64_t c = threadIdx.x; c < N; c += 256) {
+    const float x = (float)ar[c], d = (float)gr[c];
+    float r;
+    if constexpr (MODE == BWD_SOFTMAX) r = x * (d - s);
+    else if constexpr (MODE == BWD_LOG_SOFTMAX) r = d - exp_like_forward<TI>(x) * s;
+    else r = (d * (w != nullptr ? (float)w[c] : 1.0f) - x * inv * mean) * inv;
+    orow[c] = (TO)r;
+  }
+}
+
+// Middle axis: tensors viewed as [M, N, K], K contiguous.  Thread = one (m, k) column.
+template <typename TI, typename TO, int MODE>
+__global__ __launch_bounds__(256) void bwd_non_inner_kernel(const TI* __restrict__ y, const TI* __restrict__ g,
+                                                           TO* __restrict__ out, int64_t M, int64_t N, int64_t K) {
+  const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t mrow = blockIdx.y;
+  if (k >= K) return;
+  const int64_t base = mrow * N * K + k;
+  float s = 0.f;
+  for (int64_t n = 0; n < N; ++n) {
+    const float x = (float)y[base + n * K], d = (float)g[base + n * K];
+    s += MODE == BWD_SOFTMAX ? x * d : d;
+  }
+  for (int64_t n = 0; n < N; ++n) {
+    const float x = (float)y[base + n * K], d = (float)g[base + n * K];
+    out[base + n * K] = MODE == BWD_SOFTMAX ? (TO)(x * (d - s)) : (TO)(d - exp_like_forward<TI>(x) * s);
+  }
+}
+
+// Partial weight gradient of rms_norm: block (rb, cb) sums x * dy * inv_rms over rows
+// [rb * rows_per_block, ...) for its 256 columns and writes row rb of `partial` [row_blocks, N].
+template <typename T>
+__global__ __launch_bounds__(256) void rms_dw_partial_kernel(const T* __restrict__ x, const T* __restrict__ dy,
+                                                            const float* __restrict__ inv_rms,
+                                                            float* __restrict__ partial, int64_t M, int64_t N,
+                                                            int rows_per_block) {
+  const int64_t c = (int64_t)blockIdx.y * 256 + threadIdx.x;
+  if (c >= N) return;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+  int64_t r1 = r0 + rows_per_block;
+  if (r1 > M) r1 = M;
+  float s = 0.f;
+  for (int64_t r = r0; r < r1; ++r) s += (float)x[r * N + c] * (float)dy[r * N + c] * inv_rms[r];
+  partial[(int64_t)blockIdx.x * N + c] = s;
+}
+
+template <typename TI, typename TO, int VEC, int ITERS, int TPR, int MODE>
+void launch_rows(const TI* a, const TI* g, const TI* w, const float* inv_rms, TO* out, int64_t M, int N,
+                 hipStream_t st) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  hipLaunchKernelGGL((bwd_rows_kernel<TI, TO, VEC, ITERS, TPR, MODE>), dim3((unsigned)fg_cdiv(M, RPB)), dim3(BLOCK), 0,
+                     st, a, g, w, inv_rms, out, M, N);
+}
+
+// Inner-axis dispatch shared by the three modes.  The caller has checked sizes and pointers.
+template <typename TI, typename TO, int MODE>
+int bwd_rows_dispatch(const TI* a, const TI* g, const TI* w, const float* inv_rms, TO* out, int64_t M, int64_t N,
+                      hipStream_t st, const char* what) {
+  FG_REQUIRE(M < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "%s: M=%lld exceeds the grid limit", what, (long long)M);
+  constexpr int VEC = 16 / sizeof(TI);
+  const bool vec_ok = (N % VEC == 0) && fg_aligned(a, 16) && fg_aligned(g, 16) && fg_aligned(out, sizeof(TO) * VEC) &&
+                      (w == nullptr || fg_aligned(w, 16));
+  const int64_t packs = vec_ok ? N / VEC : 0;
+#define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, MODE>(a, g, w, inv_rms, out, M, (int)N, st)
+  // two input streams: one pack per thread from each, as in the fused add + norm forward
+  if (!vec_ok || packs > 2048) {
+    hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE>), dim3((unsigned)M), dim3(256), 0, st, a, g, w, inv_rms, out, M,
+                       N);
+  } else if (packs <= 64) {
+    FG_ROWS(1, 64);
+  } else if (packs <= 128) {
+    FG_ROWS(1, 128);
+  } else if (packs <= 256) {
+    FG_ROWS(1, 256);
+  } else if (packs <= 512) {
+    FG_ROWS(1, 512);
+  } else if (packs <= 1024) {
+    FG_ROWS(1, 1024);
+  } else {
+    FG_ROWS(2, 1024);
+  }
+#undef FG_ROWS
+  return fg_check_launch(what);
+}
+
+template <typename TI, typename TO, int MODE>
+int softmax_bwd_dispatch(const TI* y, const TI* g, TO* out, int64_t M, int64_t N, int64_t K, hipStream_t st,
+                         const char* what) {
+  if (K > 1) {
+    FG_REQUIRE(M < 65536, FG_ERR_UNSUPPORTED, "%s: leading extent %lld too large for the middle-axis kernel", what,
+               (long long)M);
+    hipLaunchKernelGGL((bwd_non_inner_kernel<TI, TO, MODE>), dim3((unsigned)fg_cdiv(K, 256), (unsigned)M), dim3(256), 0,
+                       st, y, g, out, M, N, K);
+    return fg_check_launch(what);
+  }
+  return bwd_rows_dispatch<TI, TO, MODE>(y, g, nullptr, nullptr, out, M, N, st, what);
+}
+
+template <int MODE>
+int softmax_bwd_entry(const void* y, const void* g, void* out, int64_t M, int64_t N, int64_t K, int dtype,
+                      int out_dtype, void* stream) {
+  const char* what = MODE == BWD_SOFTMAX ? "softmax_backward" : "log_softmax_backward";
+  FG_REQUIRE(M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "%s: negative size", what);
+  if (M == 0 || N == 0 || K == 0) return FG_OK;
+  FG_REQUIRE(y && g && out, FG_ERR_INVALID, "%s: null pointer", what);
+  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "%s: N=%lld too large", what, (long long)N);
+  FG_REQUIRE(out_dtype == dtype || dtype == FG_F32, FG_ERR_INVALID,
+             "%s: gradient dtype %d must equal the output dtype %d unless that is fp32", what, out_dtype, dtype);
+  hipStream_t st = (hipStream_t)stream;
+#define FG_CASE(DI, DO, TI, TO) \
+  if (dtype == DI && out_dtype == DO) \
+    return softmax_bwd_dispatch<TI, TO, MODE>((const TI*)y, (const TI*)g, (TO*)out, M, N, K, st, what)
+  FG_CASE(FG_F16, FG_F16, f16_t, f16_t);
+  FG_CASE(FG_BF16, FG_BF16, bf16_t, bf16_t);
+  FG_CASE(FG_F32, FG_F32, float, float);
+  FG_CASE(FG_F32, FG_F16, float, f16_t);
+  FG_CASE(FG_F32, FG_BF16, float, bf16_t);
+#undef FG_CASE
+  fg_set_error("%s: unsupported dtype pair (%d, %d)", what, dtype, out_dtype);
+  return FG_ERR_INVALID;
+}
+
+}  // namespace
+
+extern "C" int fg_softmax_backward(const void* out, const void* grad_out, void* grad_in, int64_t M, int64_t N,
+                                   int64_t K, int dtype, int grad_in_dtype, void* stream) {
+  return softmax_bwd_entry<BWD_SOFTMAX>(out, grad_out, grad_in, M, N, K, dtype, grad_in_dtype, stream);
+}
+
+extern "C" int fg_log_softmax_backward(const void* out, const void* grad_out, void* grad_in, int64_t M, int64_t N,
+                                       int64_t K, int dtype, int grad_in_dtype, void* stream) {
+  return softmax_bwd_entry<BWD_LOG_SOFTMAX>(out, grad_out, grad_in, M, N, K, dtype, grad_in_dtype, stream);
+}
+
+extern "C" int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,
+                                    float* dw_partial, int rows_per_block, int64_t M, int64_t N, int dtype,
+                                    void* stream) {
+  FG_REQUIRE(M >= 0 && N >= 0, FG_ERR_INVALID, "rms_norm_backward: negative size");
+  if (M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(x && dy && inv_rms && dx, FG_ERR_INVALID, "rms_norm_backward: null pointer");
+  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "rms_norm_backward: N=%lld too large", (long long)N);
+  FG_REQUIRE(dw_partial == nullptr || rows_per_block > 0, FG_ERR_INVALID,
+             "rms_norm_backward: rows_per_block must be positive");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = FG_ERR_INVALID;
+  const int64_t row_blocks = dw_partial ? fg_cdiv(M, rows_per_block) : 0;
+  FG_REQUIRE(row_blocks < ((int64_t)1 << 31) && fg_cdiv(N, 256) < 65536, FG_ERR_UNSUPPORTED,
+             "rms_norm_backward: problem too large for the weight-gradient grid");
+#define FG_CASE(D, T)                                                                                               \
+  if (dtype == D) {                                                                                                 \
+    rc = bwd_rows_dispatch<T, T, BWD_RMS>((const T*)x, (const T*)dy, (const T*)w, inv_rms, (T*)dx, M, N, st,        \
+                                          "rms_norm_backward");                                                     \
+    if (rc == FG_OK && dw_partial != nullptr) {                                                                     \
+      hipLaunchKernelGGL((rms_dw_partial_kernel<T>), dim3((unsigned)row_blocks, (unsigned)fg_cdiv(N, 256)), dim3(256), \
+                         0, st, (const T*)x, (const T*)dy, inv_rms, dw_partial, M, N, rows_per_block);              \
+      rc = fg_check_launch("rms_norm_backward(dw)");                                                                \
+    }                                                                                                               \
+    return rc;                                                                                                      \
+  }
+  FG_CASE(FG_F16, f16_t)
+  FG_CASE(FG_BF16, bf16_t)
+  FG_CASE(FG_F32, float)
+#undef FG_CASE
+  fg_set_error("rms_norm_backward: unsupported dtype %d", dtype);
+  return FG_ERR_INVALID;
+}

@@ -18,6 +18,7 @@ SOURCES = [
     "abi.cpp",
     "norm.hip",
     "softmax.hip",
+    "backward.hip",
     "rope.hip",
     "kvcache.hip",
     "silu_mul.hip",

@@ -1,9 +1,11 @@
-"""aten::_log_softmax forward on the gfx950 kernels (reference: src/flag_gems/ops/log_softmax.py:98-128)."""
+"""aten::_log_softmax and aten::_log_softmax_backward_data on the gfx950 kernels
+(reference: src/flag_gems/ops/log_softmax.py:98-160)."""
 import logging
 
 import torch
 
 from .. import _C
+from .softmax import _backward
 
 logger = logging.getLogger("flag_gems.ops.log_softmax")
 
@@ -33,3 +35,8 @@ def log_softmax(self, dim, half_to_float=False):
         )
     _C.check(rc, "fg_log_softmax")
     return out
+
+
+def log_softmax_backward(grad_output, output, dim, input_dtype):
+    logger.debug("GEMS LOG_SOFTMAX VJP")
+    return _backward("_log_softmax_backward_data", "out", "fg_log_softmax_backward", grad_output, output, dim, input_dtype)

@@ -80,6 +80,26 @@ int fg_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int i
 int fg_log_softmax(const void* in, void* out, int64_t M, int64_t N, int64_t K, int in_dtype,
                int out_dtype, void* stream);
 
+/* Backward of softmax / log_softmax over the middle axis of contiguous [M, N, K] views, from the forward's
+ * OUTPUT: grad_in = out * (grad_out - sum(out * grad_out))  resp.  grad_out - exp(out) * sum(grad_out),
+ * fp32 arithmetic.  out and grad_out share `dtype`; grad_in_dtype equals it, or is a 16-bit type when
+ * `dtype` is FG_F32 (the forward widened its result).
+ * Replace softmax_backward_kernel_{inner,non_inner}, src/flag_gems/ops/softmax.py:163-280,321-355, and
+ * log_softmax_backward_kernel, src/flag_gems/ops/log_softmax.py:60-96,131-160. */
+int fg_softmax_backward(const void* out, const void* grad_out, void* grad_in, int64_t M, int64_t N,
+                        int64_t K, int dtype, int grad_in_dtype, void* stream);
+int fg_log_softmax_backward(const void* out, const void* grad_out, void* grad_in, int64_t M,
+                            int64_t N, int64_t K, int dtype, int grad_in_dtype, void* stream);
+
+/* Backward of rms_norm for contiguous x, dy, dx [M, N] and the inv_rms [M] that fg_rms_norm wrote:
+ * g = dy * w, xh = x * inv_rms, dx = (g - xh * mean(xh * g)) * inv_rms (w == NULL: ones).
+ * When dw_partial is non-NULL it receives, as fp32 [ceil(M / rows_per_block), N], the sums of
+ * x * dy * inv_rms over each block of rows; their column sum is the weight gradient.
+ * Replaces rms_norm_grad_dx_kernel and rms_norm_grad_dw_kernel, src/flag_gems/ops/rms_norm.py:54-146,171-218. */
+int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,
+                         float* dw_partial, int rows_per_block, int64_t M, int64_t N, int dtype,
+                         void* stream);
+
 /* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
  * {token, head, dim}); cos/sin [max_pos, D/2] with unit inner stride.  pos == NULL means
  * position = token_index % seq_len.  q_out/k_out may alias q/k (in-place).

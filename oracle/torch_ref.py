@@ -51,6 +51,29 @@ def log_softmax(x, dim):
     return torch.nn.functional.log_softmax(to_reference(x, True), dim=dim)
 
 
+def softmax_backward(grad, out, dim):
+    """tests/test_reduction_ops.py:533-557: aten::_softmax_backward_data on fp64 copies
+    (grad_in = out * (grad - sum(out * grad)))."""
+    g, y = to_reference(grad, True), to_reference(out, True)
+    return torch.ops.aten._softmax_backward_data(g, y, dim, g.dtype)
+
+
+def log_softmax_backward(grad, out, dim):
+    """tests/test_reduction_ops.py:487-503: aten::_log_softmax_backward_data on fp64 copies
+    (grad_in = grad - exp(out) * sum(grad))."""
+    g, y = to_reference(grad, True), to_reference(out, True)
+    return torch.ops.aten._log_softmax_backward_data(g, y, dim, g.dtype)
+
+
+def rms_norm_grads(x, weight, eps, grad):
+    """tests/test_norm_ops.py:539-559: autograd through weight * (x * rsqrt(mean(x^2) + eps)), here on fp64
+    copies.  Returns (dx, dweight)."""
+    xr = to_reference(x, True).clone().requires_grad_(True)
+    wr = to_reference(weight, True).clone().requires_grad_(True)
+    y = wr * (xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + eps))
+    return torch.autograd.grad(y, (xr, wr), to_reference(grad, True))
+
+
 def rms_norm(x, weight, eps):
     """tests/test_norm_ops.py:539-544: fp32 normalisation, cast to the input dtype, then the weight
     multiply (the test does not widen to fp64 for this operator)."""

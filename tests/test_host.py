@@ -43,7 +43,7 @@ def test_use_gems_registers_and_unregisters():
     before = _cuda_kernel_of("aten::mm")
     with flag_gems.use_gems():
         assert sorted(flag_gems.all_ops()) == sorted(
-            ["_flash_attention_forward", "_log_softmax", "_softmax", "addmm", "addmm.out", "bmm", "mm", "mm.out", "rms_norm"])
+            ["_flash_attention_forward", "_log_softmax", "_log_softmax_backward_data", "_softmax", "_softmax_backward_data", "addmm", "addmm.out", "bmm", "mm", "mm.out", "rms_norm"])
         inside = _cuda_kernel_of("aten::mm")
         assert "flaggems_amd" in inside
         assert "flaggems_amd" in _cuda_kernel_of("aten::rms_norm")

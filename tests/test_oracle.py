@@ -113,6 +113,62 @@ def test_log_softmax_pinned():
     assert O.log_softmax(w, -1)[0, 1] == float("-inf")
 
 
+def test_softmax_backward_pinned():
+    """Against the Jacobian written out element by element, and against central differences of the forward."""
+    import math
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(3, 5, generator=g, dtype=torch.float64)
+    dy = torch.randn(3, 5, generator=g, dtype=torch.float64)
+    y = torch.softmax(x, -1)
+    got = O.softmax_backward(dy, y, 1)
+    got_log = O.log_softmax_backward(dy, torch.log_softmax(x, -1), 1)
+    for r in range(3):
+        for i in range(5):
+            # d softmax_j / d x_i = y_j (delta_ij - y_i);  d log_softmax_j / d x_i = delta_ij - y_i
+            want = sum(float(dy[r, j]) * float(y[r, j]) * ((1.0 if i == j else 0.0) - float(y[r, i])) for j in range(5))
+            want_log = sum(float(dy[r, j]) * ((1.0 if i == j else 0.0) - float(y[r, i])) for j in range(5))
+            assert math.isclose(float(got[r, i]), want, abs_tol=1e-12)
+            assert math.isclose(float(got_log[r, i]), want_log, abs_tol=1e-12)
+    h = 1e-6
+    for i in range(5):
+        e = torch.zeros(3, 5, dtype=torch.float64); e[:, i] = h
+        fd = ((torch.softmax(x + e, -1) - torch.softmax(x - e, -1)) * dy).sum(-1) / (2 * h)
+        assert torch.allclose(got[:, i], fd, atol=1e-8)
+    # a middle axis is the same rule applied along that axis
+    y3 = torch.softmax(torch.randn(2, 4, 3, generator=g, dtype=torch.float64), 1)
+    d3 = torch.randn(2, 4, 3, generator=g, dtype=torch.float64)
+    assert torch.allclose(O.softmax_backward(d3, y3, 1), O.softmax_backward(d3.transpose(1, 2), y3.transpose(1, 2), 2).transpose(1, 2))
+    # gradients of a softmax sum to zero along the axis
+    assert torch.allclose(got.sum(-1), torch.zeros(3, dtype=torch.float64), atol=1e-12)
+
+
+def test_rms_norm_grads_pinned():
+    """Closed form dx = inv * (g - xh * mean(xh * g)), dw = sum over rows of dy * xh, and central differences."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(4, 6, generator=g, dtype=torch.float64)
+    w = torch.randn(6, generator=g, dtype=torch.float64)
+    dy = torch.randn(4, 6, generator=g, dtype=torch.float64)
+    eps = 1e-5
+    dx, dw = O.rms_norm_grads(x, w, eps, dy)
+    inv = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    xh, gg = x * inv, dy * w
+    assert torch.allclose(dx, inv * (gg - xh * (xh * gg).mean(-1, keepdim=True)), atol=1e-12)
+    assert torch.allclose(dw, (dy * xh).sum(0), atol=1e-12)
+
+    def f(xx, ww):
+        return float(((ww * (xx * torch.rsqrt(xx.pow(2).mean(-1, keepdim=True) + eps))) * dy).sum())
+
+    h = 1e-6
+    for (r, c) in ((0, 0), (2, 5), (3, 1)):
+        e = torch.zeros_like(x); e[r, c] = h
+        assert abs((f(x + e, w) - f(x - e, w)) / (2 * h) - float(dx[r, c])) < 1e-7
+    for c in (0, 3):
+        e = torch.zeros_like(w); e[c] = h
+        assert abs((f(x, w + e) - f(x, w - e)) / (2 * h) - float(dw[c])) < 1e-7
+    # the forward these gradients belong to is the oracle's forward
+    assert torch.allclose(w * xh, O.rms_norm(x, w, eps).double(), atol=1e-12)
+
+
 def test_softmax_invariants():
     x = torch.randn(6, 11, generator=torch.Generator().manual_seed(2))
     x[0, 3] = float("-inf"); x[2] = float("-inf")
