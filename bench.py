@@ -164,6 +164,47 @@ def main():
                     workload="fused_add_rms_norm [4096,4096] bf16, eps 1e-6 (configs[0] shape)",
                     cpu=(cpu, 4 * M * N * 4 + N * 4, "oracle fused_add_rms_norm (torch CPU, fp32 in / fp64 math) on the full [4096,4096]"))
 
+    def wl_softmax_backward():
+        torch.manual_seed(0)
+        M, N = 131072, 2048
+        y = torch.softmax(torch.randn(M, N, device=dev) * 2.0, -1).to(bf16)
+        g = torch.randn(M, N, device=dev).to(bf16)
+        state = {}
+
+        def run(i):
+            state["dx"] = flag_gems.softmax_backward(g, y, 1, bf16)
+
+        ys, gs = y[:16384].cpu(), g[:16384].cpu()
+
+        def cpu():
+            O.softmax_backward(gs, ys, 1)
+
+        return dict(run=run, work=3 * M * N * 2, bound="hbm", dtype="bf16",
+                    workload="softmax backward dim=-1 [131072,2048] bf16 (grad_out, out -> grad_in)",
+                    cpu=(cpu, 3 * 16384 * N * 2, "oracle softmax_backward (torch CPU, fp64 upcast) on the first 16384 rows"))
+
+    def wl_rms_norm_backward():
+        torch.manual_seed(0)
+        M, N = 16384, 4096
+        x = torch.randn(M, N).to(bf16).to(dev).requires_grad_(True)
+        w = (torch.rand(N) + 0.5).to(bf16).to(dev).requires_grad_(True)
+        dy = torch.randn(M, N).to(bf16).to(dev)
+        y = flag_gems.rms_norm(x, [N], w, 1e-6)
+        state = {}
+
+        def run(i):
+            state["g"] = torch.autograd.grad(y, (x, w), dy, retain_graph=True)
+
+        xs, ds, wc = x.detach()[:2048].cpu(), dy[:2048].cpu(), w.detach().cpu()
+
+        def cpu():
+            O.rms_norm_grads(xs, wc, 1e-6, ds)
+
+        return dict(run=run, work=3 * M * N * 2 + 2 * N * 2, bound="hbm", dtype="bf16",
+                    workload="rms_norm backward [16384,4096] bf16: dx and dweight through autograd "
+                             "(one kernel + the sum of its partial rows)",
+                    cpu=(cpu, 3 * 2048 * N * 2, "oracle rms_norm_grads (torch CPU autograd, fp64) on the first 2048 rows"))
+
     def wl_mm(M, N, K, name, b_t=False, bias=False, bound="mfma"):
         def make():
             torch.manual_seed(0)
@@ -385,6 +426,8 @@ def main():
     workloads = {
         "softmax_c2": wl_softmax_c2,
         "fused_add_rms_norm_c1": wl_fused_add_rms_norm_c1,
+        "softmax_backward": wl_softmax_backward,
+        "rms_norm_backward": wl_rms_norm_backward,
         "mm_c3a_8192": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B row-major (configs[2]a)"),
         "mm_c3a_8192_nt": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B = W^T column-major (configs[2]a, weight layout)", b_t=True),
         "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),

@@ -9,9 +9,15 @@
 // VEC elements per thread), so HBM is read once per input and written once.  Rows that do not fit,
 // or that defeat 16-byte access, use a looped kernel that reads the row twice (the second time from
 // L2).  Middle axis (softmax only, K > 1): one thread per (m, k) column, walking N with stride K.
-// The weight gradient of rms_norm is a column sum over all rows: a first kernel leaves one fp32
-// partial row per block of rows, the caller adds the partial rows up.
+// The weight gradient of rms_norm is a column sum over all rows.  The rms kernel therefore walks a
+// group of consecutive rows per workgroup and keeps the running column sums of x * inv_rms * dy for its
+// columns in registers; each group leaves one fp32 partial row and the caller adds the partial rows up.
+// x and dy are read once for both gradients (3 accesses per element instead of 5).
 #include "fg_common.h"
+
+namespace fgk {
+int num_cus(int device);  // gemm.hip
+}
 
 namespace {
 
@@ -38,12 +44,10 @@ template <typename T> __device__ __forceinline__ float exp_like_forward(float x)
   else return __expf(x);
 }
 
-// a: y (softmax modes) or x (rms); g: dy.  w and inv_rms are read in the rms mode only (w may be null).
+// softmax / log_softmax; a: the forward's output y, g: dy.
 template <typename TI, typename TO, int VEC, int ITERS, int TPR, int MODE>
 __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const TI* __restrict__ a,
                                                                           const TI* __restrict__ g,
-                                                                          const TI* __restrict__ w,
-                                                                          const float* __restrict__ inv_rms,
                                                                           TO* __restrict__ out, int64_t M, int N) {
   constexpr int BLOCK = TPR < 256 ? 256 : TPR;
   constexpr int RPB = BLOCK / TPR;
@@ -55,11 +59,6 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
   const bool row_ok = row < M;
   const TI* ar = a + row * (int64_t)N;
   const TI* gr = g + row * (int64_t)N;
-  float inv = 1.0f;
-  if constexpr (MODE == BWD_RMS) {
-    if (row_ok) inv = inv_rms[row];
-  }
-
   float va[ITERS][VEC], vg[ITERS][VEC];
   float s = 0.f;
 #pragma unroll
@@ -68,22 +67,11 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
     if (row_ok && col < N) {
       const Pack<TI, VEC> pa = ld_pack_nt<TI, VEC>(ar + col);
       const Pack<TI, VEC> pg = ld_pack_nt<TI, VEC>(gr + col);
-      if constexpr (MODE == BWD_RMS) {
-        Pack<TI, VEC> pw;
-        if (w != nullptr) pw = ld_pack<TI, VEC>(w + col);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          va[j][e] = (float)pa.v[e] * inv;
-          vg[j][e] = w != nullptr ? (float)pg.v[e] * (float)pw.v[e] : (float)pg.v[e];
-          s += va[j][e] * vg[j][e];
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          va[j][e] = (float)pa.v[e];
-          vg[j][e] = (float)pg.v[e];
-          s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
-        }
+      for (int e = 0; e < VEC; ++e) {
+        va[j][e] = (float)pa.v[e];
+        vg[j][e] = (float)pg.v[e];
+        s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
       }
     } else {
 #pragma unroll
@@ -92,7 +80,6 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
   }
   s = row_sum<TPR>(s, smem, row_in_block, t);
   if (!row_ok) return;
-  const float mean = s / (float)N;
   TO* orow = out + row * (int64_t)N;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
@@ -103,11 +90,97 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
       for (int e = 0; e < VEC; ++e) {
         float r;
         if constexpr (MODE == BWD_SOFTMAX) r = va[j][e] * (vg[j][e] - s);
-        else if constexpr (MODE == BWD_LOG_SOFTMAX) r = vg[j][e] - exp_like_forward<TI>(va[j][e]) * s;
-        else r = (vg[j][e] - va[j][e] * mean) * inv;
+        else r = vg[j][e] - exp_like_forward<TI>(va[j][e]) * s;
         po.v[e] = (TO)r;
       }
       st_pack_nt<TO, VEC>(orow + col, po);
+    }
+  }
+}
+
+// rms_norm: dx for the rows of one group, and the group's column sums for the weight gradient.
+// Group = rows [group * rows_per_group, ...); a block holds RPB groups (one per TPR threads).  Every thread
+// of a block runs the same number of iterations, so the barriers inside row_sum are uniform.
+template <typename T, int VEC, int ITERS, int TPR>
+__global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_bwd_rows_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ w, const float* __restrict__ inv_rms,
+    T* __restrict__ dx, float* __restrict__ dw_partial, int64_t partial_rows, int64_t M, int N, int rows_per_group) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ float smem[BLOCK / 64];
+  const int tid = threadIdx.x;
+  const int row_in_block = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t group = (int64_t)blockIdx.x * RPB + row_in_block;
+  const int64_t r0 = group * rows_per_group;
+
+  float wv[ITERS][VEC], acc[ITERS][VEC];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    if (w != nullptr && col < N) {
+      const Pack<T, VEC> pw = ld_pack<T, VEC>(w + col);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) wv[j][e] = (float)pw.v[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) wv[j][e] = 1.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[j][e] = 0.f;
+  }
+
+  for (int i = 0; i < rows_per_group; ++i) {
+    const int64_t row = r0 + i;
+    const bool row_ok = row < M;
+    const float inv = row_ok ? inv_rms[row] : 0.f;
+    float xh[ITERS][VEC], d[ITERS][VEC];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      if (row_ok && col < N) {
+        const Pack<T, VEC> px = ld_pack_nt<T, VEC>(x + row * (int64_t)N + col);
+        const Pack<T, VEC> pd = ld_pack_nt<T, VEC>(dy + row * (int64_t)N + col);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          xh[j][e] = (float)px.v[e] * inv;
+          d[j][e] = (float)pd.v[e];
+          s += xh[j][e] * d[j][e] * wv[j][e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xh[j][e] = d[j][e] = 0.f;
+      }
+    }
+    s = row_sum<TPR>(s, smem, row_in_block, t);
+    const float mean = s / (float)N;
+    if (row_ok) {
+#pragma unroll
+      for (int j = 0; j < ITERS; ++j) {
+        const int col = (j * TPR + t) * VEC;
+        if (col < N) {
+          Pack<T, VEC> po;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            po.v[e] = (T)((d[j][e] * wv[j][e] - xh[j][e] * mean) * inv);
+            acc[j][e] += xh[j][e] * d[j][e];
+          }
+          st_pack_nt<T, VEC>(dx + row * (int64_t)N + col, po);
+        }
+      }
+    }
+  }
+  if (dw_partial != nullptr && group < partial_rows) {
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      if (col < N) {
+        Pack<float, VEC> pa;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) pa.v[e] = acc[j][e];
+        st_pack<float, VEC>(dw_partial + group * (int64_t)N + col, pa);
+      }
     }
   }
 }
@@ -179,28 +252,27 @@ __global__ __launch_bounds__(256) void rms_dw_partial_kernel(const T* __restrict
 }
 
 template <typename TI, typename TO, int VEC, int ITERS, int TPR, int MODE>
-void launch_rows(const TI* a, const TI* g, const TI* w, const float* inv_rms, TO* out, int64_t M, int N,
-                 hipStream_t st) {
+void launch_rows(const TI* a, const TI* g, TO* out, int64_t M, int N, hipStream_t st) {
   constexpr int BLOCK = TPR < 256 ? 256 : TPR;
   constexpr int RPB = BLOCK / TPR;
   hipLaunchKernelGGL((bwd_rows_kernel<TI, TO, VEC, ITERS, TPR, MODE>), dim3((unsigned)fg_cdiv(M, RPB)), dim3(BLOCK), 0,
-                     st, a, g, w, inv_rms, out, M, N);
+                     st, a, g, out, M, N);
 }
 
-// Inner-axis dispatch shared by the three modes.  The caller has checked sizes and pointers.
+// Inner-axis dispatch of the softmax modes.  The caller has checked sizes and pointers.
 template <typename TI, typename TO, int MODE>
-int bwd_rows_dispatch(const TI* a, const TI* g, const TI* w, const float* inv_rms, TO* out, int64_t M, int64_t N,
-                      hipStream_t st, const char* what) {
+int bwd_rows_dispatch(const TI* a, const TI* g, TO* out, int64_t M, int64_t N, hipStream_t st, const char* what) {
   FG_REQUIRE(M < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "%s: M=%lld exceeds the grid limit", what, (long long)M);
   constexpr int VEC = 16 / sizeof(TI);
-  const bool vec_ok = (N % VEC == 0) && fg_aligned(a, 16) && fg_aligned(g, 16) && fg_aligned(out, sizeof(TO) * VEC) &&
-                      (w == nullptr || fg_aligned(w, 16));
+  const bool vec_ok = (N % VEC == 0) && fg_aligned(a, 16) && fg_aligned(g, 16) && fg_aligned(out, sizeof(TO) * VEC);
   const int64_t packs = vec_ok ? N / VEC : 0;
-#define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, MODE>(a, g, w, inv_rms, out, M, (int)N, st)
+#define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, MODE>(a, g, out, M, (int)N, st)
   // two input streams: one pack per thread from each, as in the fused add + norm forward
-  if (!vec_ok || packs > 2048) {
-    hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE>), dim3((unsigned)M), dim3(256), 0, st, a, g, w, inv_rms, out, M,
-                       N);
+  if (!vec_ok || packs > 4096) {
+    hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE>), dim3((unsigned)M), dim3(256), 0, st, a, g, (const TI*)nullptr,
+                       (const float*)nullptr, out, M, N);
+  } else if (packs > 2048) {
+    FG_ROWS(4, 1024);  // vocabulary-sized rows (32000 16-bit elements)
   } else if (packs <= 64) {
     FG_ROWS(1, 64);
   } else if (packs <= 128) {
@@ -218,6 +290,52 @@ int bwd_rows_dispatch(const TI* a, const TI* g, const TI* w, const float* inv_rm
   return fg_check_launch(what);
 }
 
+// Threads per row of the rms kernel for a row of `packs` 16-byte packs (at most 2048).
+int rms_bwd_tpr(int64_t packs) { return packs <= 64 ? 64 : packs <= 128 ? 128 : packs <= 256 ? 256 : packs <= 512 ? 512 : 1024; }
+
+template <typename T, int VEC, int ITERS, int TPR>
+void launch_rms_rows(const T* x, const T* dy, const T* w, const float* inv_rms, T* dx, float* dw_partial,
+                     int64_t partial_rows, int64_t M, int N, int rows_per_group, hipStream_t st) {
+  constexpr int BLOCK = TPR < 256 ? 256 : TPR;
+  constexpr int RPB = BLOCK / TPR;
+  // every partial row gets written (groups past the last row write zeros); without partial rows one row per group
+  const int64_t groups = dw_partial != nullptr ? partial_rows : fg_cdiv(M, rows_per_group);
+  hipLaunchKernelGGL((rms_bwd_rows_kernel<T, VEC, ITERS, TPR>), dim3((unsigned)fg_cdiv(groups, RPB)), dim3(BLOCK), 0, st,
+                     x, dy, w, inv_rms, dx, dw_partial, partial_rows, M, N, rows_per_group);
+}
+
+// dw_partial (may be null) has partial_rows rows of N floats; every one of them is written.
+template <typename T>
+int rms_bwd_dispatch(const T* x, const T* dy, const T* w, const float* inv_rms, T* dx, float* dw_partial,
+                     int64_t partial_rows, int64_t M, int64_t N, hipStream_t st) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec_ok = (N % VEC == 0) && fg_aligned(x, 16) && fg_aligned(dy, 16) && fg_aligned(dx, 16) &&
+                      (w == nullptr || fg_aligned(w, 16)) && (dw_partial == nullptr || fg_aligned(dw_partial, 32));
+  const int64_t packs = vec_ok ? N / VEC : 0;
+  // rows summed into one partial row: with partial_rows groups of that many rows all M rows are covered
+  const int64_t rows_per_group = dw_partial != nullptr ? fg_cdiv(M, partial_rows) : 1;
+  if (!vec_ok || packs > 2048) {
+    hipLaunchKernelGGL((bwd_looped_kernel<T, T, BWD_RMS>), dim3((unsigned)M), dim3(256), 0, st, x, dy, w, inv_rms, dx, M,
+                       N);
+    if (dw_partial != nullptr)
+      hipLaunchKernelGGL((rms_dw_partial_kernel<T>), dim3((unsigned)partial_rows, (unsigned)fg_cdiv(N, 256)), dim3(256),
+                         0, st, x, dy, inv_rms, dw_partial, M, N, (int)rows_per_group);
+    return fg_check_launch("rms_norm_backward");
+  }
+#define FG_ROWS(ITERS, TPR)   launch_rms_rows<T, VEC, ITERS, TPR>(x, dy, w, inv_rms, dx, dw_partial, partial_rows, M, (int)N, (int)rows_per_group, st)
+  switch (rms_bwd_tpr(packs)) {
+    case 64: FG_ROWS(1, 64); break;
+    case 128: FG_ROWS(1, 128); break;
+    case 256: FG_ROWS(1, 256); break;
+    case 512: FG_ROWS(1, 512); break;
+    default:
+      if (packs <= 1024) FG_ROWS(1, 1024);
+      else FG_ROWS(2, 1024);
+  }
+#undef FG_ROWS
+  return fg_check_launch("rms_norm_backward");
+}
+
 template <typename TI, typename TO, int MODE>
 int softmax_bwd_dispatch(const TI* y, const TI* g, TO* out, int64_t M, int64_t N, int64_t K, hipStream_t st,
                          const char* what) {
@@ -228,7 +346,7 @@ int softmax_bwd_dispatch(const TI* y, const TI* g, TO* out, int64_t M, int64_t N
                        st, y, g, out, M, N, K);
     return fg_check_launch(what);
   }
-  return bwd_rows_dispatch<TI, TO, MODE>(y, g, nullptr, nullptr, out, M, N, st, what);
+  return bwd_rows_dispatch<TI, TO, MODE>(y, g, out, M, N, st, what);
 }
 
 template <int MODE>
@@ -267,35 +385,42 @@ extern "C" int fg_log_softmax_backward(const void* out, const void* grad_out, vo
   return softmax_bwd_entry<BWD_LOG_SOFTMAX>(out, grad_out, grad_in, M, N, K, dtype, grad_in_dtype, stream);
 }
 
+extern "C" int64_t fg_rms_norm_backward_partial_rows(int64_t M, int64_t N, int dtype, int device) {
+  if (M <= 0 || N <= 0) return 0;
+  const int64_t vec = dtype == FG_F32 ? 4 : 8;
+  if (N % vec != 0 || N / vec > 2048) return fg_cdiv(M, 64);
+  const int tpr = rms_bwd_tpr(N / vec);
+  const int block = tpr < 256 ? 256 : tpr;
+  // enough groups to give every CU its 2048 threads once, 8 to 64 rows each
+  const int64_t target = (int64_t)fgk::num_cus(device) * (2048 / block) * (block / tpr);
+  int64_t rows_per_group = fg_cdiv(M, target);
+  rows_per_group = rows_per_group < 8 ? 8 : rows_per_group > 64 ? 64 : rows_per_group;
+  return fg_cdiv(M, rows_per_group);
+}
+
 extern "C" int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,
-                                    float* dw_partial, int rows_per_block, int64_t M, int64_t N, int dtype,
+                                    float* dw_partial, int64_t partial_rows, int64_t M, int64_t N, int dtype,
                                     void* stream) {
   FG_REQUIRE(M >= 0 && N >= 0, FG_ERR_INVALID, "rms_norm_backward: negative size");
   if (M == 0 || N == 0) return FG_OK;
   FG_REQUIRE(x && dy && inv_rms && dx, FG_ERR_INVALID, "rms_norm_backward: null pointer");
-  FG_REQUIRE(N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "rms_norm_backward: N=%lld too large", (long long)N);
-  FG_REQUIRE(dw_partial == nullptr || rows_per_block > 0, FG_ERR_INVALID,
-             "rms_norm_backward: rows_per_block must be positive");
+  FG_REQUIRE(M < ((int64_t)1 << 31) && N < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED,
+             "rms_norm_backward: extent exceeds 2^31");
+  FG_REQUIRE(dw_partial == nullptr || (partial_rows >= 1 && partial_rows <= M), FG_ERR_INVALID,
+             "rms_norm_backward: partial_rows=%lld must lie in [1, M]", (long long)partial_rows);
+  FG_REQUIRE(fg_cdiv(N, 256) < 65536, FG_ERR_UNSUPPORTED, "rms_norm_backward: N=%lld too large", (long long)N);
   hipStream_t st = (hipStream_t)stream;
-  int rc = FG_ERR_INVALID;
-  const int64_t row_blocks = dw_partial ? fg_cdiv(M, rows_per_block) : 0;
-  FG_REQUIRE(row_blocks < ((int64_t)1 << 31) && fg_cdiv(N, 256) < 65536, FG_ERR_UNSUPPORTED,
-             "rms_norm_backward: problem too large for the weight-gradient grid");
-#define FG_CASE(D, T)                                                                                               \
-  if (dtype == D) {                                                                                                 \
-    rc = bwd_rows_dispatch<T, T, BWD_RMS>((const T*)x, (const T*)dy, (const T*)w, inv_rms, (T*)dx, M, N, st,        \
-                                          "rms_norm_backward");                                                     \
-    if (rc == FG_OK && dw_partial != nullptr) {                                                                     \
-      hipLaunchKernelGGL((rms_dw_partial_kernel<T>), dim3((unsigned)row_blocks, (unsigned)fg_cdiv(N, 256)), dim3(256), \
-                         0, st, (const T*)x, (const T*)dy, inv_rms, dw_partial, M, N, rows_per_block);              \
-      rc = fg_check_launch("rms_norm_backward(dw)");                                                                \
-    }                                                                                                               \
-    return rc;                                                                                                      \
+  switch (dtype) {
+    case FG_F16:
+      return rms_bwd_dispatch<f16_t>((const f16_t*)x, (const f16_t*)dy, (const f16_t*)w, inv_rms, (f16_t*)dx, dw_partial,
+                                     partial_rows, M, N, st);
+    case FG_BF16:
+      return rms_bwd_dispatch<bf16_t>((const bf16_t*)x, (const bf16_t*)dy, (const bf16_t*)w, inv_rms, (bf16_t*)dx,
+                                      dw_partial, partial_rows, M, N, st);
+    case FG_F32:
+      return rms_bwd_dispatch<float>((const float*)x, (const float*)dy, (const float*)w, inv_rms, (float*)dx, dw_partial,
+                                     partial_rows, M, N, st);
   }
-  FG_CASE(FG_F16, f16_t)
-  FG_CASE(FG_BF16, bf16_t)
-  FG_CASE(FG_F32, float)
-#undef FG_CASE
   fg_set_error("rms_norm_backward: unsupported dtype %d", dtype);
   return FG_ERR_INVALID;
 }

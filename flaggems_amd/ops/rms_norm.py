@@ -9,10 +9,6 @@ from .. import _C
 
 logger = logging.getLogger("flag_gems.ops.rms_norm")
 
-# rows summed by one workgroup of the weight-gradient kernel before the partial rows are added up
-_DW_ROWS_PER_BLOCK = 64
-
-
 def _composite(x, normalized_shape, weight, eps):
     # plain tensor math: used when the dtype has no kernel
     dims = tuple(range(x.ndim - len(normalized_shape), x.ndim))
@@ -48,9 +44,9 @@ def _forward(x, normalized_shape, weight, eps, want_inv_rms):
 
 
 class RmsNorm(torch.autograd.Function):
-    """Forward saves x and the per-row 1/rms; backward is one row-wise kernel for dx and, when the weight
-    needs a gradient, one column-sum kernel whose fp32 partial rows are added up by torch.sum (the split of
-    src/flag_gems/ops/rms_norm.py:149-218)."""
+    """Forward saves x and the per-row 1/rms; backward is one kernel that writes dx and, when the weight needs
+    a gradient, fp32 partial column sums (one row per group of rows) that torch.sum adds up (the reference
+    uses a kernel per gradient, src/flag_gems/ops/rms_norm.py:149-218)."""
 
     @staticmethod
     def forward(ctx, x, normalized_shape, weight, eps):
@@ -76,14 +72,15 @@ class RmsNorm(torch.autograd.Function):
         want_dw = weight is not None and ctx.needs_input_grad[2]
         if M == 0 or N == 0:
             return dx, None, (torch.zeros_like(weight) if want_dw else None), None
-        partial = None
+        partial, partial_rows = None, 0
+        lib = _C.lib()
         if want_dw:
-            row_blocks = (M + _DW_ROWS_PER_BLOCK - 1) // _DW_ROWS_PER_BLOCK
-            partial = torch.empty((row_blocks, N), dtype=torch.float32, device=x.device)
+            partial_rows = lib.fg_rms_norm_backward_partial_rows(M, N, _C.dtype_id(x.dtype), x.device.index or 0)
+            partial = torch.empty((partial_rows, N), dtype=torch.float32, device=x.device)
         with _C.device_guard(x.device):
-            rc = _C.lib().fg_rms_norm_backward(
+            rc = lib.fg_rms_norm_backward(
                 x.data_ptr(), dy.data_ptr(), inv_rms.data_ptr(), w.data_ptr() if w is not None else None,
-                dx.data_ptr(), partial.data_ptr() if partial is not None else None, _DW_ROWS_PER_BLOCK,
+                dx.data_ptr(), partial.data_ptr() if partial is not None else None, partial_rows,
                 M, N, _C.dtype_id(x.dtype), _C.current_stream(x.device),
             )
         _C.check(rc, "fg_rms_norm_backward")

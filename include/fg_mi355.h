@@ -93,11 +93,14 @@ int fg_log_softmax_backward(const void* out, const void* grad_out, void* grad_in
 
 /* Backward of rms_norm for contiguous x, dy, dx [M, N] and the inv_rms [M] that fg_rms_norm wrote:
  * g = dy * w, xh = x * inv_rms, dx = (g - xh * mean(xh * g)) * inv_rms (w == NULL: ones).
- * When dw_partial is non-NULL it receives, as fp32 [ceil(M / rows_per_block), N], the sums of
- * x * dy * inv_rms over each block of rows; their column sum is the weight gradient.
+ * When dw_partial is non-NULL it is fp32 [partial_rows, N], 32-byte aligned, 1 <= partial_rows <= M: row p
+ * receives the sums of x * dy * inv_rms over rows [p * ceil(M / partial_rows), ...); the column sum of
+ * dw_partial is the weight gradient.  fg_rms_norm_backward_partial_rows proposes a partial_rows that fills
+ * the device.  One kernel computes both gradients (x and dy are read once).
  * Replaces rms_norm_grad_dx_kernel and rms_norm_grad_dw_kernel, src/flag_gems/ops/rms_norm.py:54-146,171-218. */
+int64_t fg_rms_norm_backward_partial_rows(int64_t M, int64_t N, int dtype, int device);
 int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,
-                         float* dw_partial, int rows_per_block, int64_t M, int64_t N, int dtype,
+                         float* dw_partial, int64_t partial_rows, int64_t M, int64_t N, int dtype,
                          void* stream);
 
 /* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
