@@ -16,7 +16,7 @@ for _name in ("config", "fused", "logging_utils", "modules", "ops", "patches", "
 sys.modules[__name__ + ".runtime.register"] = _impl.runtime.register
 for _sub in ("mm", "addmm", "bmm", "softmax", "log_softmax", "rms_norm", "attention"):
     sys.modules[__name__ + ".ops." + _sub] = sys.modules["flaggems_amd.ops." + _sub]
-for _sub in ("fused_add_rms_norm", "reshape_and_cache_flash", "rotary_embedding", "silu_and_mul"):
+for _sub in ("fused_add_rms_norm", "reshape_and_cache", "reshape_and_cache_flash", "rotary_embedding", "silu_and_mul"):
     sys.modules[__name__ + ".fused." + _sub] = sys.modules["flaggems_amd.fused." + _sub]
 for _sub in ("activation", "normalization", "rotary_embedding"):
     sys.modules[__name__ + ".modules." + _sub] = sys.modules["flaggems_amd.modules." + _sub]

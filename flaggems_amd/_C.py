@@ -89,6 +89,10 @@ _SIGNATURES = {
         c_int,
         [c_vp, c_vp, c_vp, c_vp, c_vp, c_int, c_i64, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_int, c_vp],
     ),
+    "fg_reshape_and_cache": (
+        c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_vp, c_int, c_i64, c_int, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_int, c_vp],
+    ),
     "fg_silu_and_mul": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
     "fg_softmax_backward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),
     "fg_log_softmax_backward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),

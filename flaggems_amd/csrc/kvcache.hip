@@ -1,4 +1,4 @@
-// reshape_and_cache_flash for gfx950: scatter of K and V token rows into the paged caches.
+// reshape_and_cache_flash and reshape_and_cache for gfx950: scatter of K and V token rows into the paged caches.
 //
 // One wave copies one (token, tensor) row of n = H*D elements: lanes stride through the row in
 // 16-byte pieces, so both the gather side (token stride arbitrary) and the scatter side (slot
@@ -62,7 +62,73 @@ int cache_dispatch(const void* key, const void* value, void* kc, void* vc, const
   return fg_check_launch("reshape_and_cache_flash");
 }
 
+// The older cache layout: key_cache [blocks, H, D/x, block_size, x], value_cache [blocks, H, D, block_size]
+// (x elements = 16 bytes of one head stay together in the key cache; the value cache is transposed so that
+// the tokens of a page are contiguous per feature).  One workgroup per token, one element per thread and
+// step: the value side is a scatter of single elements by construction.
+template <typename U, typename SLOT>
+__global__ __launch_bounds__(256) void cache_scatter_v0_kernel(const U* __restrict__ key, const U* __restrict__ value,
+                                                              U* __restrict__ kc, U* __restrict__ vc,
+                                                              const SLOT* __restrict__ slots, int H, int D,
+                                                              int block_size, int x, int64_t num_blocks,
+                                                              int64_t key_stride, int64_t value_stride) {
+  const int64_t tok = blockIdx.x;
+  const int64_t slot = (int64_t)slots[tok];
+  if (slot < 0) return;  // padding token
+  const int64_t blk = slot / block_size;
+  if (blk >= num_blocks) return;  // a slot outside the cache is dropped rather than written somewhere
+  const int64_t off = slot - blk * block_size;
+  const int n = H * D, dx = D / x;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int head = i / D, ho = i - head * D;
+    const int xi = ho / x, xo = ho - xi * x;
+    kc[(((blk * H + head) * dx + xi) * block_size + off) * x + xo] = key[tok * key_stride + i];
+    vc[((blk * H + head) * D + ho) * block_size + off] = value[tok * value_stride + i];
+  }
+}
+
+template <typename U>
+int cache_v0_launch(const void* key, const void* value, void* kc, void* vc, const void* slots, int slot_is_i64,
+                    int64_t num_tokens, int H, int D, int block_size, int x, int64_t num_blocks, int64_t key_stride,
+                    int64_t value_stride, hipStream_t st) {
+  if (slot_is_i64)
+    hipLaunchKernelGGL((cache_scatter_v0_kernel<U, int64_t>), dim3((unsigned)num_tokens), dim3(256), 0, st, (const U*)key,
+                       (const U*)value, (U*)kc, (U*)vc, (const int64_t*)slots, H, D, block_size, x, num_blocks,
+                       key_stride, value_stride);
+  else
+    hipLaunchKernelGGL((cache_scatter_v0_kernel<U, int32_t>), dim3((unsigned)num_tokens), dim3(256), 0, st, (const U*)key,
+                       (const U*)value, (U*)kc, (U*)vc, (const int32_t*)slots, H, D, block_size, x, num_blocks,
+                       key_stride, value_stride);
+  return fg_check_launch("reshape_and_cache");
+}
+
 }  // namespace
+
+extern "C" int fg_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                                    const void* slot_mapping, int slot_is_i64, int64_t num_tokens, int H, int D,
+                                    int block_size, int x, int64_t num_blocks, int64_t key_stride,
+                                    int64_t value_stride, int elem_bytes, void* stream) {
+  FG_REQUIRE(num_tokens >= 0 && H >= 0 && D >= 0 && num_blocks >= 0, FG_ERR_INVALID, "reshape_and_cache: negative size");
+  FG_REQUIRE(block_size > 0 && x > 0, FG_ERR_INVALID, "reshape_and_cache: block_size and x must be positive");
+  FG_REQUIRE(D % x == 0, FG_ERR_INVALID, "reshape_and_cache: head size %d is not a multiple of x = %d", D, x);
+  FG_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4, FG_ERR_INVALID,
+             "reshape_and_cache: element size %d", elem_bytes);
+  if (num_tokens == 0 || (int64_t)H * D == 0 || num_blocks == 0) return FG_OK;
+  FG_REQUIRE(key && value && key_cache && value_cache && slot_mapping, FG_ERR_INVALID, "reshape_and_cache: null pointer");
+  FG_REQUIRE(num_tokens < ((int64_t)1 << 31) && (int64_t)H * D < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED,
+             "reshape_and_cache: problem too large for one launch");
+  FG_REQUIRE(key_stride >= (int64_t)H * D && value_stride >= (int64_t)H * D, FG_ERR_INVALID,
+             "reshape_and_cache: token stride smaller than a token (%d x %d)", H, D);
+  hipStream_t st = (hipStream_t)stream;
+  if (elem_bytes == 2)
+    return cache_v0_launch<uint16_t>(key, value, key_cache, value_cache, slot_mapping, slot_is_i64, num_tokens, H, D,
+                                     block_size, x, num_blocks, key_stride, value_stride, st);
+  if (elem_bytes == 4)
+    return cache_v0_launch<uint32_t>(key, value, key_cache, value_cache, slot_mapping, slot_is_i64, num_tokens, H, D,
+                                     block_size, x, num_blocks, key_stride, value_stride, st);
+  return cache_v0_launch<uint8_t>(key, value, key_cache, value_cache, slot_mapping, slot_is_i64, num_tokens, H, D,
+                                  block_size, x, num_blocks, key_stride, value_stride, st);
+}
 
 extern "C" int fg_reshape_and_cache_flash(const void* key, const void* value, void* key_cache, void* value_cache,
                                           const void* slot_mapping, int slot_is_i64, int64_t num_tokens, int H, int D,

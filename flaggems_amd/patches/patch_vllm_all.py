@@ -2,9 +2,9 @@
 (reference: src/flag_gems/patches/patch_vllm_all.py:9-368).
 
 Installed: RMSNorm.forward_cuda, RotaryEmbedding.forward_cuda, SiluAndMul.forward_cuda, the v1
-FlashAttentionImpl.forward and the `_C::silu_and_mul` kernel.  The reference also replaces the MLA decode,
-the vLLM-v0 paged-cache write, two MoE routing kernels and the FA3 scheduler-metadata op; those are not
-operators of this package and stay on vLLM's own kernels.
+FlashAttentionImpl.forward, PagedAttention.write_to_paged_cache and the `_C::silu_and_mul` kernel.  The
+reference also replaces the MLA decode, two MoE routing kernels and the FA3 scheduler-metadata op; those are
+not operators of this package and stay on vLLM's own kernels.
 """
 from typing import Optional, Tuple
 
@@ -14,7 +14,6 @@ from .patch_util import patch_module_method, patch_vllm_lib
 
 # what apply_gems_patches_to_vllm() leaves alone, for its report
 _LEFT_ON_VLLM = (
-    "PagedAttention.write_to_paged_cache",
     "TritonMLAImpl._forward_decode",
     "torch.ops._moe_C.moe_align_block_size",
     "torch.ops._moe_C.topk_softmax",
@@ -74,6 +73,14 @@ def custom_silu_and_mul(out: torch.Tensor, input: torch.Tensor):
     silu_and_mul_out(input[..., :d], input[..., d:], out)
 
 
+def custom_gems_write_to_paged_cache(key, value, key_cache, value_cache, slot_mapping, kv_cache_dtype, k_scale, v_scale):
+    """PagedAttention.write_to_paged_cache (a static method of the v0 backend): K/V rows into the
+    [blocks, heads, head_size / x, block_size, x] / [blocks, heads, head_size, block_size] caches."""
+    from ..fused.reshape_and_cache import reshape_and_cache
+
+    reshape_and_cache(key, value, key_cache, value_cache, slot_mapping.flatten(), kv_cache_dtype, k_scale, v_scale)
+
+
 def custom_gems_flash_attention_impl_forward(
     self,
     layer: torch.nn.Module,
@@ -131,6 +138,7 @@ def custom_gems_flash_attention_impl_forward(
 def apply_gems_patches_to_vllm(verbose=True):
     """Install the replacements above into an importable vLLM (raises ImportError without one)."""
     import vllm  # noqa: F401
+    from vllm.attention.ops.paged_attn import PagedAttention
     from vllm.model_executor.layers.activation import SiluAndMul
     from vllm.model_executor.layers.layernorm import RMSNorm
     from vllm.model_executor.layers.rotary_embedding import RotaryEmbedding
@@ -138,6 +146,7 @@ def apply_gems_patches_to_vllm(verbose=True):
 
     patch_module_method(RMSNorm, "forward_cuda", custom_gems_rms_forward_cuda, verbose)
     patch_module_method(RotaryEmbedding, "forward_cuda", custom_gems_rope_forward_cuda, verbose)
+    patch_module_method(PagedAttention, "write_to_paged_cache", custom_gems_write_to_paged_cache, verbose)
     patch_module_method(SiluAndMul, "forward_cuda", custom_gems_silu_and_mul, verbose)
     patch_module_method(FlashAttentionImpl, "forward", custom_gems_flash_attention_impl_forward, verbose)
     patch_vllm_lib("_C", "silu_and_mul", custom_silu_and_mul, "CUDA", verbose)

@@ -126,6 +126,16 @@ int fg_reshape_and_cache_flash(const void* key, const void* value, void* key_cac
                                int64_t key_stride, int64_t value_stride, int64_t block_stride,
                                int elem_bytes, void* stream);
 
+/* The same scatter into the older cache layout: key_cache [num_blocks, H, D/x, block_size, x] and
+ * value_cache [num_blocks, H, D, block_size], both contiguous; key/value [num_tokens, H, D] with a dense
+ * [H, D] block per token and the given token strides (elements).  Slots < 0 and slots past the last block
+ * are skipped.  Bit-exact copy of elem_bytes-sized elements.
+ * Replaces reshape_and_cache_kernel, src/flag_gems/fused/reshape_and_cache.py:12-112. */
+int fg_reshape_and_cache(const void* key, const void* value, void* key_cache, void* value_cache,
+                         const void* slot_mapping, int slot_is_i64, int64_t num_tokens, int H, int D,
+                         int block_size, int x, int64_t num_blocks, int64_t key_stride,
+                         int64_t value_stride, int elem_bytes, void* stream);
+
 /* out[r,c] = silu(a[r,c]) * b[r,c] (fp32 arithmetic), rows of unit inner stride.
  * Replaces silu_and_mul_kernel, src/flag_gems/fused/silu_and_mul.py:12-17,47-53. */
 int fg_silu_and_mul(const void* a, const void* b, void* out, int64_t rows, int64_t cols,

@@ -266,6 +266,22 @@ def reshape_and_cache_flash(key, value, key_cache, value_cache, slot_mapping):
     return kc, vc
 
 
+def reshape_and_cache(key, value, key_cache, value_cache, slot_mapping):
+    """tests/test_attention_ops.py:1304-1315: python loop scatter into key_cache
+    [blocks, heads, head_size / x, block_size, x] and value_cache [blocks, heads, head_size, block_size].
+    Returns updated clones."""
+    key, value = to_reference(key), to_reference(value)
+    kc, vc = to_reference(key_cache).clone(), to_reference(value_cache).clone()
+    block_size = kc.shape[3]
+    reshaped_key = key.reshape(key.shape[0], *kc[0, :, :, 0, :].shape)
+    for i, s in enumerate(to_reference(slot_mapping).tolist()):
+        if s < 0:
+            continue
+        kc[s // block_size, :, :, s % block_size, :] = reshaped_key[i]
+        vc[s // block_size, :, :, s % block_size] = value[i]
+    return kc, vc
+
+
 def gems_tolerance(dtype, reduce_dim=1, atol=1e-4):
     """(atol, rtol) of src/flag_gems/testing/__init__.py:41-49."""
     rtol = {torch.float16: 1e-3, torch.bfloat16: 0.016, torch.float32: 1.3e-6, torch.float64: 1e-7}[dtype]

@@ -113,6 +113,34 @@ def test_log_softmax_pinned():
     assert O.log_softmax(w, -1)[0, 1] == float("-inf")
 
 
+def test_reshape_and_cache_v0_layout_pinned():
+    """Element by element against the index formula of the layout: key element (head h, feature f) of the token
+    in slot s sits at key_cache[s // bs, h, f // x, s % bs, f % x], value at value_cache[s // bs, h, f, s % bs]."""
+    g = torch.Generator().manual_seed(21)
+    T, H, D, bs, nb, x = 5, 3, 8, 4, 6, 4
+    key = torch.randn(T, H, D, generator=g); value = torch.randn(T, H, D, generator=g)
+    kc = torch.randn(nb, H, D // x, bs, x, generator=g); vc = torch.randn(nb, H, D, bs, generator=g)
+    slots = torch.tensor([7, -1, 0, 23, 12])
+    nk, nv = O.reshape_and_cache(key, value, kc, vc, slots)
+    touched_k = torch.zeros_like(kc, dtype=torch.bool); touched_v = torch.zeros_like(vc, dtype=torch.bool)
+    for t, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        for h in range(H):
+            for f in range(D):
+                assert nk[s // bs, h, f // x, s % bs, f % x] == key[t, h, f]
+                assert nv[s // bs, h, f, s % bs] == value[t, h, f]
+                touched_k[s // bs, h, f // x, s % bs, f % x] = True
+                touched_v[s // bs, h, f, s % bs] = True
+    assert torch.equal(nk[~touched_k], kc[~touched_k]) and torch.equal(nv[~touched_v], vc[~touched_v])
+    assert int(touched_k.sum()) == 4 * H * D
+    # the same tokens through the flash layout land in the same (block, offset, head, feature) cells
+    fk, fv = O.reshape_and_cache_flash(key, value, torch.zeros(nb, bs, H, D), torch.zeros(nb, bs, H, D), slots)
+    zk, zv = O.reshape_and_cache(key, value, torch.zeros_like(kc), torch.zeros_like(vc), slots)
+    assert torch.equal(zk.permute(0, 3, 1, 2, 4).reshape(nb, bs, H, D), fk)
+    assert torch.equal(zv.permute(0, 3, 1, 2), fv)
+
+
 def test_softmax_backward_pinned():
     """Against the Jacobian written out element by element, and against central differences of the forward."""
     import math

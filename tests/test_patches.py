@@ -13,6 +13,7 @@ from flag_gems.patches import patch_util, patch_vllm_all
 
 def _fake_vllm(monkeypatch):
     names = {
+        "vllm.attention.ops.paged_attn": ["PagedAttention"],
         "vllm.model_executor.layers.activation": ["SiluAndMul"],
         "vllm.model_executor.layers.layernorm": ["RMSNorm"],
         "vllm.model_executor.layers.rotary_embedding": ["RotaryEmbedding"],
@@ -26,7 +27,8 @@ def _fake_vllm(monkeypatch):
             if sub not in sys.modules:
                 monkeypatch.setitem(sys.modules, sub, types.ModuleType(sub))
         for c in cls_names:
-            cls = type(c, (), {"forward_cuda": lambda self, *a: "native", "forward": lambda self, *a: "native"})
+            cls = type(c, (), {"forward_cuda": lambda self, *a: "native", "forward": lambda self, *a: "native",
+                               "write_to_paged_cache": staticmethod(lambda *a: "native")})
             setattr(sys.modules[mod_name], c, cls)
             classes[c] = cls
     return classes
@@ -61,6 +63,7 @@ def test_installer_patches_methods_and_library_kernel(monkeypatch, capsys):
     assert classes["RotaryEmbedding"].forward_cuda is patch_vllm_all.custom_gems_rope_forward_cuda
     assert classes["SiluAndMul"].forward_cuda is patch_vllm_all.custom_gems_silu_and_mul
     assert classes["FlashAttentionImpl"].forward is patch_vllm_all.custom_gems_flash_attention_impl_forward
+    assert classes["PagedAttention"].write_to_paged_cache is patch_vllm_all.custom_gems_write_to_paged_cache
     assert keys == [("silu_and_mul", "CUDA")]
     torch.ops._C.silu_and_mul(torch.empty(2, 4), torch.ones(2, 8))
     assert seen == [(2, 8)]
