@@ -29,14 +29,16 @@ __global__ __launch_bounds__(256) void cache_scatter_kernel(const char* __restri
   const int64_t n = row_bytes / (int64_t)sizeof(U);
   // four pieces per lane in flight: the row is short, so the copy lives on memory-level parallelism
   int64_t i = threadIdx.x & 63;
+  // streaming accesses: neither the token rows nor the cache lines written here are read again soon
   for (; i + 192 < n; i += 256) {
-    const U a = src[i], b = src[i + 64], c = src[i + 128], d = src[i + 192];
-    dst[i] = a;
-    dst[i + 64] = b;
-    dst[i + 128] = c;
-    dst[i + 192] = d;
+    const U a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + 64),
+            c = __builtin_nontemporal_load(src + i + 128), d = __builtin_nontemporal_load(src + i + 192);
+    __builtin_nontemporal_store(a, dst + i);
+    __builtin_nontemporal_store(b, dst + i + 64);
+    __builtin_nontemporal_store(c, dst + i + 128);
+    __builtin_nontemporal_store(d, dst + i + 192);
   }
-  for (; i < n; i += 64) dst[i] = src[i];
+  for (; i < n; i += 64) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 template <typename SLOT>
