@@ -258,22 +258,31 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 // Read straight into MFMA fragments, this layout gives every load instruction 16 rows x 64 bytes: half
 // cache lines, and only as many bytes in flight as registers can hold.  Here the rows go to LDS by
 // asynchronous copies (global_load_lds) instead, 8 rows x 128 bytes per instruction, into a private
-// ring of kcRing slots per wave, issued kcRing-1 steps ahead of their use; fragments are read back
+// ring of slots per wave, issued ring-1 steps ahead of their use; fragments are read back
 // from LDS (the 16-byte pieces of a row are permuted by the row number on the way in, so that the
 // sixteen lanes of a fragment read hit different banks).  The output tile is 16 rows x 16 columns:
 // with that few columns a workgroup's range usually covers whole tiles (N = 4096 gives exactly one
 // tile per CU of a 256-CU part) and there is nothing to fix up between workgroups; split tiles use
 // the same ticket scheme as above.  Requires K % 64 == 0.
-constexpr int kcTileN = 16, kcStepK = 64, kcRing = 8;
-constexpr int kcSlotB = kcTileN * kcStepK * 2;            // bytes of one ring slot
-constexpr int kcLdsBytes = kWaves * kcRing * kcSlotB;     // 128 KB
-constexpr int kcTileElems = 16 * kcTileN;
+// Wide outputs (N >= 8192) take 32-column tiles on a ring of 4 slots instead: the same bytes in flight, but
+// every A fragment (which all workgroups fetch from L2 at the same time) feeds two column blocks, and a
+// workgroup restarts its pipeline half as often.
+constexpr int kcStepK = 64;
+constexpr int kcLdsBytes = kWaves * 8 * 16 * kcStepK * 2;  // 128 KB: 8 slots of 16 rows, or 4 slots of 32 rows, per wave
 
-template <typename T>
+template <typename T, int TN, int RING>
 __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   typedef typename Mfma16<T>::Frag Frag;
+  constexpr int SLOTB = TN * kcStepK * 2;      // bytes of one ring slot
+  constexpr int NCB = TN / 16;                 // 16-column blocks per tile
+  constexpr int NDMA = TN / 8;                 // copy instructions per step (8 rows x 128 bytes each)
+  constexpr int OPS = NDMA + 2;                // memory operations per step
+  constexpr int TILE_ELEMS = 16 * TN;
+  static_assert(kWaves * RING * SLOTB == kcLdsBytes, "ring does not fill the LDS budget");
+  static_assert(OPS * (RING - 1) < 64, "wait count exceeds the counter");
+  static_assert(TILE_ELEMS <= kBlock, "one thread per output element");
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  __shared__ float red[kWaves][kcTileElems];
+  __shared__ float red[kWaves][TILE_ELEMS];
   __shared__ unsigned ticket_s;
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -282,8 +291,9 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   const int M = (int)g.M, N = (int)g.N;
   const char* A = (const char*)g.A;
   const char* B = (const char*)g.B;
-  char* const ring = lds + __builtin_amdgcn_readfirstlane(wave) * (kcRing * kcSlotB);
-  // fragment of MFMA h: row m of the slot, 16-byte piece 4h + grp, stored at position piece ^ (row & 7)
+  char* const ring = lds + __builtin_amdgcn_readfirstlane(wave) * (RING * SLOTB);
+  // fragment of MFMA h of column block c: row 16c + m of the slot, 16-byte piece 4h + grp, stored at position
+  // piece ^ (row & 7); (16c + m) & 7 == m & 7, so the block only adds c * 2048 bytes
   int rd[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) rd[h] = m * 128 + (((4 * h + grp) ^ (m & 7)) << 4);
@@ -298,7 +308,7 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
     const int64_t tile_end = tile_begin + a.ksteps;
     const int ks0 = (int)(u - tile_begin);
     const int ks1 = (int)((u_end < tile_end ? u_end : tile_end) - tile_begin);
-    const int n0 = tile * kcTileN;
+    const int n0 = tile * TN;
 
     const int nsteps = ks1 - ks0;
     const int share = (nsteps + kWaves - 1) / kWaves;
@@ -306,12 +316,14 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
     const int my1 = (my0 + share < ks1) ? my0 + share : ks1;
     const int nmine = my1 - my0;
 
-    f32x4v acc = f32x4v{0.f, 0.f, 0.f, 0.f};
+    f32x4v acc[NCB];
+#pragma unroll
+    for (int c = 0; c < NCB; ++c) acc[c] = f32x4v{0.f, 0.f, 0.f, 0.f};
     if (nmine > 0) {
       // copy instruction i of a step: slot rows 8i + lane/8, the lane's piece chosen so that it lands permuted
-      const char* bsrc[2];
+      const char* bsrc[NDMA];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < NDMA; ++i) {
         const int r = 8 * i + (lane >> 3);
         const int c = (lane & 7) ^ (r & 7);
         int n = n0 + r;
@@ -321,67 +333,81 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       const char* asrc[2];
 #pragma unroll
       for (int h = 0; h < 2; ++h) asrc[h] = A + ((int64_t)arow * g.sam + (4 * h + grp) * 8) * 2;
-      u32x4 af[kcRing][2];
-      // Every step issues the same four memory operations, so the count to wait for is a constant; steps
-      // past the end of the share re-read the last one (served by the caches) and are not computed.
+      u32x4 af[RING][2];
+      // Every step issues the same memory operations, so the count to wait for is a constant; steps past the
+      // end of the share re-read the last one (served by the caches) and are not computed.
+      // Every workgroup would otherwise walk K in the same order at the same time, all of them asking L2 for the
+      // same lines of A (and, with power-of-two row lengths, the same memory channels for B): each wave starts its
+      // share at its own offset and wraps around.  The order is a function of (workgroup, wave), so results stay
+      // bit-identical from run to run.
+      const int rot = (int)(((unsigned)w * 13u + (unsigned)wave * 5u) % (unsigned)nmine);
       auto issue = [&](int step, auto pc) {
         constexpr int p = decltype(pc)::value;
         const int sidx = step < nmine ? step : nmine - 1;
-        const int64_t koff = (int64_t)(my0 + sidx) * (kcStepK * 2);
-        char* slot = ring + p * kcSlotB;
-        __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[0] + koff), FGK_LDSP(slot), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[1] + koff), FGK_LDSP(slot), 16, 1024, 0);
+        int kidx = sidx + rot;
+        kidx = kidx >= nmine ? kidx - nmine : kidx;
+        const int64_t koff = (int64_t)(my0 + kidx) * (kcStepK * 2);
+        char* slot = ring + p * SLOTB;
+        static_for<0, NDMA>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[i] + koff), FGK_LDSP(slot), 16, i * 1024, 0);
+        });
         af[p][0] = *reinterpret_cast<const u32x4*>(asrc[0] + koff);
         af[p][1] = *reinterpret_cast<const u32x4*>(asrc[1] + koff);
       };
       auto compute = [&](auto pc) {
         constexpr int p = decltype(pc)::value;
-        const char* slot = ring + p * kcSlotB;
+        const char* slot = ring + p * SLOTB;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const Frag bf = *reinterpret_cast<const Frag*>(slot + rd[h]);
-          acc = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, af[p][h]), acc);
+        for (int c = 0; c < NCB; ++c) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const Frag bf = *reinterpret_cast<const Frag*>(slot + c * 2048 + rd[h]);
+            acc[c] = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, af[p][h]), acc[c]);
+          }
         }
       };
-      static_for<0, kcRing - 1>([&](auto pc) {
+      static_for<0, RING - 1>([&](auto pc) {
         issue(decltype(pc)::value, pc);
         __builtin_amdgcn_sched_barrier(0);
       });
-      // whole rounds of the ring: issue, wait for the step issued kcRing-1 steps ago, compute -- no branches,
+      // whole rounds of the ring: issue, wait for the step issued RING-1 steps ago, compute -- no branches,
       // so the number of operations in flight at every wait is known
       int i = 0;
-      for (; i + kcRing <= nmine; i += kcRing) {
-        static_for<0, kcRing>([&](auto pc) {
+      for (; i + RING <= nmine; i += RING) {
+        static_for<0, RING>([&](auto pc) {
           constexpr int p = decltype(pc)::value;
-          issue(i + p + kcRing - 1, IntC<(p + kcRing - 1) % kcRing>{});
-          FGK_WAIT_VM(4 * (kcRing - 1));
+          issue(i + p + RING - 1, IntC<(p + RING - 1) % RING>{});
+          FGK_WAIT_VM(OPS * (RING - 1));
           compute(pc);
           __builtin_amdgcn_sched_barrier(0);
         });
       }
-      // the rest (fewer than kcRing steps) is already on its way
+      // the rest (fewer than RING steps) is already on its way
       FGK_WAIT_VM(0);
       const int rest = nmine - i;
-      static_for<0, kcRing - 1>([&](auto pc) {
+      static_for<0, RING - 1>([&](auto pc) {
         if (decltype(pc)::value < rest) compute(pc);
       });
     }
 
-    // ---- add the 8 waves' accumulators through LDS; thread t < 256 ends up with element t ----------
+    // ---- add the 8 waves' accumulators through LDS; thread t < TILE_ELEMS ends up with element t ----------
     __syncthreads();  // red[] of the previous segment is no longer read
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[wave][i * 64 + lane] = acc[i];
+    for (int c = 0; c < NCB; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][(c * 4 + i) * 64 + lane] = acc[c][i];
     __syncthreads();
     float sum = 0.f;
-    if (tid < kcTileElems) {
+    if (tid < TILE_ELEMS) {
 #pragma unroll
       for (int v = 0; v < kWaves; ++v) sum += red[v][tid];
     }
 
     bool finish = (ks0 == 0 && ks1 == a.ksteps);
     if (!finish) {
-      float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * kcTileElems;
-      if (tid < kcTileElems) st_coherent(slot + tid, sum);
+      float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * TILE_ELEMS;
+      if (tid < TILE_ELEMS) st_coherent(slot + tid, sum);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();
       const int w_first = worker_of(a.per, a.rem, tile_begin);
@@ -392,22 +418,23 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       if (ticket_s == (unsigned)(w_last - w_first)) {
         finish = true;
         sum = 0.f;
-        if (tid < kcTileElems) {
+        if (tid < TILE_ELEMS) {
           for (int w2 = w_first; w2 <= w_last; ++w2) {
             const float* src =
-                a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * kcTileElems;
+                a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * TILE_ELEMS;
             sum += ld_coherent(src + tid);
           }
         }
         if (tid == 0) __hip_atomic_store(a.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    if (finish && tid < kcTileElems) {
+    if (finish && tid < TILE_ELEMS) {
       T* C = (T*)g.C;
       const T* bias = (const T*)g.bias;
-      const int el = tid & 63, i = tid >> 6;
+      // element tid = (c * 4 + i) * 64 + el of the accumulators: row el & 15, column 16c + 4 * (el >> 4) + i
+      const int el = tid & 63, i = (tid >> 6) & 3, cb = tid >> 8;
       const int em = el & 15, eg = el >> 4;
-      const int n = n0 + 4 * eg + i;
+      const int n = n0 + 16 * cb + 4 * eg + i;
       if (em < M && n < N) {
         float v = sum;
         if (bias != nullptr) v = v * g.alpha + (float)bias[(int64_t)em * g.sim + (int64_t)n * g.sin] * g.beta;
@@ -419,11 +446,11 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   }
 }
 
-template <typename T>
+template <typename T, int TN, int RING>
 int launch_kc(const SkinnyArgs& a, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kern = gemm_skinny_kc_kernel<T>;
+  auto kern = gemm_skinny_kc_kernel<T, TN, RING>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kcLdsBytes);
   });
@@ -461,7 +488,10 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   a.g = g;
   // K-contiguous B with K a multiple of 64: the kernel that stages B through LDS, on 16-column tiles
   const bool kc = b_kind == 2 && g.K % kcStepK == 0 && getenv("FG_SKINNY_NO_LDS") == nullptr;
-  a.tiles_n = (int)fg_cdiv(g.N, kc ? kcTileN : kTileN);
+  // 32-column tiles once they still give every CU a tile of its own (measurement aid: FG_SKINNY_TILE=16|32)
+  int kc_tile = g.N >= 32 * (int64_t)num_cu ? 32 : 16;
+  if (const char* e = getenv("FG_SKINNY_TILE")) kc_tile = atoi(e) == 32 ? 32 : atoi(e) == 16 ? 16 : kc_tile;
+  a.tiles_n = (int)fg_cdiv(g.N, kc ? kc_tile : kTileN);
   a.ksteps = (int)fg_cdiv(g.K, kc ? kcStepK : kStepK);
   const int64_t units = (int64_t)a.tiles_n * a.ksteps;
   if (num_cu > kMaxWorkers) num_cu = kMaxWorkers;
@@ -471,7 +501,8 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   char* ws = (char*)workspace;
   a.tickets = (unsigned*)(ws + kTicketOffset);
   a.partials = (float*)(ws + kPartialOffset);
-  if (kc) return dtype == FG_BF16 ? launch_kc<bf16_t>(a, st) : launch_kc<f16_t>(a, st);
+  if (kc && kc_tile == 32) return dtype == FG_BF16 ? launch_kc<bf16_t, 32, 4>(a, st) : launch_kc<f16_t, 32, 4>(a, st);
+  if (kc) return dtype == FG_BF16 ? launch_kc<bf16_t, 16, 8>(a, st) : launch_kc<f16_t, 16, 8>(a, st);
   dim3 grid((unsigned)a.workers), block(kBlock);
   if (dtype == FG_BF16) {
     if (b_kind == 1) hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, true>), grid, block, 0, st, a);

@@ -150,6 +150,9 @@ SK_CASES = [
     # K a multiple of 8 but not of 64, K an odd multiple of 64
     (16, 24, 2048, _C.SCHED_AUTO), (2, 8200, 1024, _C.SCHED_AUTO), (5, 1000, 1032, _C.SCHED_AUTO),
     (9, 4096, 1088, _C.SCHED_AUTO),
+    # ... wide outputs (32-column tiles when B = W^T): whole tiles per workgroup, split tiles, a ragged last tile
+    (16, 12288, 4096, _C.SCHED_AUTO), (5, 8192, 1088, _C.SCHED_AUTO), (16, 32000, 4096, _C.SCHED_AUTO),
+    (7, 8456, 2048, _C.SCHED_AUTO),
     # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
     (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
