@@ -81,6 +81,15 @@ __device__ __forceinline__ void st_pack_nt(T* p, const Pack<T, VEC>& v) {
   }
 }
 
+// Waits until every vector-memory operation this wave has issued, stores included, has completed.
+// A workgroup-scope release fence does not emit this wait on gfx950 (the waves of a workgroup share
+// one L1, so the fence has nothing to order for them), and a device-scope release would write the
+// whole L2 back.  Publishing device-coherent (write-through) stores to another workgroup through a
+// later atomic therefore spells the wait out: stores complete, then the barrier, then the atomic.
+__device__ __forceinline__ void fg_wait_vmem_done() {
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (0xF << 8));  // vmcnt(0); expcnt and lgkmcnt not waited for
+}
+
 // ---------------------------------------------------------------------------------------------
 // wavefront-64 reductions.  The first four butterfly steps stay inside a row of 16 lanes and use
 // DPP modifiers (no LDS traffic); the last two cross rows through ds_bpermute.

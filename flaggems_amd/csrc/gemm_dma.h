@@ -361,8 +361,9 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
             for (int e = 0; e < 16; ++e)
               __hip_atomic_store(slot + ((i * TN + j) * 16 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
-        // device-coherent stores: waiting for their completion before the ticket publishes them
+        // device-coherent stores: every one of them has completed before the ticket publishes them
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        fg_wait_vmem_done();
         __syncthreads();
         const int w_first = sk_worker_of(g.sk_per, g.sk_rem, tile_begin);
         const int w_last = sk_worker_of(g.sk_per, g.sk_rem, tile_end - 1);

@@ -193,11 +193,11 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
       for (int j = 0; j < kEPT; ++j) st_coherent(slot + tid + kBlock * j, sum[j]);
       // The partial tile is written with device-coherent (write-through) stores, so no cache
-      // write-back is needed to publish it: it is enough that every store has completed
-      // (the workgroup-scope fence waits for that) before the ticket is drawn.  A device-scope
-      // release/acquire pair here would flush and invalidate the whole L2 and costs more than the
-      // rest of the kernel.
+      // write-back is needed to publish it: it is enough that every store has completed before the
+      // ticket is drawn.  A device-scope release/acquire pair here would flush and invalidate the
+      // whole L2 and costs more than the rest of the kernel.
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      fg_wait_vmem_done();
       __syncthreads();  // every thread's slice of the partial tile is out
       const int w_first = worker_of(a.per, a.rem, tile_begin);
       const int w_last = worker_of(a.per, a.rem, tile_end - 1);
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 constexpr int kcStepK = 64;
 constexpr int kcLdsBytes = kWaves * 8 * 16 * kcStepK * 2;  // 128 KB: 8 slots of 16 rows, or 4 slots of 32 rows, per wave
 
-template <typename T, int TN, int RING>
+template <typename T, int TN, int RING, bool A_LINES>
 __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   typedef typename Mfma16<T>::Frag Frag;
   constexpr int SLOTB = TN * kcStepK * 2;      // bytes of one ring slot
@@ -297,7 +297,6 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   int rd[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) rd[h] = m * 128 + (((4 * h + grp) ^ (m & 7)) << 4);
-  const int arow = m < M ? m : M - 1;  // rows beyond M are computed on a copy of the last row and never stored
 
   const int64_t u_begin = range_begin(a.per, a.rem, w);
   const int64_t u_end = range_begin(a.per, a.rem, w + 1);
@@ -330,9 +329,23 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
         n = n < N ? n : N - 1;
         bsrc[i] = B + ((int64_t)n * g.sbn + c * 8) * 2 - i * 1024;  // the instruction offset moves both addresses
       }
+      // A_LINES (more than 8 rows): A is fetched in whole cache lines, load j of a step covering rows 8j .. 8j+7
+      // with eight lanes per row (a load in fragment order touches 16 half lines; measured 4 us of a 30 us call).
+      // The fragment of MFMA h, piece 4h + grp of row m, then sits in load m / 8 of lane (m % 8) * 8 + 4h + grp and
+      // is fetched from there with ds_bpermute when the step is computed.  With few rows the lanes of a fragment
+      // load share their lines anyway and the loads go straight to fragment order (load h = MFMA h).
+      // Rows beyond M are computed on a copy of the last row and never stored.
       const char* asrc[2];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) asrc[h] = A + ((int64_t)arow * g.sam + (4 * h + grp) * 8) * 2;
+      for (int j = 0; j < 2; ++j) {
+        int fr = A_LINES ? 8 * j + (lane >> 3) : m;
+        fr = fr < M ? fr : M - 1;
+        asrc[j] = A + ((int64_t)fr * g.sam + (A_LINES ? (lane & 7) : 4 * j + grp) * 8) * 2;
+      }
+      int perm[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) perm[h] = ((m & 7) * 8 + 4 * h + grp) * 4;
+      const bool upper = m >= 8;
       u32x4 af[RING][2];
       // Every step issues the same memory operations, so the count to wait for is a constant; steps past the
       // end of the share re-read the last one (served by the caches) and are not computed.
@@ -358,12 +371,26 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       auto compute = [&](auto pc) {
         constexpr int p = decltype(pc)::value;
         const char* slot = ring + p * SLOTB;
+        u32x4 fa[2];
+        if constexpr (A_LINES) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const int lo = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][0][d]);
+              const int hi = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][1][d]);
+              fa[h][d] = (uint32_t)(upper ? hi : lo);
+            }
+        } else {
+          fa[0] = af[p][0];
+          fa[1] = af[p][1];
+        }
 #pragma unroll
         for (int c = 0; c < NCB; ++c) {
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const Frag bf = *reinterpret_cast<const Frag*>(slot + c * 2048 + rd[h]);
-            acc[c] = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, af[p][h]), acc[c]);
+            acc[c] = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, fa[h]), acc[c]);
           }
         }
       };
@@ -409,6 +436,7 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * TILE_ELEMS;
       if (tid < TILE_ELEMS) st_coherent(slot + tid, sum);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      fg_wait_vmem_done();
       __syncthreads();
       const int w_first = worker_of(a.per, a.rem, tile_begin);
       const int w_last = worker_of(a.per, a.rem, tile_end - 1);
@@ -446,11 +474,11 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   }
 }
 
-template <typename T, int TN, int RING>
-int launch_kc(const SkinnyArgs& a, hipStream_t st) {
+template <typename T, int TN, int RING, bool A_LINES>
+int launch_kc_t(const SkinnyArgs& a, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kern = gemm_skinny_kc_kernel<T, TN, RING>;
+  auto kern = gemm_skinny_kc_kernel<T, TN, RING, A_LINES>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kcLdsBytes);
   });
@@ -460,6 +488,11 @@ int launch_kc(const SkinnyArgs& a, hipStream_t st) {
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)a.workers), dim3(kBlock), kcLdsBytes, st, a);
   return fg_check_launch("gemm(stream-K, skinny)");
+}
+
+template <typename T, int TN, int RING>
+int launch_kc(const SkinnyArgs& a, hipStream_t st) {
+  return a.g.M > 8 ? launch_kc_t<T, TN, RING, true>(a, st) : launch_kc_t<T, TN, RING, false>(a, st);
 }
 
 }  // namespace

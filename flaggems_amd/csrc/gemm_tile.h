@@ -384,8 +384,9 @@ __global__ __launch_bounds__(kThreads) void gemm_streamk_kernel(GemmArgs g) {
             __hip_atomic_store(slot + ((i * TC::TN + j) * 16 + e) * kThreads + tid, acc[i][j][e], __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
       // device-coherent stores need no cache write-back to be visible; waiting for their completion
-      // (workgroup-scope fence) before the ticket is enough, and far cheaper than flushing L2
+      // before the ticket is enough, and far cheaper than flushing L2
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      fg_wait_vmem_done();
       __syncthreads();  // every thread's slice of the partial tile is out
       const int w_first = sk_worker_of(g.sk_per, g.sk_rem, tile_begin);
       const int w_last = sk_worker_of(g.sk_per, g.sk_rem, tile_end - 1);
