@@ -23,14 +23,25 @@ namespace {
 
 enum { BWD_SOFTMAX = 0, BWD_LOG_SOFTMAX = 1, BWD_RMS = 2 };
 
-template <int TPR>
+// Barrier that orders LDS traffic only: global loads issued before it (the next row's prefetch) stay in flight,
+// where __syncthreads() would wait for them.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// LIGHT: the barriers order LDS traffic only (for the kernel that keeps global loads in flight across them).
+template <int TPR, bool LIGHT = false>
 __device__ __forceinline__ float row_sum(float v, float* smem, int row_in_block, int t) {
   v = wave_sum(v);
   if constexpr (TPR > 64) {
     constexpr int WPR = TPR / 64;  // waves per row
-    __syncthreads();
+    if constexpr (LIGHT) lds_barrier();
+    else __syncthreads();
     if ((t & 63) == 0) smem[row_in_block * WPR + (t >> 6)] = v;
-    __syncthreads();
+    if constexpr (LIGHT) lds_barrier();
+    else __syncthreads();
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < WPR; ++i) s += smem[row_in_block * WPR + i];
@@ -100,8 +111,80 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
 
 // rms_norm: dx for the rows of one group, and the group's column sums for the weight gradient.
 // Group = rows [group * rows_per_group, ...); a block holds RPB groups (one per TPR threads).  Every thread
-// of a block runs the same number of iterations, so the barriers inside row_sum are uniform.
-template <typename T, int VEC, int ITERS, int TPR>
+// of a block runs the same number of iterations, so the barriers inside row_sum are uniform.  The packs of a
+// row are requested one row ahead (two buffers, the loop advances two rows per trip), so that they travel while
+// the current row is reduced.
+// The loads are unconditional (a row past the end is read from the last row, a column past the end from column
+// 0, both discarded later): without branches around them the compiler's wait counts stay exact and the requests of
+// the next row really remain in flight across the reduction.
+template <typename T, int VEC, int ITERS, int TPR, bool CLAMP>
+__device__ __forceinline__ void rms_bwd_fetch(Pack<T, VEC> (&px)[ITERS], Pack<T, VEC> (&pd)[ITERS], float& pinv, bool ok,
+                                              int64_t row, int64_t M, const T* __restrict__ x, const T* __restrict__ dy,
+                                              const float* __restrict__ inv_rms, int N, int t) {
+  if constexpr (CLAMP) {
+    const int64_t rr = ok ? row : M - 1;
+    const float v = inv_rms[rr];
+    pinv = ok ? v : 0.f;
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      const int cc = col < N ? col : 0;
+      px[j] = ld_pack_nt<T, VEC>(x + rr * (int64_t)N + cc);
+      pd[j] = ld_pack_nt<T, VEC>(dy + rr * (int64_t)N + cc);
+    }
+  } else {
+    pinv = ok ? inv_rms[row] : 0.f;
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      if (ok && col < N) {
+        px[j] = ld_pack_nt<T, VEC>(x + row * (int64_t)N + col);
+        pd[j] = ld_pack_nt<T, VEC>(dy + row * (int64_t)N + col);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) px[j].v[e] = pd[j].v[e] = (T)0.f;
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, int ITERS, int TPR, bool LIGHT>
+__device__ __forceinline__ void rms_bwd_row(const Pack<T, VEC> (&cx)[ITERS], const Pack<T, VEC> (&cd)[ITERS], float inv,
+                                            bool row_ok, int64_t row, const float (&wv)[ITERS][VEC],
+                                            float (&acc)[ITERS][VEC], float* smem, T* __restrict__ dx, int N, int t,
+                                            int row_in_block) {
+  float xh[ITERS][VEC], d[ITERS][VEC];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const bool col_ok = (j * TPR + t) * VEC < N;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      xh[j][e] = col_ok ? (float)cx[j].v[e] * inv : 0.f;
+      d[j][e] = col_ok ? (float)cd[j].v[e] : 0.f;
+      s += xh[j][e] * d[j][e] * wv[j][e];
+    }
+  }
+  s = row_sum<TPR, LIGHT>(s, smem, row_in_block, t);
+  const float mean = s / (float)N;
+  if (row_ok) {
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      if (col < N) {
+        Pack<T, VEC> po;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          po.v[e] = (T)((d[j][e] * wv[j][e] - xh[j][e] * mean) * inv);
+          acc[j][e] += xh[j][e] * d[j][e];
+        }
+        st_pack_nt<T, VEC>(dx + row * (int64_t)N + col, po);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, int ITERS, int TPR, bool PREFETCH>
 __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_bwd_rows_kernel(
     const T* __restrict__ x, const T* __restrict__ dy, const T* __restrict__ w, const float* __restrict__ inv_rms,
     T* __restrict__ dx, float* __restrict__ dw_partial, int64_t partial_rows, int64_t M, int N, int rows_per_group) {
@@ -130,45 +213,30 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_bwd_rows_kernel(
     for (int e = 0; e < VEC; ++e) acc[j][e] = 0.f;
   }
 
-  for (int i = 0; i < rows_per_group; ++i) {
-    const int64_t row = r0 + i;
-    const bool row_ok = row < M;
-    const float inv = row_ok ? inv_rms[row] : 0.f;
-    float xh[ITERS][VEC], d[ITERS][VEC];
-    float s = 0.f;
-#pragma unroll
-    for (int j = 0; j < ITERS; ++j) {
-      const int col = (j * TPR + t) * VEC;
-      if (row_ok && col < N) {
-        const Pack<T, VEC> px = ld_pack_nt<T, VEC>(x + row * (int64_t)N + col);
-        const Pack<T, VEC> pd = ld_pack_nt<T, VEC>(dy + row * (int64_t)N + col);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          xh[j][e] = (float)px.v[e] * inv;
-          d[j][e] = (float)pd.v[e];
-          s += xh[j][e] * d[j][e] * wv[j][e];
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) xh[j][e] = d[j][e] = 0.f;
+  if constexpr (PREFETCH) {
+    Pack<T, VEC> ax[ITERS], ad[ITERS], bx[ITERS], bd[ITERS];
+    float ainv, binv = 0.f;
+    rms_bwd_fetch<T, VEC, ITERS, TPR, true>(ax, ad, ainv, r0 < M, r0, M, x, dy, inv_rms, N, t);
+    for (int i = 0; i < rows_per_group; i += 2) {
+      const int64_t row = r0 + i;
+      const bool second = i + 1 < rows_per_group;  // uniform over the block, like every branch in this loop
+      if (second) rms_bwd_fetch<T, VEC, ITERS, TPR, true>(bx, bd, binv, row + 1 < M, row + 1, M, x, dy, inv_rms, N, t);
+      rms_bwd_row<T, VEC, ITERS, TPR, true>(ax, ad, ainv, row < M, row, wv, acc, smem, dx, N, t, row_in_block);
+      if (second) {
+        if (i + 2 < rows_per_group)
+          rms_bwd_fetch<T, VEC, ITERS, TPR, true>(ax, ad, ainv, row + 2 < M, row + 2, M, x, dy, inv_rms, N, t);
+        rms_bwd_row<T, VEC, ITERS, TPR, true>(bx, bd, binv, row + 1 < M, row + 1, wv, acc, smem, dx, N, t, row_in_block);
       }
     }
-    s = row_sum<TPR>(s, smem, row_in_block, t);
-    const float mean = s / (float)N;
-    if (row_ok) {
-#pragma unroll
-      for (int j = 0; j < ITERS; ++j) {
-        const int col = (j * TPR + t) * VEC;
-        if (col < N) {
-          Pack<T, VEC> po;
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) {
-            po.v[e] = (T)((d[j][e] * wv[j][e] - xh[j][e] * mean) * inv);
-            acc[j][e] += xh[j][e] * d[j][e];
-          }
-          st_pack_nt<T, VEC>(dx + row * (int64_t)N + col, po);
-        }
-      }
+  } else {
+    // one row per group (no weight gradient wanted: a leaner kernel, three workgroups per CU instead of two), or
+    // two packs per thread, where a second buffer would not fit the registers of a 1024-thread block: fetch and use
+    for (int i = 0; i < rows_per_group; ++i) {
+      const int64_t row = r0 + i;
+      Pack<T, VEC> ax[ITERS], ad[ITERS];
+      float ainv;
+      rms_bwd_fetch<T, VEC, ITERS, TPR, false>(ax, ad, ainv, row < M, row, M, x, dy, inv_rms, N, t);
+      rms_bwd_row<T, VEC, ITERS, TPR, false>(ax, ad, ainv, row < M, row, wv, acc, smem, dx, N, t, row_in_block);
     }
   }
   if (dw_partial != nullptr && group < partial_rows) {
@@ -300,8 +368,12 @@ void launch_rms_rows(const T* x, const T* dy, const T* w, const float* inv_rms, 
   constexpr int RPB = BLOCK / TPR;
   // every partial row gets written (groups past the last row write zeros); without partial rows one row per group
   const int64_t groups = dw_partial != nullptr ? partial_rows : fg_cdiv(M, rows_per_group);
-  hipLaunchKernelGGL((rms_bwd_rows_kernel<T, VEC, ITERS, TPR>), dim3((unsigned)fg_cdiv(groups, RPB)), dim3(BLOCK), 0, st,
-                     x, dy, w, inv_rms, dx, dw_partial, partial_rows, M, N, rows_per_group);
+  if (ITERS == 1 && rows_per_group > 1)
+    hipLaunchKernelGGL((rms_bwd_rows_kernel<T, VEC, ITERS, TPR, ITERS == 1>), dim3((unsigned)fg_cdiv(groups, RPB)),
+                       dim3(BLOCK), 0, st, x, dy, w, inv_rms, dx, dw_partial, partial_rows, M, N, rows_per_group);
+  else
+    hipLaunchKernelGGL((rms_bwd_rows_kernel<T, VEC, ITERS, TPR, false>), dim3((unsigned)fg_cdiv(groups, RPB)),
+                       dim3(BLOCK), 0, st, x, dy, w, inv_rms, dx, dw_partial, partial_rows, M, N, rows_per_group);
 }
 
 // dw_partial (may be null) has partial_rows rows of N floats; every one of them is written.
