@@ -270,19 +270,28 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 constexpr int kcStepK = 64;
 constexpr int kcLdsBytes = kWaves * 8 * 16 * kcStepK * 2;  // 128 KB: 8 slots of 16 rows, or 4 slots of 32 rows, per wave
 
-template <typename T, int TN, int RING, bool A_LINES>
+// MB = 16-row blocks of A (1, 2 or 4: up to 64 rows).  Every B fragment read from LDS feeds MB MFMAs.  With MB > 1
+// the cross-wave reduction buffer would not fit next to the ring, so it lives in the ring itself: after the last
+// step of a segment every wave's copies have landed, each wave writes its accumulators into its own ring region,
+// and a barrier at the start of the next segment keeps that segment's copies from overwriting sums still being read.
+template <typename T, int TN, int RING, bool A_LINES, int MB>
 __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   typedef typename Mfma16<T>::Frag Frag;
   constexpr int SLOTB = TN * kcStepK * 2;      // bytes of one ring slot
   constexpr int NCB = TN / 16;                 // 16-column blocks per tile
   constexpr int NDMA = TN / 8;                 // copy instructions per step (8 rows x 128 bytes each)
-  constexpr int OPS = NDMA + 2;                // memory operations per step
-  constexpr int TILE_ELEMS = 16 * TN;
-  static_assert(kWaves * RING * SLOTB == kcLdsBytes, "ring does not fill the LDS budget");
+  constexpr int NAL = 2 * MB;                  // A loads per step
+  constexpr int OPS = NDMA + NAL;              // memory operations per step
+  constexpr int TILE_ELEMS = 16 * MB * TN;
+  constexpr int EPT = (TILE_ELEMS + kBlock - 1) / kBlock;  // tile elements per thread in the block-wide phases
+  constexpr int WAVE_RING = RING * SLOTB;
+  static_assert(kWaves * WAVE_RING <= kcLdsBytes, "ring exceeds the LDS budget");
   static_assert(OPS * (RING - 1) < 64, "wait count exceeds the counter");
-  static_assert(TILE_ELEMS <= kBlock, "one thread per output element");
+  static_assert(MB == 1 || A_LINES, "several row blocks are fetched in whole lines");
+  static_assert(TILE_ELEMS * 4 <= WAVE_RING, "a wave's accumulators fit its own ring region");
+  static_assert(TILE_ELEMS % kBlock == 0 || TILE_ELEMS < kBlock, "whole elements per thread");
+  static_assert(TILE_ELEMS <= kTileElems, "partial tiles fit the workspace slots");
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  __shared__ float red[kWaves][TILE_ELEMS];
   __shared__ unsigned ticket_s;
   const GemmArgs& g = a.g;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -291,7 +300,8 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
   const int M = (int)g.M, N = (int)g.N;
   const char* A = (const char*)g.A;
   const char* B = (const char*)g.B;
-  char* const ring = lds + __builtin_amdgcn_readfirstlane(wave) * (RING * SLOTB);
+  char* const ring = lds + __builtin_amdgcn_readfirstlane(wave) * WAVE_RING;
+  float* const red_mine = reinterpret_cast<float*>(ring);  // this wave's slice of the reduction buffer
   // fragment of MFMA h of column block c: row 16c + m of the slot, 16-byte piece 4h + grp, stored at position
   // piece ^ (row & 7); (16c + m) & 7 == m & 7, so the block only adds c * 2048 bytes
   int rd[2];
@@ -315,9 +325,13 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
     const int my1 = (my0 + share < ks1) ? my0 + share : ks1;
     const int nmine = my1 - my0;
 
-    f32x4v acc[NCB];
+    __syncthreads();  // the sums of the previous segment (kept in the ring) are no longer read
+
+    f32x4v acc[MB][NCB];
 #pragma unroll
-    for (int c = 0; c < NCB; ++c) acc[c] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+      for (int c = 0; c < NCB; ++c) acc[rb][c] = f32x4v{0.f, 0.f, 0.f, 0.f};
     if (nmine > 0) {
       // copy instruction i of a step: slot rows 8i + lane/8, the lane's piece chosen so that it lands permuted
       const char* bsrc[NDMA];
@@ -331,13 +345,13 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       }
       // A_LINES (more than 8 rows): A is fetched in whole cache lines, load j of a step covering rows 8j .. 8j+7
       // with eight lanes per row (a load in fragment order touches 16 half lines; measured 4 us of a 30 us call).
-      // The fragment of MFMA h, piece 4h + grp of row m, then sits in load m / 8 of lane (m % 8) * 8 + 4h + grp and
-      // is fetched from there with ds_bpermute when the step is computed.  With few rows the lanes of a fragment
-      // load share their lines anyway and the loads go straight to fragment order (load h = MFMA h).
-      // Rows beyond M are computed on a copy of the last row and never stored.
-      const char* asrc[2];
+      // The fragment of MFMA h of row block rb, piece 4h + grp of row 16rb + m, then sits in load 2rb + m / 8 of
+      // lane (m % 8) * 8 + 4h + grp and is fetched from there with ds_bpermute when the step is computed.  With few
+      // rows the lanes of a fragment load share their lines anyway and the loads go straight to fragment order
+      // (load h = MFMA h).  Rows beyond M are computed on a copy of the last row and never stored.
+      const char* asrc[NAL];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NAL; ++j) {
         int fr = A_LINES ? 8 * j + (lane >> 3) : m;
         fr = fr < M ? fr : M - 1;
         asrc[j] = A + ((int64_t)fr * g.sam + (A_LINES ? (lane & 7) : 4 * j + grp) * 8) * 2;
@@ -346,14 +360,14 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) perm[h] = ((m & 7) * 8 + 4 * h + grp) * 4;
       const bool upper = m >= 8;
-      u32x4 af[RING][2];
-      // Every step issues the same memory operations, so the count to wait for is a constant; steps past the
-      // end of the share re-read the last one (served by the caches) and are not computed.
+      u32x4 af[RING][NAL];
       // Every workgroup would otherwise walk K in the same order at the same time, all of them asking L2 for the
       // same lines of A (and, with power-of-two row lengths, the same memory channels for B): each wave starts its
       // share at its own offset and wraps around.  The order is a function of (workgroup, wave), so results stay
       // bit-identical from run to run.
       const int rot = (int)(((unsigned)w * 13u + (unsigned)wave * 5u) % (unsigned)nmine);
+      // Every step issues the same memory operations, so the count to wait for is a constant; steps past the
+      // end of the share re-read the last one (served by the caches) and are not computed.
       auto issue = [&](int step, auto pc) {
         constexpr int p = decltype(pc)::value;
         const int sidx = step < nmine ? step : nmine - 1;
@@ -365,32 +379,36 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
           constexpr int i = decltype(ic)::value;
           __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[i] + koff), FGK_LDSP(slot), 16, i * 1024, 0);
         });
-        af[p][0] = *reinterpret_cast<const u32x4*>(asrc[0] + koff);
-        af[p][1] = *reinterpret_cast<const u32x4*>(asrc[1] + koff);
+#pragma unroll
+        for (int j = 0; j < NAL; ++j) af[p][j] = *reinterpret_cast<const u32x4*>(asrc[j] + koff);
       };
       auto compute = [&](auto pc) {
         constexpr int p = decltype(pc)::value;
         const char* slot = ring + p * SLOTB;
-        u32x4 fa[2];
+        u32x4 fa[MB][2];
         if constexpr (A_LINES) {
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
+          for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              const int lo = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][0][d]);
-              const int hi = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][1][d]);
-              fa[h][d] = (uint32_t)(upper ? hi : lo);
-            }
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+              for (int d = 0; d < 4; ++d) {
+                const int lo = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][2 * rb][d]);
+                const int hi = __builtin_amdgcn_ds_bpermute(perm[h], (int)af[p][2 * rb + 1][d]);
+                fa[rb][h][d] = (uint32_t)(upper ? hi : lo);
+              }
         } else {
-          fa[0] = af[p][0];
-          fa[1] = af[p][1];
+          fa[0][0] = af[p][0];
+          fa[0][1] = af[p][1];
         }
 #pragma unroll
         for (int c = 0; c < NCB; ++c) {
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const Frag bf = *reinterpret_cast<const Frag*>(slot + c * 2048 + rd[h]);
-            acc[c] = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, fa[h]), acc[c]);
+#pragma unroll
+            for (int rb = 0; rb < MB; ++rb)
+              acc[rb][c] = Mfma16<T>::mma(bf, __builtin_bit_cast(Frag, fa[rb][h]), acc[rb][c]);
           }
         }
       };
@@ -418,23 +436,33 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       });
     }
 
-    // ---- add the 8 waves' accumulators through LDS; thread t < TILE_ELEMS ends up with element t ----------
-    __syncthreads();  // red[] of the previous segment is no longer read
+    // ---- add the 8 waves' accumulators through LDS (the wave's own ring region: all its copies have landed
+    // and its fragment reads are done); thread t ends up with elements t + kBlock * j ---------------------------
 #pragma unroll
-    for (int c = 0; c < NCB; ++c)
+    for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[wave][(c * 4 + i) * 64 + lane] = acc[c][i];
+      for (int c = 0; c < NCB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red_mine[((rb * NCB + c) * 4 + i) * 64 + lane] = acc[rb][c][i];
     __syncthreads();
-    float sum = 0.f;
-    if (tid < TILE_ELEMS) {
+    float sum[EPT];
 #pragma unroll
-      for (int v = 0; v < kWaves; ++v) sum += red[v][tid];
+    for (int j = 0; j < EPT; ++j) {
+      const int e = tid + kBlock * j;
+      float sacc = 0.f;
+      if (e < TILE_ELEMS) {
+#pragma unroll
+        for (int v = 0; v < kWaves; ++v) sacc += reinterpret_cast<const float*>(lds + v * WAVE_RING)[e];
+      }
+      sum[j] = sacc;
     }
 
     bool finish = (ks0 == 0 && ks1 == a.ksteps);
     if (!finish) {
       float* slot = a.partials + ((int64_t)w * 2 + (u_begin < tile_begin ? 1 : 0)) * TILE_ELEMS;
-      if (tid < TILE_ELEMS) st_coherent(slot + tid, sum);
+#pragma unroll
+      for (int j = 0; j < EPT; ++j)
+        if (tid + kBlock * j < TILE_ELEMS) st_coherent(slot + tid + kBlock * j, sum[j]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       fg_wait_vmem_done();
       __syncthreads();
@@ -445,40 +473,47 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       __syncthreads();
       if (ticket_s == (unsigned)(w_last - w_first)) {
         finish = true;
-        sum = 0.f;
-        if (tid < TILE_ELEMS) {
-          for (int w2 = w_first; w2 <= w_last; ++w2) {
-            const float* src =
-                a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * TILE_ELEMS;
-            sum += ld_coherent(src + tid);
-          }
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) sum[j] = 0.f;
+        for (int w2 = w_first; w2 <= w_last; ++w2) {
+          const float* src =
+              a.partials + ((int64_t)w2 * 2 + (range_begin(a.per, a.rem, w2) < tile_begin ? 1 : 0)) * TILE_ELEMS;
+#pragma unroll
+          for (int j = 0; j < EPT; ++j)
+            if (tid + kBlock * j < TILE_ELEMS) sum[j] += ld_coherent(src + tid + kBlock * j);
         }
         if (tid == 0) __hip_atomic_store(a.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    if (finish && tid < TILE_ELEMS) {
+    if (finish) {
       T* C = (T*)g.C;
       const T* bias = (const T*)g.bias;
-      // element tid = (c * 4 + i) * 64 + el of the accumulators: row el & 15, column 16c + 4 * (el >> 4) + i
-      const int el = tid & 63, i = (tid >> 6) & 3, cb = tid >> 8;
-      const int em = el & 15, eg = el >> 4;
-      const int n = n0 + 16 * cb + 4 * eg + i;
-      if (em < M && n < N) {
-        float v = sum;
-        if (bias != nullptr) v = v * g.alpha + (float)bias[(int64_t)em * g.sim + (int64_t)n * g.sin] * g.beta;
-        else if (g.alpha != 1.0f) v = v * g.alpha;
-        C[(int64_t)em * g.scm + (int64_t)n * g.scn] = (T)v;
+#pragma unroll
+      for (int j = 0; j < EPT; ++j) {
+        // element e = ((rb * NCB + cb) * 4 + i) * 64 + el of the accumulators: row 16rb + (el & 15),
+        // column 16cb + 4 * (el >> 4) + i
+        const int e = tid + kBlock * j;
+        const int el = e & 63, i = (e >> 6) & 3, blk = e >> 8;
+        const int cb = blk % NCB, rb = blk / NCB;
+        const int em = 16 * rb + (el & 15), eg = el >> 4;
+        const int n = n0 + 16 * cb + 4 * eg + i;
+        if (e < TILE_ELEMS && em < M && n < N) {
+          float v = sum[j];
+          if (bias != nullptr) v = v * g.alpha + (float)bias[(int64_t)em * g.sim + (int64_t)n * g.sin] * g.beta;
+          else if (g.alpha != 1.0f) v = v * g.alpha;
+          C[(int64_t)em * g.scm + (int64_t)n * g.scn] = (T)v;
+        }
       }
     }
     u = tile_begin + ks1;
   }
 }
 
-template <typename T, int TN, int RING, bool A_LINES>
+template <typename T, int TN, int RING, bool A_LINES, int MB>
 int launch_kc_t(const SkinnyArgs& a, hipStream_t st) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kern = gemm_skinny_kc_kernel<T, TN, RING, A_LINES>;
+  auto kern = gemm_skinny_kc_kernel<T, TN, RING, A_LINES, MB>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kcLdsBytes);
   });
@@ -490,9 +525,19 @@ int launch_kc_t(const SkinnyArgs& a, hipStream_t st) {
   return fg_check_launch("gemm(stream-K, skinny)");
 }
 
-template <typename T, int TN, int RING>
-int launch_kc(const SkinnyArgs& a, hipStream_t st) {
-  return a.g.M > 8 ? launch_kc_t<T, TN, RING, true>(a, st) : launch_kc_t<T, TN, RING, false>(a, st);
+// Up to 16 rows: 16-column tiles on 8 slots, or 32-column tiles on 4 slots (wide outputs).  17..32 rows: the same
+// with two row blocks.  33..64 rows: four row blocks, always on 32-column tiles (10 memory operations per step on an
+// 8-slot ring would overrun the wait counter, and the A fragments of four row blocks want two column blocks to feed).
+template <typename T>
+int launch_kc(const SkinnyArgs& a, int tile, hipStream_t st) {
+  const int64_t M = a.g.M;
+  if (M > 32) return launch_kc_t<T, 32, 4, true, 4>(a, st);
+  if (tile == 32) {
+    if (M > 16) return launch_kc_t<T, 32, 4, true, 2>(a, st);
+    return M > 8 ? launch_kc_t<T, 32, 4, true, 1>(a, st) : launch_kc_t<T, 32, 4, false, 1>(a, st);
+  }
+  if (M > 16) return launch_kc_t<T, 16, 8, true, 2>(a, st);
+  return M > 8 ? launch_kc_t<T, 16, 8, true, 1>(a, st) : launch_kc_t<T, 16, 8, false, 1>(a, st);
 }
 
 }  // namespace
@@ -500,15 +545,24 @@ int launch_kc(const SkinnyArgs& a, hipStream_t st) {
 // 0: not a case for this kernel; 1: B row-major (N contiguous); 2: B = W^T (K contiguous)
 int skinny_supported(const GemmArgs& g, int dtype, int amode, int bmode) {
   if (dtype != FG_F16 && dtype != FG_BF16) return 0;
-  if (g.M > 16 || amode != LOAD_K) return 0;
+  if (g.M > 64 || amode != LOAD_K) return 0;
   if (g.K < 1024) return 0;  // worth it only when K is deep enough to give every CU several k-steps
+  // 17..64 rows: only the kernel that stages a K-contiguous B through LDS has the row blocks for them.  Every
+  // column tile re-reads its rows of A from L2, M / 32 bytes per byte of B, so it pays where the 128x128 tile
+  // kernels cannot fill the machine (narrow outputs) and, up to 32 rows, for outputs of moderate width; measured
+  // against those kernels on 4096..32000 columns with K = 4096..14336.
+  if (g.M > 16) {
+    if (bmode != LOAD_K || g.K % kcStepK != 0 || getenv("FG_SKINNY_NO_LDS") != nullptr) return 0;
+    const bool pays = g.N <= 8192 || (g.M <= 32 && g.N <= 24576);
+    return pays || getenv("FG_SKINNY_ROWS64") != nullptr ? 2 : 0;
+  }
   if (bmode == LOAD_K) return 2;
   if (bmode == LOAD_MN) return 1;
   return 0;
 }
 
 size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int num_cu) {
-  if (M > 16 || K < 1024) return 0;
+  if (M > 64 || K < 1024) return 0;
   return kPartialOffset + (size_t)num_cu * 2 * kTileElems * sizeof(float);
 }
 
@@ -524,6 +578,7 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   // 32-column tiles once they still give every CU a tile of its own (measurement aid: FG_SKINNY_TILE=16|32)
   int kc_tile = g.N >= 32 * (int64_t)num_cu ? 32 : 16;
   if (const char* e = getenv("FG_SKINNY_TILE")) kc_tile = atoi(e) == 32 ? 32 : atoi(e) == 16 ? 16 : kc_tile;
+  if (g.M > 32) kc_tile = 32;
   a.tiles_n = (int)fg_cdiv(g.N, kc ? kc_tile : kTileN);
   a.ksteps = (int)fg_cdiv(g.K, kc ? kcStepK : kStepK);
   const int64_t units = (int64_t)a.tiles_n * a.ksteps;
@@ -534,8 +589,8 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   char* ws = (char*)workspace;
   a.tickets = (unsigned*)(ws + kTicketOffset);
   a.partials = (float*)(ws + kPartialOffset);
-  if (kc && kc_tile == 32) return dtype == FG_BF16 ? launch_kc<bf16_t, 32, 4>(a, st) : launch_kc<f16_t, 32, 4>(a, st);
-  if (kc) return dtype == FG_BF16 ? launch_kc<bf16_t, 16, 8>(a, st) : launch_kc<f16_t, 16, 8>(a, st);
+  if (kc) return dtype == FG_BF16 ? launch_kc<bf16_t>(a, kc_tile, st) : launch_kc<f16_t>(a, kc_tile, st);
+  FG_REQUIRE(g.M <= 16, FG_ERR_UNSUPPORTED, "gemm(stream-K, skinny): more than 16 rows need the LDS-staged kernel");
   dim3 grid((unsigned)a.workers), block(kBlock);
   if (dtype == FG_BF16) {
     if (b_kind == 1) hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, true>), grid, block, 0, st, a);

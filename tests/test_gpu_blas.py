@@ -153,6 +153,11 @@ SK_CASES = [
     # ... wide outputs (32-column tiles when B = W^T): whole tiles per workgroup, split tiles, a ragged last tile
     (16, 12288, 4096, _C.SCHED_AUTO), (5, 8192, 1088, _C.SCHED_AUTO), (16, 32000, 4096, _C.SCHED_AUTO),
     (7, 8456, 2048, _C.SCHED_AUTO),
+    # ... 17 to 64 rows (two and four row blocks in the LDS-staged kernel when B = W^T): narrow and wide outputs, ragged N,
+    # every tile split between workgroups, K an odd multiple of 64
+    (32, 4096, 4096, _C.SCHED_AUTO), (64, 8192, 4096, _C.SCHED_AUTO), (17, 1000, 2048, _C.SCHED_STREAM_K),
+    (48, 8456, 1088, _C.SCHED_STREAM_K), (33, 152, 1024, _C.SCHED_STREAM_K), (64, 4096, 14336, _C.SCHED_AUTO),
+    (24, 11008, 4096, _C.SCHED_AUTO), (64, 12288, 4096, _C.SCHED_AUTO),
     # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
     (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
