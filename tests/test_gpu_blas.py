@@ -158,6 +158,8 @@ SK_CASES = [
     (32, 4096, 4096, _C.SCHED_AUTO), (64, 8192, 4096, _C.SCHED_AUTO), (17, 1000, 2048, _C.SCHED_STREAM_K),
     (48, 8456, 1088, _C.SCHED_STREAM_K), (33, 152, 1024, _C.SCHED_STREAM_K), (64, 4096, 14336, _C.SCHED_AUTO),
     (24, 11008, 4096, _C.SCHED_AUTO), (64, 12288, 4096, _C.SCHED_AUTO),
+    # ... and wide outputs with 17 to 64 rows (one copy of A per workgroup, eight column tiles in lockstep)
+    (24, 32000, 4096, _C.SCHED_STREAM_K), (64, 22016, 4096, _C.SCHED_STREAM_K), (40, 9000, 1024, _C.SCHED_STREAM_K),
     # ... and the tile stream-K kernel: few tiles / ragged waves / K and M,N tails
     (384, 384, 4096, _C.SCHED_STREAM_K), (1000, 1300, 2048, _C.SCHED_STREAM_K), (2048, 2304, 1024, _C.SCHED_STREAM_K),
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
