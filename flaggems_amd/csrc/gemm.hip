@@ -18,8 +18,9 @@ int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace,
 
 // implemented in gemm_dma.hip
 bool dma_supported(const GemmArgs& g, int elem_bytes);
-void dma_pick_tile(int64_t M, int64_t N, int num_cu, int* bm, int* bn);
-int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st);
+double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep);
+double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, int* workers);
+int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st);
 int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st);
 
 int num_cus(int device) {
@@ -101,9 +102,10 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
     // the machine best (even a lone 128x128 workgroup per CU runs twice as fast as the register-staged kernel).
     if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr) {
       int bm = 256, bn = 256;
-      dma_pick_tile(g.M, g.N, num_cu, &bm, &bn);
+      bool deep = false;
+      dma_pick_tile(g.M, g.N, g.K, num_cu, &bm, &bn, &deep);
       set_tiles(g, bm, bn, BK);
-      return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, st);
+      return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, deep, st);
     }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
@@ -198,12 +200,19 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
           use_streamk = true;
         } else {
           // auto: stream-K when the tiles cannot fill the machine and K is deep enough to hand every workgroup
-          // at least four K steps; fuller grids run data-parallel.  The direct-to-LDS main loop is worth
-          // sharing up to 0.9 waves of tiles, the register-staged one up to half a wave.
+          // at least four K steps; fuller grids run data-parallel.  The register-staged main loop is worth
+          // sharing up to half a wave of tiles; for the direct-to-LDS one the two duration models decide.
           const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
           const int64_t iters = fg_cdiv(K, 64);
           const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && getenv("FG_GEMM_NO_DMA") == nullptr;
-          use_streamk = (dma ? tiles * 10 <= (int64_t)cu * 9 : tiles * 2 <= (int64_t)cu) && tiles * iters >= 4 * (int64_t)cu;
+          if (dma) {
+            int bm, bn, workers;
+            bool deep;
+            use_streamk = tiles <= cu && tiles * iters >= 4 * (int64_t)cu &&
+                          dma_streamk_plan(tiles, iters, cu, &workers) < dma_pick_tile(M, N, K, cu, &bm, &bn, &deep);
+          } else {
+            use_streamk = tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;
+          }
         }
       }
     }

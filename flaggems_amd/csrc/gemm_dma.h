@@ -48,7 +48,9 @@ namespace fgk {
 
 constexpr int kDmaRowB = 128;   // bytes of K per stage per A row
 constexpr int kDmaBK = 64;
-constexpr int dma_lds_bytes(int bm, int bn) { return 2 * (bm + bn) * kDmaRowB; }  // two stages of (A tile + B tile)
+constexpr int dma_lds_bytes(int bm, int bn, int stages = 2) { return stages * (bm + bn) * kDmaRowB; }  // stages of (A tile + B tile)
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
 #define FGK_LDSP(p) ((__attribute__((address_space(3))) void*)(p))
 #define FGK_GLBP(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -137,7 +139,8 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
 }
 
 // Main loop over the K steps [kb0, kb0 + nk) of tile (tm, tn); `finish` receives the accumulators.
-template <typename T, bool B_KC, int BM, int BN, typename F>
+// NS = number of LDS stages: K step kb lives in stage kb % NS and is requested NS - 1 steps ahead.
+template <typename T, bool B_KC, int BM, int BN, int NS, typename F>
 __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish) {
   static_assert(sizeof(T) == 2, "16-bit element types");
   typedef typename Mfma<T>::Frag Frag;
@@ -152,6 +155,8 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   constexpr int RBB = BN * 2;                      // N-contiguous B: bytes per k-row of the tile
   constexpr int CPRB = RBB / 16, RPI = 1024 / RBB; // ... chunks per k-row, k-rows per DMA instruction
   static_assert(HALF <= NMF && NRD <= NMF, "one LDS read or DMA per MFMA");
+  static_assert(NS >= 2 && NS <= 4 && NDMA * (NS - 1) + HALF <= 63, "outstanding DMAs must fit the vmcnt counter");
+  auto stage_off = [](int kb) { return (NS == 2 ? (kb & 1) : NS == 4 ? (kb & 3) : kb % NS) * STAGEB; };
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int row0 = tm * BM, col0 = tn * BN;
@@ -195,7 +200,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
-    char* l = (IS_A ? dma_a : dma_b) + (kb & 1) * STAGEB + (jj >> 2) * 4096;
+    char* l = (IS_A ? dma_a : dma_b) + stage_off(kb) + (jj >> 2) * 4096;
     const char* gp;
     if constexpr (IS_A) gp = a_src[jj] + (int64_t)kb * kDmaRowB;
     else gp = b_src[jj] + (int64_t)kb * b_step;
@@ -242,7 +247,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   auto read_one = [&](int stage, auto sc, auto xc, int set) {
     constexpr int S = decltype(sc)::value;
     constexpr int x = decltype(xc)::value;
-    const int sb = (stage & 1) * STAGEB;
+    const int sb = stage_off(stage);
     if constexpr (x < TM) {
       fa[set][x] = *reinterpret_cast<const Frag*>(lds + sb + a_lane + x * 32 * kDmaRowB + pos[S]);
     } else if constexpr (B_KC) {
@@ -263,11 +268,14 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     for (int j = TN; j < 4; ++j) fb[0][j] = fb[1][j] = u32x4{0u, 0u, 0u, 0u};
   }
 
-  // ---- prologue: stage 0, and the head of stage 1 (the part sub-step 3 of the step before would issue)
-  static_for<0, NDMA>([&](auto jc) { issue(0, jc); });
-  if (nk > 1) {
-    static_for<0, HALF>([&](auto jc) { issue(1, jc); });
-    FGK_WAIT_VM(HALF);
+  // ---- prologue: K steps 0 .. NS-2, and the head of step NS-1 (the part sub-step 3 of the step before would issue)
+  static_for<0, NS - 1>([&](auto sc) {
+    constexpr int s = decltype(sc)::value;
+    if (s < nk) static_for<0, NDMA>([&](auto jc) { issue(s, jc); });
+  });
+  if (nk >= NS) {
+    static_for<0, HALF>([&](auto jc) { issue(NS - 1, jc); });
+    FGK_WAIT_VM(NDMA * (NS - 2) + HALF);  // K step 0 has landed
   } else {
     FGK_WAIT_VM(0);
   }
@@ -276,11 +284,14 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   wait_reads(0);
   __builtin_amdgcn_sched_barrier(0);
 
-  // One K step.  REFILL_TAIL: sub-step 0 issues the second half of the DMAs of stage kb+1;
-  // REFILL_HEAD: sub-step 3 issues the first half of the DMAs of stage kb+2.
-  auto k_step = [&](int kb, auto tail_c, auto head_c) {
+  // One K step.  REFILL_TAIL: sub-step 0 issues the second half of the DMAs of K step kb+NS-1;
+  // REFILL_HEAD: sub-step 3 issues the first half of the DMAs of K step kb+NS (into the stage this step
+  // has just finished reading).  LATER = DMAs that may still be in flight once K step kb+1 has landed:
+  // those of the K steps behind it, which retire in order after it.
+  auto k_step = [&](int kb, auto tail_c, auto head_c, auto later_c) {
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
     constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
+    constexpr int LATER = decltype(later_c)::value;
     static_for<0, 4>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
       constexpr int cur = s & 1, nxt = cur ^ 1;
@@ -292,12 +303,12 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
           if constexpr (s < 3) read_one(kb, IntC<s + 1>{}, xc, nxt);
           else read_one(kb + 1, IntC<0>{}, xc, nxt);
         }
-        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + 2, IntC<x>{});
-        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + 1, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
+        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + NS, IntC<x>{});
+        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + NS - 1, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       if constexpr (s == 2) {
-        FGK_WAIT_VM(0);
+        FGK_WAIT_VM(LATER);
         wait_reads(nxt);
         __builtin_amdgcn_s_barrier();
       } else {
@@ -307,22 +318,27 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     });
   };
   int kb = 0;
-  for (; kb < nk - 2; ++kb) k_step(kb, IntC<1>{}, IntC<1>{});
-  if (kb == nk - 2) {
-    k_step(kb, IntC<1>{}, IntC<0>{});
-    ++kb;
-  }
-  k_step(kb, IntC<0>{}, IntC<0>{});
+  for (; kb < nk - NS; ++kb) k_step(kb, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{});
+  // the last NS steps (fewer when nk < NS), by the number r of K steps behind them: nothing new to request
+  // except the second half of the last step, and ever fewer DMAs left in flight
+  static_for<0, NS - 1>([&](auto ic) {
+    constexpr int r = NS - 1 - decltype(ic)::value;
+    if (kb == nk - 1 - r) {
+      k_step(kb, IntC<(r >= NS - 1 ? 1 : 0)>{}, IntC<0>{}, IntC<NDMA * cmin(NS - 2, r - 1)>{});
+      ++kb;
+    }
+  });
+  k_step(kb, IntC<0>{}, IntC<0>{}, IntC<0>{});
 
   finish(acc);
 }
 
-template <typename T, bool B_KC, int BM, int BN>
-__global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
+template <typename T, bool B_KC, int BM, int BN, int NS = 2>
+__global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
-  dma_tile_mainloop<T, B_KC, BM, BN>(g, lds, tm, tn, 0, (int)(g.K / kDmaBK),
+  dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, 0, (int)(g.K / kDmaBK),
                                      [&](f32x16 (&acc)[BM / 64][BN / 64]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); });
 }
 
@@ -330,7 +346,7 @@ __global__ __launch_bounds__(256, (BM + BN <= 256 ? 2 : 1)) void gemm_dma_kernel
 // in equal contiguous ranges to the workgroups; a tile split between workgroups is finished by whichever
 // of them arrives last (ticket per tile, fp32 partial tiles in the workspace, added in workgroup order so
 // the result does not depend on who finishes).  Same scheme as gemm_streamk_kernel in gemm_tile.h.
-template <typename T, bool B_KC>
+template <typename T, bool B_KC, int NS>
 __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
   constexpr int BM = 128, BN = 128, TM = 2, TN = 2;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -348,7 +364,7 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
     int tm, tn;
     tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
     __syncthreads();  // the LDS stages of the previous segment are no longer read
-    dma_tile_mainloop<T, B_KC, BM, BN>(g, lds, tm, tn, it0, it1 - it0, [&](f32x16 (&acc)[TM][TN]) {
+    dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, it0, it1 - it0, [&](f32x16 (&acc)[TM][TN]) {
       bool finish = (it0 == 0 && it1 == g.iters_per_tile);
       if (!finish) {
         // slot 0 of a workgroup: the tile it starts in; slot 1: a tile it enters from the left

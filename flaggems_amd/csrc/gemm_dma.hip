@@ -18,12 +18,13 @@ bool dma_supported(const GemmArgs& g, int elem_bytes) {
   return false;
 }
 
-template <typename T, bool B_KC, int BM, int BN>
+template <typename T, bool B_KC, int BM, int BN, int NS>
 static int launch_dma_t(const GemmArgs& g, hipStream_t st) {
-  constexpr int LDS = dma_lds_bytes(BM, BN);
+  constexpr int LDS = dma_lds_bytes(BM, BN, NS);
+  static_assert(LDS <= 160 * 1024, "LDS of one CU");
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kern = gemm_dma_kernel<T, B_KC, BM, BN>;
+  auto kern = gemm_dma_kernel<T, B_KC, BM, BN, NS>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   });
@@ -36,37 +37,78 @@ static int launch_dma_t(const GemmArgs& g, hipStream_t st) {
   return fg_check_launch("gemm");
 }
 
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, int NS>
 static int launch_dma_b(const GemmArgs& g, hipStream_t st) {
-  return g.sbk == 1 ? launch_dma_t<T, true, BM, BN>(g, st) : launch_dma_t<T, false, BM, BN>(g, st);
+  return g.sbk == 1 ? launch_dma_t<T, true, BM, BN, NS>(g, st) : launch_dma_t<T, false, BM, BN, NS>(g, st);
 }
 
-// Tile choice: the candidate whose busiest CU finishes first.  A CU runs ceil(tiles / CUs) tiles; a tile
-// costs its area over its efficiency relative to the 256x256 tile (the smaller tiles read more LDS bytes
-// per flop).  Two 128x128 workgroups share a CU and overlap well; one alone leaves the matrix cores idle
-// while it waits.  The efficiencies are measured on MI355X (1024..8192-row problems).
-void dma_pick_tile(int64_t M, int64_t N, int num_cu, int* bm, int* bn) {
-  *bm = 256; *bn = 256;
-  if (const char* e = getenv("FG_GEMM_TILE")) {  // measurement aid: "256x256" | "256x128" | "128x128"
+// Duration model of a data-parallel launch, in microseconds.  A CU holds one workgroup (two for the two-stage
+// 128x128 kernel), so the tiles run in rounds of num_cu; a K step of one round costs `lone` when few CUs are busy
+// and `loaded` when all are (the matrix cores then share the power budget), in between in proportion to the fill.
+// Constants measured on MI355X, bf16, weights not resident in the caches (1024..4096-row problems, K = 4096 and 11008).
+struct DmaTileCost { int bm, bn; bool deep; double lone, loaded; };
+static const DmaTileCost kDmaTiles[] = {
+    {256, 256, false, 1.30, 1.72},
+    {256, 128, true, 0.73, 0.94},
+    {128, 128, true, 0.58, 0.60},
+};
+static double dma_dp_cost(const DmaTileCost& t, int64_t M, int64_t N, int64_t K, int num_cu) {
+  const int64_t tiles = fg_cdiv(M, t.bm) * fg_cdiv(N, t.bn);
+  const int64_t full = tiles / num_cu, last = tiles % num_cu;
+  double steps = (double)full * t.loaded;
+  if (last > 0) steps += t.lone + (t.loaded - t.lone) * (double)last / num_cu;
+  return steps * (double)(K / kDmaBK);
+}
+
+// Tile choice: the candidate the model above finishes first.  Returns its estimated duration.
+double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep) {
+  if (const char* e = getenv("FG_GEMM_TILE")) {  // measurement aid: "256x256" | "256x128" | "128x128", "s" appended = two stages
     int a = 0, b = 0;
-    if (sscanf(e, "%dx%d", &a, &b) == 2 && (a == 256 || a == 128) && (b == 256 || b == 128) && a >= b) {
-      *bm = a; *bn = b;
-      return;
+    char c = 0;
+    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && (a == 256 || a == 128) && (b == 256 || b == 128) && a >= b) {
+      *bm = a; *bn = b; *deep = c != 's';
+      return 0.0;
     }
   }
-  auto per_cu = [&](int tm, int tn) { return (double)fg_cdiv(fg_cdiv(M, tm) * fg_cdiv(N, tn), (int64_t)num_cu); };
-  const double c256 = per_cu(256, 256);
-  const double c256x128 = per_cu(256, 128) * 0.5 / 0.90;
-  const double t128 = per_cu(128, 128);
-  const double c128 = 0.25 * (2.0 * (double)((int64_t)t128 / 2) / 0.86 + (double)((int64_t)t128 % 2) / 0.63);
-  double best = c256;
-  if (c256x128 < best) { best = c256x128; *bm = 256; *bn = 128; }
-  if (c128 < best) { best = c128; *bm = 128; *bn = 128; }
+  double best = 0.0;
+  bool have = false;
+  for (const DmaTileCost& t : kDmaTiles) {
+    const double c = dma_dp_cost(t, M, N, K, num_cu);
+    if (!have || c < best) { best = c; *bm = t.bm; *bn = t.bn; *deep = t.deep; have = true; }
+  }
+  return best;
 }
 
-// g.tiles_m / g.tiles_n must describe bm x bn tiles.
-int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st) {
-#define FG_DMA(T) (bm == 256 && bn == 256 ? launch_dma_b<T, 256, 256>(g, st) : bm == 256 ? launch_dma_b<T, 256, 128>(g, st) : launch_dma_b<T, 128, 128>(g, st))
+// Stream-K on 128x128 tiles: how many workgroups share the `sk_tiles` cooperative tiles, and the estimated duration of
+// that launch in microseconds.  Either every CU takes an equal share of the K steps (tile boundaries then fall
+// inside the shares: a workgroup restarts its pipeline in a second tile and more tiles need a fix-up), or each tile
+// is cut into s equal parts, s a divisor of the K steps per tile, on sk_tiles * s <= num_cu workgroups.  Measured:
+// ~20 us of launch, first fetch and fix-up (~10 us less when no tile is shared at all) and 0.42 us per K step for
+// the aligned cut.  With equal shares the workgroups of one tile row read different K ranges at the same time, L2
+// reuse drops and the launch can turn bandwidth-bound: ~7 us more and 0.6 us per K step.
+double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, int* workers) {
+  const int64_t total = sk_tiles * iters_per_tile;
+  if (total <= 0) { *workers = 0; return 0.0; }
+  int64_t w = total < num_cu ? total : num_cu;
+  const bool aligned = total % w == 0 && ((total / w) % iters_per_tile == 0 || iters_per_tile % (total / w) == 0);
+  double best = aligned ? 20.0 + 0.42 * (double)(total / w) : 27.0 + 0.6 * (double)fg_cdiv(total, w);
+  *workers = (int)w;
+  if (getenv("FG_GEMM_SK_EVEN") != nullptr) return best;  // measurement and test aid: always equal shares
+  for (int64_t s = 1; s <= iters_per_tile && sk_tiles * s <= num_cu; ++s) {
+    if (iters_per_tile % s != 0) continue;
+    const double c = (s == 1 ? 10.0 : 20.0) + 0.42 * (double)(iters_per_tile / s);
+    if (c < best) { best = c; *workers = (int)(sk_tiles * s); }
+  }
+  return best;
+}
+
+// g.tiles_m / g.tiles_n must describe bm x bn tiles.  `deep`: as many LDS stages as one workgroup per CU can
+// hold (3 for 256x128, 4 for 128x128) instead of two.
+int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st) {
+#define FG_DMA(T)                                                                                       \
+  (bm == 256 && bn == 256 ? launch_dma_b<T, 256, 256, 2>(g, st)                                         \
+   : bm == 256 ? (deep ? launch_dma_b<T, 256, 128, 3>(g, st) : launch_dma_b<T, 256, 128, 2>(g, st))     \
+               : (deep ? launch_dma_b<T, 128, 128, 4>(g, st) : launch_dma_b<T, 128, 128, 2>(g, st)))
   if (dtype == FG_BF16) return FG_DMA(bf16_t);
   return FG_DMA(f16_t);
 #undef FG_DMA
@@ -77,24 +119,24 @@ int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st) {
 // is less than a wave of them) are shared K step by K step between one workgroup per CU; full waves in front of
 // them run data-parallel.  `g` must satisfy dma_supported(); the workspace is the one streamk_workspace_bytes()
 // sizes (tickets + two partial tiles per workgroup).
-template <typename T, bool B_KC>
+template <typename T, bool B_KC, int NS>
 static int launch_dma_streamk_t(const GemmArgs& g, int dp_tiles, hipStream_t st) {
-  constexpr int LDS = dma_lds_bytes(128, 128);
+  constexpr int LDS = dma_lds_bytes(128, 128, 2), LDS_SK = dma_lds_bytes(128, 128, NS);
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto dp = gemm_dma_kernel<T, B_KC, 128, 128>;
-  auto sk = gemm_dma_streamk_kernel<T, B_KC>;
+  auto dp = gemm_dma_kernel<T, B_KC, 128, 128, 2>;
+  auto sk = gemm_dma_streamk_kernel<T, B_KC, NS>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(dp), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (attr_err == hipSuccess)
-      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(sk), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(sk), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_SK);
   });
   if (attr_err != hipSuccess) {
     fg_set_error("gemm(stream-K): cannot reserve %d bytes of LDS: %s", LDS, hipGetErrorString(attr_err));
     return FG_ERR_LAUNCH;
   }
   if (dp_tiles > 0) hipLaunchKernelGGL(dp, dim3((unsigned)dp_tiles), dim3(256), LDS, st, g);
-  if (g.sk_tiles > 0) hipLaunchKernelGGL(sk, dim3((unsigned)g.sk_workers), dim3(256), LDS, st, g);
+  if (g.sk_tiles > 0) hipLaunchKernelGGL(sk, dim3((unsigned)g.sk_workers), dim3(256), LDS_SK, st, g);
   return fg_check_launch("gemm(stream-K)");
 }
 
@@ -112,8 +154,8 @@ int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_
   int64_t sk_tiles = 0;
   fg_streamk_partition(tiles, g.iters_per_tile, num_cu, &sk_tiles, nullptr, nullptr);
   const int64_t total_iters = sk_tiles * g.iters_per_tile;
-  int workers = num_cu;
-  if (total_iters < workers) workers = (int)total_iters;
+  int workers = 0;
+  dma_streamk_plan(sk_tiles, g.iters_per_tile, num_cu, &workers);
   g.sk_tiles = (int)sk_tiles;
   g.sk_workers = workers;
   g.sk_per = workers > 0 ? total_iters / workers : 0;
@@ -124,9 +166,10 @@ int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_
   g.partials = (float*)(ws + kPartialOffset);
   const int dp_tiles = (int)(tiles - sk_tiles);
   const bool kc = g.sbk == 1;
+  // one workgroup per CU: all of its LDS goes into a four-stage ring
   if (dtype == FG_BF16)
-    return kc ? launch_dma_streamk_t<bf16_t, true>(g, dp_tiles, st) : launch_dma_streamk_t<bf16_t, false>(g, dp_tiles, st);
-  return kc ? launch_dma_streamk_t<f16_t, true>(g, dp_tiles, st) : launch_dma_streamk_t<f16_t, false>(g, dp_tiles, st);
+    return kc ? launch_dma_streamk_t<bf16_t, true, 4>(g, dp_tiles, st) : launch_dma_streamk_t<bf16_t, false, 4>(g, dp_tiles, st);
+  return kc ? launch_dma_streamk_t<f16_t, true, 4>(g, dp_tiles, st) : launch_dma_streamk_t<f16_t, false, 4>(g, dp_tiles, st);
 }
 
 }  // namespace fgk

@@ -165,8 +165,12 @@ SK_CASES = [
     (495, 5333, 71, _C.SCHED_STREAM_K), (640, 640, 8192, _C.SCHED_AUTO), (128, 128, 64, _C.SCHED_STREAM_K),
     # ... and the same schedule on the direct-to-LDS main loop (aligned operands, K a multiple of 64): less than
     # a wave of tiles (chosen automatically), ragged edges with bias, full waves in front of the shared tiles
-    (512, 4096, 4096, _C.SCHED_AUTO), (256, 4096, 1024, _C.SCHED_AUTO), (1000, 1304, 2048, _C.SCHED_STREAM_K),
+    (512, 4096, 4096, _C.SCHED_AUTO), (256, 4096, 1024, _C.SCHED_STREAM_K), (1000, 1304, 2048, _C.SCHED_STREAM_K),
     (3000, 4104, 1024, _C.SCHED_STREAM_K), (130, 136, 64, _C.SCHED_STREAM_K),
+    # ... tiles cut into equal parts on fewer workgroups than CUs (96 tiles in halves, 24 tiles in eighths, 43 K steps
+    # per tile left whole), and K steps that no divisor spreads well (equal shares across tile boundaries)
+    (384, 4096, 4096, _C.SCHED_STREAM_K), (384, 1024, 8192, _C.SCHED_AUTO), (1024, 2048, 2752, _C.SCHED_STREAM_K),
+    (200, 1000, 2752, _C.SCHED_STREAM_K),
 ]
 
 
@@ -191,6 +195,29 @@ def test_stream_k(gpu, M, N, K, schedule, dtype, b_col_major):
     for _ in range(10):
         e = torch.empty_like(c)
         _gemm.gemm(a, b, bias, e, 0.5, 2.0, schedule=schedule)
+        assert torch.equal(c, e)
+
+
+# The direct-to-LDS stream-K kernel normally cuts tiles into equal parts; with FG_GEMM_SK_EVEN set it deals equal
+# shares of the K steps to all CUs instead, so shares cross tile boundaries (two partial tiles per workgroup,
+# three or four contributors per tile).
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(384, 4096, 4096), (640, 4096, 2752), (1000, 1304, 2048), (3000, 4104, 1024), (200, 1000, 2752)])
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_stream_k_equal_shares(gpu, monkeypatch, M, N, K, dtype, b_col_major):
+    monkeypatch.setenv("FG_GEMM_SK_EVEN", "1")
+    torch.manual_seed(4)
+    a = torch.randn(M, K, dtype=dtype, device=gpu) / K ** 0.5
+    b = _operand(K, N, dtype, gpu, b_col_major) / K ** 0.5
+    bias = torch.randn(N, dtype=dtype, device=gpu).broadcast_to(M, N)
+    ref = O.mm(a, b) * 0.5 + bias.double().cpu() * 2.0
+    c = torch.empty(M, N, dtype=dtype, device=gpu)
+    _gemm.gemm(a, b, bias, c, 0.5, 2.0, schedule=_C.SCHED_STREAM_K)
+    assert _gemm.last_schedule() == _C.SCHED_STREAM_K
+    gems_assert_close(c, ref, dtype, reduce_dim=K)
+    for _ in range(10):
+        e = torch.empty_like(c)
+        _gemm.gemm(a, b, bias, e, 0.5, 2.0, schedule=_C.SCHED_STREAM_K)
         assert torch.equal(c, e)
 
 
@@ -236,11 +263,13 @@ def test_mm_addmm_large_tiles(gpu, M, N, K, dtype, b_col_major):
 
 
 # The direct-to-LDS kernel exists for three tile sizes; the library picks by how the tile count fills the
-# machine.  Each is forced in turn on ragged shapes (edge tiles in M and N, one to several K steps) and, with
-# no forcing, on shapes whose automatic choice is the 128x128 and the 256x128 tile.
+# machine.  Each is forced in turn on ragged shapes (edge tiles in M and N; one to four K steps, which is fewer
+# than or as many as the LDS ring has stages, and seventeen) and, with no forcing, on shapes whose automatic
+# choice is the 128x128 and the 256x128 tile.  The two smaller tiles run with a ring of four / three stages;
+# an "s" appended forces their two-stage variants.
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tile", ["256x256", "256x128", "128x128", None])
-@pytest.mark.parametrize("M,N,K", [(1024, 4096, 128), (1100, 4104, 64), (2040, 4104, 256), (1537, 2824, 192)])
+@pytest.mark.parametrize("tile", ["256x256", "256x128", "128x128", "256x128s", "128x128s", None])
+@pytest.mark.parametrize("M,N,K", [(1024, 4096, 128), (1100, 4104, 64), (2040, 4104, 256), (1537, 2824, 192), (1100, 2824, 1088)])
 @pytest.mark.parametrize("b_col_major", [False, True])
 def test_mm_addmm_tile_sizes(gpu, monkeypatch, M, N, K, dtype, tile, b_col_major):
     if tile is None:
