@@ -233,7 +233,7 @@ def main():
                      cpu=(cpu, cw, "torch.mm on the host in fp32, first %d rows of A" % rows))
             d["post"] = lambda: {"schedule": {1: "data-parallel", 2: "stream-K"}.get(_gemm.last_schedule())}
             if (M, N, K) == (8192, 8192, 8192) and not b_t and not bias:
-                d["traffic"] = 1781420000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
+                d["traffic"] = 1771500000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
             return d
         return make
 
@@ -280,7 +280,7 @@ def main():
         def cpu():
             O.paged_attention(qc, kcc, vcc, [ls], [ls], btc, D ** -0.5, compute_dtype=torch.float32)
 
-        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1835020000,
+        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1835830000,
                     workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
                     cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
 
@@ -433,6 +433,10 @@ def main():
         "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),
         "mm_c3b_skinny_nt": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, B = W^T of a [N, K] weight, stream-K",
                                   b_t=True, bound="hbm"),
+        "mm_chunk_1024_nt": wl_mm(1024, 12288, 4096, "mm bf16 M=1024 N=12288 K=4096, B = W^T (a 1024-token prefill chunk "
+                                  "through a fused QKV weight: less than one round of 256x256 tiles)", b_t=True),
+        "mm_chunk_512_nt": wl_mm(512, 4096, 4096, "mm bf16 M=512 N=4096 K=4096, B = W^T (half a round of 128x128 tiles: "
+                                 "each tile cut in two)", b_t=True),
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "flash_attn_decode": wl_decode,
