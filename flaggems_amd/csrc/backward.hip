@@ -319,6 +319,28 @@ __global__ __launch_bounds__(256) void rms_dw_partial_kernel(const T* __restrict
   partial[(int64_t)blockIdx.x * N + c] = s;
 }
 
+// Column sums of the partial rows: out[c] = sum over r of partial[r, c], rounded once to T.  A workgroup owns 32
+// columns (one 128-byte line per row); its 32 row lanes each add every 32nd row, then lane 0 adds the 32 sums in
+// order, so the result does not depend on timing.
+template <typename T>
+__global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restrict__ partial, T* __restrict__ out,
+                                                          int64_t rows, int64_t N) {
+  __shared__ float part[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t c = (int64_t)blockIdx.x * 32 + tx;
+  float s = 0.f;
+  if (c < N)
+    for (int64_t r = ty; r < rows; r += 32) s += partial[r * N + c];
+  part[ty][tx] = s;
+  __syncthreads();
+  if (ty == 0 && c < N) {
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) t += part[i][tx];
+    out[c] = (T)t;
+  }
+}
+
 template <typename TI, typename TO, int VEC, int ITERS, int TPR, int MODE>
 void launch_rows(const TI* a, const TI* g, TO* out, int64_t M, int N, hipStream_t st) {
   constexpr int BLOCK = TPR < 256 ? 256 : TPR;
@@ -468,6 +490,32 @@ extern "C" int64_t fg_rms_norm_backward_partial_rows(int64_t M, int64_t N, int d
   int64_t rows_per_group = fg_cdiv(M, target);
   rows_per_group = rows_per_group < 8 ? 8 : rows_per_group > 64 ? 64 : rows_per_group;
   return fg_cdiv(M, rows_per_group);
+}
+
+extern "C" int fg_rms_norm_backward_dw(const float* dw_partial, int64_t partial_rows, int64_t N, void* dw, int dtype,
+                                       void* stream) {
+  FG_REQUIRE(partial_rows >= 0 && N >= 0, FG_ERR_INVALID, "rms_norm_backward_dw: negative size");
+  if (N == 0) return FG_OK;
+  FG_REQUIRE(dw && (dw_partial || partial_rows == 0), FG_ERR_INVALID, "rms_norm_backward_dw: null pointer");
+  FG_REQUIRE(fg_cdiv(N, 32) < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "rms_norm_backward_dw: N=%lld too large",
+             (long long)N);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)fg_cdiv(N, 32));
+  switch (dtype) {
+    case FG_F16:
+      hipLaunchKernelGGL(column_sum_kernel<f16_t>, grid, dim3(1024), 0, st, dw_partial, (f16_t*)dw, partial_rows, N);
+      break;
+    case FG_BF16:
+      hipLaunchKernelGGL(column_sum_kernel<bf16_t>, grid, dim3(1024), 0, st, dw_partial, (bf16_t*)dw, partial_rows, N);
+      break;
+    case FG_F32:
+      hipLaunchKernelGGL(column_sum_kernel<float>, grid, dim3(1024), 0, st, dw_partial, (float*)dw, partial_rows, N);
+      break;
+    default:
+      fg_set_error("rms_norm_backward_dw: bad dtype %d", dtype);
+      return FG_ERR_INVALID;
+  }
+  return fg_check_launch("rms_norm_backward_dw");
 }
 
 extern "C" int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,

@@ -45,7 +45,7 @@ def _forward(x, normalized_shape, weight, eps, want_inv_rms):
 
 class RmsNorm(torch.autograd.Function):
     """Forward saves x and the per-row 1/rms; backward is one kernel that writes dx and, when the weight needs
-    a gradient, fp32 partial column sums (one row per group of rows) that torch.sum adds up (the reference
+    a gradient, fp32 partial column sums (one row per group of rows) that a second small kernel adds up (the reference
     uses a kernel per gradient, src/flag_gems/ops/rms_norm.py:149-218)."""
 
     @staticmethod
@@ -83,11 +83,15 @@ class RmsNorm(torch.autograd.Function):
                 dx.data_ptr(), partial.data_ptr() if partial is not None else None, partial_rows,
                 M, N, _C.dtype_id(x.dtype), _C.current_stream(x.device),
             )
-        _C.check(rc, "fg_rms_norm_backward")
-        dw = None
-        if want_dw:
-            # added up in fp32 and rounded once (the reference rounds the partial rows to x.dtype first)
-            dw = torch.sum(partial, dim=0).to(x.dtype).reshape(weight.shape)
+            _C.check(rc, "fg_rms_norm_backward")
+            dw = None
+            if want_dw:
+                # added up in fp32 and rounded once (the reference rounds the partial rows to x.dtype first)
+                dw = torch.empty(weight.shape, dtype=x.dtype, device=x.device)
+                rc = lib.fg_rms_norm_backward_dw(
+                    partial.data_ptr(), partial_rows, N, dw.data_ptr(), _C.dtype_id(x.dtype), _C.current_stream(x.device)
+                )
+                _C.check(rc, "fg_rms_norm_backward_dw")
         return dx, None, dw, None
 
 

@@ -96,12 +96,16 @@ int fg_log_softmax_backward(const void* out, const void* grad_out, void* grad_in
  * When dw_partial is non-NULL it is fp32 [partial_rows, N], 32-byte aligned, 1 <= partial_rows <= M: row p
  * receives the sums of x * dy * inv_rms over rows [p * ceil(M / partial_rows), ...); the column sum of
  * dw_partial is the weight gradient.  fg_rms_norm_backward_partial_rows proposes a partial_rows that fills
- * the device.  One kernel computes both gradients (x and dy are read once).
+ * the device.  One kernel computes both gradients (x and dy are read once).  fg_rms_norm_backward_dw adds the
+ * rows of dw_partial up in fp32, in a fixed order, and writes the weight gradient dw [N] in `dtype`, rounded once
+ * (the reference rounds its partial rows to the input dtype and sums them with torch.sum, rms_norm.py:205-218).
  * Replaces rms_norm_grad_dx_kernel and rms_norm_grad_dw_kernel, src/flag_gems/ops/rms_norm.py:54-146,171-218. */
 int64_t fg_rms_norm_backward_partial_rows(int64_t M, int64_t N, int dtype, int device);
 int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, const void* w, void* dx,
                          float* dw_partial, int64_t partial_rows, int64_t M, int64_t N, int dtype,
                          void* stream);
+int fg_rms_norm_backward_dw(const float* dw_partial, int64_t partial_rows, int64_t N, void* dw, int dtype,
+                            void* stream);
 
 /* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
  * {token, head, dim}); cos/sin [max_pos, D/2] with unit inner stride.  pos == NULL means

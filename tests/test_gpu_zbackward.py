@@ -111,3 +111,29 @@ def test_rms_norm_backward_variants(gpu):
     # without a graph the forward kernel alone runs and nothing is saved
     with torch.no_grad():
         assert not flag_gems.rms_norm(x, [96], None, 1e-6).requires_grad
+
+
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("rows,N", [(1, 32), (7, 33), (32, 4096), (100, 1000), (1024, 4096), (513, 8200), (0, 64)])
+def test_rms_norm_backward_dw_column_sum(gpu, rows, N, dtype):
+    """fg_rms_norm_backward_dw through the C ABI: fp32 column sums of the partial rows, rounded once to the
+    output dtype, identical from call to call."""
+    from flaggems_amd import _C
+
+    torch.manual_seed(rows + N)
+    partial = torch.randn(rows, N, dtype=torch.float32, device=gpu) * 3.0
+    lib = _C.lib()
+    outs = []
+    for _ in range(3):
+        dw = torch.full((N,), float("nan"), dtype=dtype, device=gpu)
+        rc = lib.fg_rms_norm_backward_dw(partial.data_ptr() if rows else None, rows, N, dw.data_ptr(), _C.dtype_id(dtype),
+                                         _C.current_stream(dw.device))
+        assert rc == 0, _C.last_error()
+        outs.append(dw)
+    ref = partial.double().sum(0).cpu()
+    # fp32 accumulation of `rows` terms of size ~3, then one rounding to dtype
+    eps = {torch.float16: 1e-3, torch.bfloat16: 7.8e-3, torch.float32: 1.2e-7}[dtype]
+    err = (outs[0].double().cpu() - ref).abs()
+    bound = ref.abs() * eps + 1e-5 * max(rows, 1)
+    assert bool((err <= bound).all()), float((err - bound).max())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
