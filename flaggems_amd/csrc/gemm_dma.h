@@ -394,17 +394,36 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
             for (int j = 0; j < TN; ++j)
 #pragma unroll
               for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-          for (int w2 = w_first; w2 <= w_last; ++w2) {
-            const float* src =
-                g.partials + ((int64_t)w2 * 2 + (sk_begin(g.sk_per, g.sk_rem, w2) < tile_begin ? 1 : 0)) * (BM * BN);
+          auto slot_of = [&](int w2) {
+            return g.partials + ((int64_t)w2 * 2 + (sk_begin(g.sk_per, g.sk_rem, w2) < tile_begin ? 1 : 0)) * (BM * BN) + tid;
+          };
+          // contributors in workgroup order, two at a time: both partial tiles are requested before either is added,
+          // so a pair costs one trip to memory
+          int w2 = w_first;
+          for (; w2 < w_last; w2 += 2) {
+            const float* s0 = slot_of(w2);
+            const float* s1 = slot_of(w2 + 1);
+            float t0[TM * TN * 16], t1[TM * TN * 16];
+#pragma unroll
+            for (int x = 0; x < TM * TN * 16; ++x) t0[x] = __hip_atomic_load(s0 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int x = 0; x < TM * TN * 16; ++x) t1[x] = __hip_atomic_load(s1 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = (acc[i][j][e] + t0[(i * TN + j) * 16 + e]) + t1[(i * TN + j) * 16 + e];
+          }
+          if (w2 == w_last) {
+            const float* s0 = slot_of(w2);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
               for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                  acc[i][j][e] += __hip_atomic_load(src + ((i * TN + j) * 16 + e) * 256 + tid, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
+                  acc[i][j][e] += __hip_atomic_load(s0 + ((i * TN + j) * 16 + e) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
           if (tid == 0) __hip_atomic_store(g.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
