@@ -42,30 +42,40 @@ static int launch_dma_b(const GemmArgs& g, hipStream_t st) {
   return g.sbk == 1 ? launch_dma_t<T, true, BM, BN, NS>(g, st) : launch_dma_t<T, false, BM, BN, NS>(g, st);
 }
 
-// Duration model of a data-parallel launch, in microseconds.  A CU holds one workgroup (two for the two-stage
-// 128x128 kernel), so the tiles run in rounds of num_cu; a K step of one round costs `lone` when few CUs are busy
-// and `loaded` when all are (the matrix cores then share the power budget), in between in proportion to the fill.
-// Constants measured on MI355X, bf16, weights not resident in the caches (1024..4096-row problems, K = 4096 and 11008).
+// Duration model of a data-parallel launch, in microseconds.  A CU holds one workgroup, so the tiles run in rounds
+// of num_cu.  A K step of a round that is the whole launch costs `lone` when few CUs are busy and `loaded` when all
+// are (the matrix cores then share the power budget); in between the cost follows the cube of the fill (half a round
+// still runs at the lone rate).  A ragged round behind full ones starts while their stragglers finish: it adds
+// 0.55 to 1.0 of a lone round on top of that.  Constants measured on MI355X, bf16, K = 4096, weights not resident in
+// the caches, 16 to 512 tiles of each size.
 struct DmaTileCost { int bm, bn; bool deep; double lone, loaded; };
 static const DmaTileCost kDmaTiles[] = {
-    {256, 256, false, 1.30, 1.72},
-    {256, 128, true, 0.73, 0.94},
-    {128, 128, true, 0.58, 0.60},
+    {256, 256, false, 1.31, 1.75},
+    {192, 256, false, 1.20, 1.375},
+    {256, 128, true, 0.77, 0.97},
+    {128, 256, true, 0.84, 1.00},
+    {128, 128, true, 0.58, 0.59},
 };
 static double dma_dp_cost(const DmaTileCost& t, int64_t M, int64_t N, int64_t K, int num_cu) {
   const int64_t tiles = fg_cdiv(M, t.bm) * fg_cdiv(N, t.bn);
   const int64_t full = tiles / num_cu, last = tiles % num_cu;
+  const double f = (double)last / num_cu;
   double steps = (double)full * t.loaded;
-  if (last > 0) steps += t.lone + (t.loaded - t.lone) * (double)last / num_cu;
+  if (last > 0) steps += (full > 0 ? t.lone * (0.55 + 0.45 * f) : t.lone) + (t.loaded - t.lone) * f * f * f;
   return steps * (double)(K / kDmaBK);
+}
+static bool dma_tile_exists(int bm, int bn) {
+  for (const DmaTileCost& t : kDmaTiles)
+    if (t.bm == bm && t.bn == bn) return true;
+  return false;
 }
 
 // Tile choice: the candidate the model above finishes first.  Returns its estimated duration.
 double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep) {
-  if (const char* e = getenv("FG_GEMM_TILE")) {  // measurement aid: "256x256" | "256x128" | "128x128", "s" appended = two stages
+  if (const char* e = getenv("FG_GEMM_TILE")) {  // measurement aid: one of the tiles above as "256x128"; "s" appended = two stages
     int a = 0, b = 0;
     char c = 0;
-    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && (a == 256 || a == 128) && (b == 256 || b == 128) && a >= b) {
+    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && dma_tile_exists(a, b)) {
       *bm = a; *bn = b; *deep = c != 's';
       return 0.0;
     }
@@ -103,15 +113,21 @@ double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, in
 }
 
 // g.tiles_m / g.tiles_n must describe bm x bn tiles.  `deep`: as many LDS stages as one workgroup per CU can
-// hold (3 for 256x128, 4 for 128x128) instead of two.
+// hold (3 for 256x128 and 128x256, 4 for 128x128) instead of two.
 int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st) {
-#define FG_DMA(T)                                                                                       \
-  (bm == 256 && bn == 256 ? launch_dma_b<T, 256, 256, 2>(g, st)                                         \
-   : bm == 256 ? (deep ? launch_dma_b<T, 256, 128, 3>(g, st) : launch_dma_b<T, 256, 128, 2>(g, st))     \
-               : (deep ? launch_dma_b<T, 128, 128, 4>(g, st) : launch_dma_b<T, 128, 128, 2>(g, st)))
-  if (dtype == FG_BF16) return FG_DMA(bf16_t);
-  return FG_DMA(f16_t);
+#define FG_DMA(T)                                                                                         \
+  do {                                                                                                    \
+    if (bm == 256 && bn == 256) return launch_dma_b<T, 256, 256, 2>(g, st);                               \
+    if (bm == 192 && bn == 256) return launch_dma_b<T, 192, 256, 2>(g, st);                               \
+    if (bm == 256 && bn == 128) return deep ? launch_dma_b<T, 256, 128, 3>(g, st) : launch_dma_b<T, 256, 128, 2>(g, st); \
+    if (bm == 128 && bn == 256) return deep ? launch_dma_b<T, 128, 256, 3>(g, st) : launch_dma_b<T, 128, 256, 2>(g, st); \
+    if (bm == 128 && bn == 128) return deep ? launch_dma_b<T, 128, 128, 4>(g, st) : launch_dma_b<T, 128, 128, 2>(g, st); \
+  } while (0)
+  if (dtype == FG_BF16) FG_DMA(bf16_t);
+  else FG_DMA(f16_t);
 #undef FG_DMA
+  fg_set_error("gemm: no direct-to-LDS kernel for %d x %d tiles", bm, bn);
+  return FG_ERR_UNSUPPORTED;
 }
 
 

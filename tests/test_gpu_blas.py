@@ -262,13 +262,13 @@ def test_mm_addmm_large_tiles(gpu, M, N, K, dtype, b_col_major):
     gems_assert_close(out[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
 
 
-# The direct-to-LDS kernel exists for three tile sizes; the library picks by how the tile count fills the
+# The direct-to-LDS kernel exists for five tile sizes; the library picks by how the tile count fills the
 # machine.  Each is forced in turn on ragged shapes (edge tiles in M and N; one to four K steps, which is fewer
 # than or as many as the LDS ring has stages, and seventeen) and, with no forcing, on shapes whose automatic
 # choice is the 128x128 and the 256x128 tile.  The two smaller tiles run with a ring of four / three stages;
 # an "s" appended forces their two-stage variants.
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tile", ["256x256", "256x128", "128x128", "256x128s", "128x128s", None])
+@pytest.mark.parametrize("tile", ["256x256", "192x256", "256x128", "128x256", "128x128", "256x128s", "128x256s", "128x128s", None])
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 128), (1100, 4104, 64), (2040, 4104, 256), (1537, 2824, 192), (1100, 2824, 1088)])
 @pytest.mark.parametrize("b_col_major", [False, True])
 def test_mm_addmm_tile_sizes(gpu, monkeypatch, M, N, K, dtype, tile, b_col_major):
