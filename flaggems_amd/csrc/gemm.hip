@@ -72,10 +72,24 @@ int launch_dp_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
     if (amode == LOAD_K && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_K, LOAD_MN>(g, st);
     if (amode == LOAD_MN && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_MN, LOAD_K>(g, st);
     if (amode == LOAD_MN && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_MN, LOAD_MN>(g, st);
+    // operands contiguous along one axis but not aligned for the modes above
+    if (amode == LOAD_KU && bmode == LOAD_KU) return launch_dp<T, BM, BN, LOAD_KU, LOAD_KU>(g, st);
+    if (amode == LOAD_KU && bmode == LOAD_MNU) return launch_dp<T, BM, BN, LOAD_KU, LOAD_MNU>(g, st);
+    if (amode == LOAD_MNU && bmode == LOAD_KU) return launch_dp<T, BM, BN, LOAD_MNU, LOAD_KU>(g, st);
+    if (amode == LOAD_MNU && bmode == LOAD_MNU) return launch_dp<T, BM, BN, LOAD_MNU, LOAD_MNU>(g, st);
   } else {
     if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
+    if (amode == LOAD_KU && bmode == LOAD_KU) return launch_dp<T, BM, BN, LOAD_KU, LOAD_KU>(g, st);
   }
   return launch_dp<T, BM, BN, LOAD_GEN, LOAD_GEN>(g, st);
+}
+
+// Load mode of an operand that pick_mode() turned away: the element-aligned vector modes when it is contiguous
+// along K or along its row index, element-wise otherwise.
+int pick_mode_unaligned(int64_t rows, int64_t K, int64_t s_row, int64_t s_k, int elem_bytes) {
+  if (s_k == 1 || K == 1) return LOAD_KU;
+  if (elem_bytes == 2 && (s_row == 1 || rows == 1)) return LOAD_MNU;
+  return LOAD_GEN;
 }
 
 // Load mode of an operand whose element (row, k) lives at base[row*s_row + k*s_k].
@@ -109,7 +123,7 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
     }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
-    if (amode != LOAD_GEN && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
+    if (amode != LOAD_GEN && amode != LOAD_KU && amode != LOAD_MNU && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
       set_tiles(g, 256, 256, BK);
       return launch_dp_modes<T, 256, 256>(g, amode, bmode, st);
     }
@@ -182,8 +196,14 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
   const int eb = ab_dtype == FG_F32 ? 4 : 2;
   int amode = pick_mode(A, M, K, sam, sak, eb);
   int bmode = pick_mode(B, N, K, sbn, sbk, eb);
-  if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_K || bmode != LOAD_K)))
-    amode = bmode = LOAD_GEN;
+  if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_K || bmode != LOAD_K))) {
+    // one kernel serves both operands: either both take an element-aligned vector mode or both go element by element
+    amode = pick_mode_unaligned(M, K, sam, sak, eb);
+    bmode = pick_mode_unaligned(N, K, sbn, sbk, eb);
+    if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_KU || bmode != LOAD_KU)))
+      amode = bmode = LOAD_GEN;
+  }
+  const bool vec_unaligned = amode == LOAD_KU || amode == LOAD_MNU;
   const int cu = num_cus(-1);
 
   // ---- schedule --------------------------------------------------------------------------------
@@ -211,7 +231,8 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
             use_streamk = tiles <= cu && tiles * iters >= 4 * (int64_t)cu &&
                           dma_streamk_plan(tiles, iters, cu, &workers) < dma_pick_tile(M, N, K, cu, &bm, &bn, &deep);
           } else {
-            use_streamk = tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;
+            // (the stream-K kernels have no element-aligned vector modes: such operands stay data-parallel)
+            use_streamk = !vec_unaligned && tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;
           }
         }
       }

@@ -18,6 +18,10 @@
 //   LOAD_MN  the operand is contiguous along its M/N index (A column-major, B row-major): each
 //            thread loads an 8(k) x 8(mn) block as eight 16-byte rows, transposes it in registers
 //            with v_perm_b32 and stores eight 16-byte K-runs.  16-bit types only.
+//   LOAD_KU / LOAD_MNU  the same two layouts without the alignment and divisibility conditions (a row stride or
+//            K that is not a multiple of 8 elements, a base that is only element-aligned): the 16-byte loads are
+//            declared element-aligned, and a group that straddles the end of K or of the rows is assembled
+//            element by element, zeros past the end.
 //   LOAD_GEN any strides, any alignment, full bounds checks: element-wise.
 // The vector modes never read out of bounds: row indices are clamped to the last valid row (the
 // duplicate rows are never stored) and 16-byte groups that lie past K are replaced by zeros.
@@ -26,7 +30,7 @@
 
 namespace fgk {
 
-enum { LOAD_K = 0, LOAD_MN = 1, LOAD_GEN = 2 };
+enum { LOAD_K = 0, LOAD_MN = 1, LOAD_GEN = 2, LOAD_KU = 3, LOAD_MNU = 4 };
 
 constexpr int kRowBytes = 128;   // K bytes per tile row per stage
 constexpr int kPitch = 144;      // LDS pitch of a tile row
@@ -146,6 +150,99 @@ template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_MN> {
 #pragma unroll
       for (int rr = 0; rr < 8; ++rr) {
         // K-run of row rr: dword d = { k = 2d (low half), k = 2d + 1 (high half) }
+        const unsigned sel = (rr & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) o[d] = __builtin_amdgcn_perm(r[i][2 * d + 1][rr >> 1], r[i][2 * d][rr >> 1], sel);
+        *reinterpret_cast<u32x4*>(lds + (rb * 8 + rr) * kPitch + kb * 16) = o;
+      }
+    }
+  }
+};
+
+// 16 bytes from an address that is only aligned to the element type.
+template <typename T> __device__ __forceinline__ u32x4 load16_elem_aligned(const T* p) {
+  u32x4 v;
+  __builtin_memcpy(&v, p, 16);
+  return v;
+}
+
+template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_KU> {
+  static constexpr int EPC = 16 / sizeof(T);
+  static constexpr int N = (ROWS * 8 + kThreads - 1) / kThreads;
+  u32x4 r[N];
+  // element (row, k) lives at base[row * s_row + k]
+  __device__ __forceinline__ void fetch(const T* base, int64_t s_row, int64_t /*s_k*/, int row0, int rows_total,
+                                        int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = i * kThreads + tid;
+      const int row = idx >> 3, c = idx & 7;
+      if (ROWS * 8 % kThreads != 0 && idx >= ROWS * 8) continue;
+      int gr = row0 + row;
+      gr = gr < rows_total ? gr : rows_total - 1;
+      const int k = k0 + c * EPC;
+      const T* p = base + (int64_t)gr * s_row + k;
+      if (k + EPC <= K) {
+        r[i] = load16_elem_aligned(p);
+      } else {
+        T e[EPC];
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) e[j] = (k + j < K) ? p[j] : (T)0.0f;
+        u32x4 v;
+        __builtin_memcpy(&v, e, 16);
+        r[i] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = i * kThreads + tid;
+      if (ROWS * 8 % kThreads != 0 && idx >= ROWS * 8) continue;
+      *reinterpret_cast<u32x4*>(lds + (idx >> 3) * kPitch + (idx & 7) * 16) = r[i];
+    }
+  }
+};
+
+template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_MNU> {
+  static_assert(sizeof(T) == 2, "the transposing stager handles 16-bit elements");
+  static constexpr int N = (ROWS + kThreads - 1) / kThreads;  // 8x8 blocks per thread
+  u32x4 r[N][8];
+  // element (row, k) lives at base[k * s_k + row]
+  __device__ __forceinline__ void fetch(const T* base, int64_t /*s_row*/, int64_t s_k, int row0, int rows_total,
+                                        int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int blk = i * kThreads + tid;
+      if (ROWS % kThreads != 0 && blk >= ROWS) continue;
+      const int kb = blk & 7, rb = blk >> 3;
+      const int gr = row0 + rb * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = k0 + kb * 8 + j;
+        const T* p = base + (int64_t)k * s_k + gr;
+        if (k < K && gr + 8 <= rows_total) {
+          r[i][j] = load16_elem_aligned(p);
+        } else {
+          T e[8];
+#pragma unroll
+          for (int rr = 0; rr < 8; ++rr) e[rr] = (k < K && gr + rr < rows_total) ? p[rr] : (T)0.0f;
+          u32x4 v;
+          __builtin_memcpy(&v, e, 16);
+          r[i][j] = v;
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int blk = i * kThreads + tid;
+      if (ROWS % kThreads != 0 && blk >= ROWS) continue;
+      const int kb = blk & 7, rb = blk >> 3;
+#pragma unroll
+      for (int rr = 0; rr < 8; ++rr) {
         const unsigned sel = (rr & 1) ? 0x07060302u : 0x05040100u;
         u32x4 o;
 #pragma unroll

@@ -305,3 +305,32 @@ def test_mm_full_size_properties(gpu):
         gems_assert_close(c[rows], O.mm(a[rows], bb), torch.bfloat16, reduce_dim=n)
         # doubling A doubles C exactly (power-of-two scaling commutes with every rounding)
         assert torch.equal(flag_gems.mm(a * 2, bb), c * 2)
+
+
+def _shifted(rows, cols, dtype, dev, transposed, shift, pad):
+    """A (rows, cols) operand contiguous along cols (along rows when transposed), `shift` elements into its
+    buffer and with `pad` unused elements behind every line: base and row stride only element-aligned."""
+    r, c = (cols, rows) if transposed else (rows, cols)
+    buf = torch.randn(shift + r * (c + pad) + 8, dtype=dtype, device=dev)
+    t = buf[shift:shift + r * (c + pad)].view(r, c + pad)[:, :c]
+    return t.t() if transposed else t
+
+
+# Operands that are contiguous along one axis but miss the alignment of the 16-byte staging modes (K or the row
+# stride not a multiple of 8 elements, a base address that is only element-aligned, ragged row counts): the
+# element-aligned vector modes for 16-bit types (fp32: both operands K-contiguous; else element by element).
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("M,N,K", [(300, 500, 1004), (257, 129, 71), (128, 136, 64), (1, 9, 3), (513, 1001, 130)])
+@pytest.mark.parametrize("b_col_major", [False, True])
+@pytest.mark.parametrize("a_col_major", [False, True])
+@pytest.mark.parametrize("shift,pad", [(0, 0), (3, 5), (1, 0)])
+def test_mm_unaligned_operands(gpu, M, N, K, dtype, a_col_major, b_col_major, shift, pad):
+    torch.manual_seed(M + N + K + shift)
+    a = _shifted(M, K, dtype, gpu, a_col_major, shift, pad)
+    b = _shifted(K, N, dtype, gpu, b_col_major, shift, pad)
+    ref = O.mm(a, b)
+    res = flag_gems.mm(a, b)
+    gems_assert_close(res, ref, dtype, reduce_dim=K)
+    bias = torch.randn(N, dtype=dtype, device=gpu)
+    res = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
+    gems_assert_close(res, O.addmm(bias, a, b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
