@@ -80,15 +80,18 @@ int launch_dp_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
   } else {
     if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
     if (amode == LOAD_KU && bmode == LOAD_KU) return launch_dp<T, BM, BN, LOAD_KU, LOAD_KU>(g, st);
+    if (amode == LOAD_KU && bmode == LOAD_MNU) return launch_dp<T, BM, BN, LOAD_KU, LOAD_MNU>(g, st);
+    if (amode == LOAD_MNU && bmode == LOAD_KU) return launch_dp<T, BM, BN, LOAD_MNU, LOAD_KU>(g, st);
+    if (amode == LOAD_MNU && bmode == LOAD_MNU) return launch_dp<T, BM, BN, LOAD_MNU, LOAD_MNU>(g, st);
   }
   return launch_dp<T, BM, BN, LOAD_GEN, LOAD_GEN>(g, st);
 }
 
 // Load mode of an operand that pick_mode() turned away: the element-aligned vector modes when it is contiguous
 // along K or along its row index, element-wise otherwise.
-int pick_mode_unaligned(int64_t rows, int64_t K, int64_t s_row, int64_t s_k, int elem_bytes) {
+int pick_mode_unaligned(int64_t rows, int64_t K, int64_t s_row, int64_t s_k) {
   if (s_k == 1 || K == 1) return LOAD_KU;
-  if (elem_bytes == 2 && (s_row == 1 || rows == 1)) return LOAD_MNU;
+  if (s_row == 1 || rows == 1) return LOAD_MNU;
   return LOAD_GEN;
 }
 
@@ -198,10 +201,9 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
   int bmode = pick_mode(B, N, K, sbn, sbk, eb);
   if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_K || bmode != LOAD_K))) {
     // one kernel serves both operands: either both take an element-aligned vector mode or both go element by element
-    amode = pick_mode_unaligned(M, K, sam, sak, eb);
-    bmode = pick_mode_unaligned(N, K, sbn, sbk, eb);
-    if (amode == LOAD_GEN || bmode == LOAD_GEN || (eb == 4 && (amode != LOAD_KU || bmode != LOAD_KU)))
-      amode = bmode = LOAD_GEN;
+    amode = pick_mode_unaligned(M, K, sam, sak);
+    bmode = pick_mode_unaligned(N, K, sbn, sbk);
+    if (amode == LOAD_GEN || bmode == LOAD_GEN) amode = bmode = LOAD_GEN;
   }
   const bool vec_unaligned = amode == LOAD_KU || amode == LOAD_MNU;
   const int cu = num_cus(-1);

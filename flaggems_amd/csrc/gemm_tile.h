@@ -21,7 +21,7 @@
 //   LOAD_KU / LOAD_MNU  the same two layouts without the alignment and divisibility conditions (a row stride or
 //            K that is not a multiple of 8 elements, a base that is only element-aligned): the 16-byte loads are
 //            declared element-aligned, and a group that straddles the end of K or of the rows is assembled
-//            element by element, zeros past the end.
+//            element by element, zeros past the end.  LOAD_MNU also exists for 32-bit elements (4 x 4 blocks).
 //   LOAD_GEN any strides, any alignment, full bounds checks: element-wise.
 // The vector modes never read out of bounds: row indices are clamped to the last valid row (the
 // duplicate rows are never stored) and 16-byte groups that lie past K are replaced by zeros.
@@ -206,7 +206,7 @@ template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_KU> {
 };
 
 template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_MNU> {
-  static_assert(sizeof(T) == 2, "the transposing stager handles 16-bit elements");
+  static_assert(sizeof(T) == 2, "16-bit elements; the 32-bit specialization follows");
   static constexpr int N = (ROWS + kThreads - 1) / kThreads;  // 8x8 blocks per thread
   u32x4 r[N][8];
   // element (row, k) lives at base[k * s_k + row]
@@ -249,6 +249,48 @@ template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_MNU> {
         for (int d = 0; d < 4; ++d) o[d] = __builtin_amdgcn_perm(r[i][2 * d + 1][rr >> 1], r[i][2 * d][rr >> 1], sel);
         *reinterpret_cast<u32x4*>(lds + (rb * 8 + rr) * kPitch + kb * 16) = o;
       }
+    }
+  }
+};
+
+// 32-bit elements: a thread takes a 4(k) x 4(mn) block as four 16-byte rows; its transpose is a renaming of registers.
+template <int ROWS> struct Stager<float, ROWS, LOAD_MNU> {
+  static constexpr int N = (ROWS * 2 + kThreads - 1) / kThreads;  // blocks per thread: 8 k-chunks x ROWS/4 row groups
+  u32x4 r[N][4];
+  // element (row, k) lives at base[k * s_k + row]
+  __device__ __forceinline__ void fetch(const float* base, int64_t /*s_row*/, int64_t s_k, int row0, int rows_total,
+                                        int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int blk = i * kThreads + tid;
+      if (ROWS * 2 % kThreads != 0 && blk >= ROWS * 2) continue;
+      const int kb = blk & 7, rb = blk >> 3;
+      const int gr = row0 + rb * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = k0 + kb * 4 + j;
+        const float* p = base + (int64_t)k * s_k + gr;
+        if (k < K && gr + 4 <= rows_total) {
+          r[i][j] = load16_elem_aligned(p);
+        } else {
+          u32x4 v;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) v[rr] = (k < K && gr + rr < rows_total) ? __builtin_bit_cast(uint32_t, p[rr]) : 0u;
+          r[i][j] = v;
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int blk = i * kThreads + tid;
+      if (ROWS * 2 % kThreads != 0 && blk >= ROWS * 2) continue;
+      const int kb = blk & 7, rb = blk >> 3;
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        *reinterpret_cast<u32x4*>(lds + (rb * 4 + rr) * kPitch + kb * 16) =
+            u32x4{r[i][0][rr], r[i][1][rr], r[i][2][rr], r[i][3][rr]};
     }
   }
 };

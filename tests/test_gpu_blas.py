@@ -318,7 +318,7 @@ def _shifted(rows, cols, dtype, dev, transposed, shift, pad):
 
 # Operands that are contiguous along one axis but miss the alignment of the 16-byte staging modes (K or the row
 # stride not a multiple of 8 elements, a base address that is only element-aligned, ragged row counts): the
-# element-aligned vector modes for 16-bit types (fp32: both operands K-contiguous; else element by element).
+# element-aligned vector modes (also what fp32 operands that are contiguous along M or N take).
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
 @pytest.mark.parametrize("M,N,K", [(300, 500, 1004), (257, 129, 71), (128, 136, 64), (1, 9, 3), (513, 1001, 130)])
 @pytest.mark.parametrize("b_col_major", [False, True])
