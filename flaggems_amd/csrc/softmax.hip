@@ -3,8 +3,9 @@
 // Inner axis (K == 1): the row lives in registers as fp32 (TPR threads per row, ITERS packs of VEC
 // elements per thread, same column interleave as the norm kernels), so HBM is read once and
 // written once.  max and sum use wave64 butterflies plus one LDS step when a row spans waves.
-// Rows that do not fit registers, or that defeat 16-byte access, use a looped online-softmax
-// kernel (two reads of the row, the second from L2).
+// Rows that do not fit registers, or whose start is only element-aligned, take a two-sweep online-softmax
+// kernel with one workgroup per row (the second read comes from L2), or, up to 1024 elements, a kernel
+// with one wave per row.
 // Middle axis (K > 1): threads run along the contiguous K axis and walk N with stride K.
 //
 // Arithmetic follows the reference kernels: fp32, e = exp(x - max), out = e / sum.  -inf inputs
@@ -106,31 +107,143 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
   }
 }
 
-// Any N: one block per row, online (max, sum) then a second sweep.
-template <typename TI, typename TO, bool LOG>
-__global__ __launch_bounds__(256) void softmax_looped_kernel(const TI* __restrict__ in, TO* __restrict__ out,
-                                                            int64_t M, int64_t N) {
-  __shared__ float smem[4];
+// Rows that do not fit the registers of one workgroup (more than 8192 packs of 16 bytes) or whose
+// start is only element-aligned (N not a multiple of the pack): one workgroup per row, two sweeps.  The first keeps a
+// running (max, sum) per thread, rescaled once per 16-byte pack; the second reads the row again (from L2 for all but
+// the longest rows), and writes.  Loads and stores are 16-byte accesses declared element-aligned; up to four of them
+// per thread are in flight.  The N % VEC elements behind the last full pack go one per thread.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld_pack_u(const T* p) {
+  Pack<T, VEC> v;
+  __builtin_memcpy(&v, p, sizeof(T) * VEC);
+  return v;
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_pack_u(T* p, const Pack<T, VEC>& v) {
+  __builtin_memcpy(p, &v, sizeof(T) * VEC);
+}
+
+template <typename TI, typename TO, bool LOG, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void softmax_long_kernel(const TI* __restrict__ in, TO* __restrict__ out, int64_t M,
+                                                            int64_t N) {
+  constexpr int VEC = 16 / sizeof(TI);
+  constexpr int UNROLL = 4;
+  __shared__ float smem[BLOCK / 64];
   const int64_t row = blockIdx.x;
   const TI* xr = in + row * N;
   TO* yr = out + row * N;
+  const int64_t packs = N / VEC;
+  const int64_t tail0 = packs * VEC;
+  const int t = threadIdx.x;
   float m = -INFINITY, z = 0.f;
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
-    const float x = (float)xr[c];
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<TI, VEC> px[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      if (p0 + (int64_t)u * BLOCK < packs) px[u] = ld_pack_u<TI, VEC>(xr + (p0 + (int64_t)u * BLOCK) * VEC);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (p0 + (int64_t)u * BLOCK < packs) {
+        float x[VEC];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          x[e] = (float)px[u].v[e];
+          pm = fmaxf(pm, x[e]);
+        }
+        const float mn = fmaxf(m, pm);
+        // mn == -inf only while every element seen so far is -inf: keep z at 0 instead of NaN.
+        if (mn != -INFINITY) {
+          float acc = 0.f;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc += __expf(x[e] - mn);
+          z = z * __expf(m - mn) + acc;
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          if (x[e] != x[e]) z = x[e];  // fmaxf drops a NaN: put it into the sum by hand
+        m = mn;
+      }
+    }
+  }
+  if (t < N - tail0) {
+    const float x = (float)xr[tail0 + t];
     const float mn = fmaxf(m, x);
-    // mn == -inf only while every element seen so far is -inf: keep z at 0 instead of NaN.
     if (mn != -INFINITY) z = z * __expf(m - mn) + __expf(x - mn);
     if (x != x) z = x;
     m = mn;
   }
-  const float mr = row_reduce<256>(m, smem, 0, threadIdx.x, OpMax(), -INFINITY);
+  const float mr = row_reduce<BLOCK>(m, smem, 0, t, OpMax(), -INFINITY);
   float zz = (m == -INFINITY) ? 0.f : z * __expf(m - mr);
   if (z != z) zz = z;
-  const float s = row_reduce<256>(zz, smem, 0, threadIdx.x, OpSum(), 0.f);
+  const float s = row_reduce<BLOCK>(zz, smem, 0, t, OpSum(), 0.f);
   const float log_s = LOG ? logf(s) : 0.f;
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
-    const float d = (float)xr[c] - mr;
-    yr[c] = LOG ? (TO)(d - log_s) : (TO)(__expf(d) / s);
+  const float inv = 1.0f / s;
+  auto result = [&](float x) -> TO {
+    const float d = x - mr;
+    if constexpr (LOG) return (TO)(d - log_s);
+    else if constexpr (sizeof(TO) == 4) return (TO)(__expf(d) / s);
+    else return (TO)(__expf(d) * inv);
+  };
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<TI, VEC> px[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      if (p0 + (int64_t)u * BLOCK < packs) px[u] = ld_pack_u<TI, VEC>(xr + (p0 + (int64_t)u * BLOCK) * VEC);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (p0 + (int64_t)u * BLOCK < packs) {
+        Pack<TO, VEC> po;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) po.v[e] = result((float)px[u].v[e]);
+        st_pack_u<TO, VEC>(yr + (p0 + (int64_t)u * BLOCK) * VEC, po);
+      }
+    }
+  }
+  if (t < N - tail0) yr[tail0 + t] = result((float)xr[tail0 + t]);
+}
+
+// Short rows whose start is only element-aligned (N <= 1024, not a multiple of the pack): one wave per row, element
+// j * 64 + lane in register j, no LDS and no barrier.
+template <typename TI, typename TO, bool LOG, int ITERS>
+__global__ __launch_bounds__(256) void softmax_short_kernel(const TI* __restrict__ in, TO* __restrict__ out, int64_t M,
+                                                           int N) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;  // the whole wave leaves
+  const TI* xr = in + row * (int64_t)N;
+  TO* yr = out + row * (int64_t)N;
+  float v[ITERS];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    v[j] = c < N ? (float)xr[c] : -INFINITY;
+    m = fmaxf(m, v[j]);
+  }
+  m = wave_max(m);
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    if constexpr (LOG) {
+      v[j] -= m;
+      s += fast_exp<sizeof(TI) == 4>(v[j]);
+    } else {
+      v[j] = fast_exp<sizeof(TI) == 4>(v[j] - m);
+      s += v[j];
+    }
+  }
+  s = wave_sum(s);
+  const float inv = 1.0f / s;
+  const float log_s = LOG ? logf(s) : 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    if (c < N) {
+      if constexpr (LOG) yr[c] = (TO)(v[j] - log_s);
+      else if constexpr (sizeof(TO) == 4) yr[c] = (TO)(v[j] / s);
+      else yr[c] = (TO)(v[j] * inv);
+    }
   }
 }
 
@@ -181,8 +294,21 @@ int softmax_dispatch(const TI* in, TO* out, int64_t M, int64_t N, int64_t K, hip
   const bool vec_ok = (N % VEC == 0) && fg_aligned(in, 16) && fg_aligned(out, sizeof(TO) * VEC);
   const int64_t packs = vec_ok ? N / VEC : 0;
 #define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, LOG>(in, out, M, (int)N, st)
-  if (!vec_ok || packs > 1024 * 8) {
-    hipLaunchKernelGGL((softmax_looped_kernel<TI, TO, LOG>), dim3((unsigned)M), dim3(256), 0, st, in, out, M, N);
+  if (!vec_ok && N <= 1024) {
+#define FG_SHORT(ITERS)                                                                                                  \
+  hipLaunchKernelGGL((softmax_short_kernel<TI, TO, LOG, ITERS>), dim3((unsigned)fg_cdiv(M, 4)), dim3(256), 0, st, in, out, \
+                     M, (int)N)
+    if (N <= 64) FG_SHORT(1);
+    else if (N <= 128) FG_SHORT(2);
+    else if (N <= 256) FG_SHORT(4);
+    else if (N <= 512) FG_SHORT(8);
+    else FG_SHORT(16);
+#undef FG_SHORT
+  } else if (!vec_ok || packs > 1024 * 8) {
+    if (N >= 2048)
+      hipLaunchKernelGGL((softmax_long_kernel<TI, TO, LOG, 1024>), dim3((unsigned)M), dim3(1024), 0, st, in, out, M, N);
+    else
+      hipLaunchKernelGGL((softmax_long_kernel<TI, TO, LOG, 256>), dim3((unsigned)M), dim3(256), 0, st, in, out, M, N);
   } else if (packs <= 64) {
     FG_ROWS(1, 64);
   } else if (packs <= 128) {

@@ -70,7 +70,8 @@ def test_fused_add_rms_norm(gpu, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", SOFTMAX_SHAPES + [(16, 2048), (7, 40999), (5, 33), (3, 70000)])
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES + [(16, 2048), (7, 40999), (5, 33), (3, 70000), (9, 1001), (6, 100), (4, 300),
+                                                    (3, 600), (5, 1500), (2, 131072)])
 @pytest.mark.parametrize("neg_inf", [False, True])
 def test_softmax(gpu, shape, dtype, neg_inf):
     torch.manual_seed(0)
@@ -86,6 +87,25 @@ def test_softmax(gpu, shape, dtype, neg_inf):
     if dtype != torch.float32:
         res = flag_gems.softmax(x, -1, True)
         gems_assert_close(res, O.softmax(x, -1), torch.float32, equal_nan=True)
+
+
+# Rows of every kernel of the inner axis (registers; one wave per short unaligned row; two sweeps for unaligned and
+# for long rows) with a NaN, with nothing but -inf, with -inf in front of the first finite value, and untouched.
+@pytest.mark.parametrize("dtype", FLOAT_DTYPES)
+@pytest.mark.parametrize("N", [33, 256, 1001, 1500, 4097, 70001, 131072])
+def test_softmax_special_rows(gpu, N, dtype):
+    torch.manual_seed(N)
+    x = torch.randn(5, N, dtype=dtype, device=gpu)
+    x[0, N // 3] = float("nan")
+    x[1] = float("-inf")
+    x[2, : N - 2] = float("-inf")
+    x[3, N - 1] = float("nan")
+    for fn, ref_fn in ((flag_gems.softmax, O.softmax), (flag_gems.log_softmax, O.log_softmax)):
+        res = fn(x, -1)
+        ref = ref_fn(x, -1)
+        assert torch.isnan(res[0]).all() and torch.isnan(res[1]).all() and torch.isnan(res[3]).all()
+        gems_assert_close(res[2], ref[2], dtype, equal_nan=True)
+        gems_assert_close(res[4], ref[4], dtype)
 
 
 # log_softmax: the same kernels with (x - max) - log(sum) as the last step (reference test:
