@@ -253,33 +253,117 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_bwd_rows_kernel(
   }
 }
 
-// Any N, any alignment: one 256-thread block per row, element-wise access, two sweeps.
-template <typename TI, typename TO, int MODE>
-__global__ __launch_bounds__(256) void bwd_looped_kernel(const TI* __restrict__ a, const TI* __restrict__ g,
-                                                        const TI* __restrict__ w, const float* __restrict__ inv_rms,
-                                                        TO* __restrict__ out, int64_t M, int64_t N) {
-  __shared__ float smem[4];
+// Rows too long for the registers of one workgroup, or whose start is only element-aligned: one workgroup per row,
+// two sweeps of element-aligned 16-byte accesses (the second sweep reads from L2 for all but the longest rows); the
+// N % VEC elements behind the last full pack go one per thread.
+template <typename TI, typename TO, int MODE, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void bwd_looped_kernel(const TI* __restrict__ a, const TI* __restrict__ g,
+                                                          const TI* __restrict__ w, const float* __restrict__ inv_rms,
+                                                          TO* __restrict__ out, int64_t M, int64_t N) {
+  constexpr int VEC = 16 / sizeof(TI);
+  constexpr int UNROLL = 2;
+  __shared__ float smem[BLOCK / 64];
   const int64_t row = blockIdx.x;
   const TI* ar = a + row * N;
   const TI* gr = g + row * N;
   TO* orow = out + row * N;
+  const int64_t packs = N / VEC, tail0 = packs * VEC;
+  const int t = threadIdx.x;
   const float inv = MODE == BWD_RMS ? inv_rms[row] : 1.0f;
+  const bool has_w = MODE == BWD_RMS && w != nullptr;
   float s = 0.f;
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<TI, VEC> pa[UNROLL], pg[UNROLL], pw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        pa[u] = ld_pack_u<TI, VEC>(ar + p * VEC);
+        pg[u] = ld_pack_u<TI, VEC>(gr + p * VEC);
+        if (has_w) pw[u] = ld_pack_u<TI, VEC>(w + p * VEC);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (p0 + (int64_t)u * BLOCK < packs) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = (float)pa[u].v[e], d = (float)pg[u].v[e];
+          if constexpr (MODE == BWD_SOFTMAX) s += x * d;
+          else if constexpr (MODE == BWD_LOG_SOFTMAX) s += d;
+          else s += x * inv * d * (has_w ? (float)pw[u].v[e] : 1.0f);
+        }
+      }
+    }
+  }
+  if (t < N - tail0) {
+    const int64_t c = tail0 + t;
     const float x = (float)ar[c], d = (float)gr[c];
     if constexpr (MODE == BWD_SOFTMAX) s += x * d;
     else if constexpr (MODE == BWD_LOG_SOFTMAX) s += d;
-    else s += x * inv * d * (w != nullptr ? (float)w[c] : 1.0f);
+    else s += x * inv * d * (has_w ? (float)w[c] : 1.0f);
   }
-  s = row_sum<256>(s, smem, 0, threadIdx.x);
+  s = row_sum<BLOCK>(s, smem, 0, t);
   const float mean = s / (float)N;
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
-    const float x = (float)ar[c], d = (float)gr[c];
-    float r;
-    if constexpr (MODE == BWD_SOFTMAX) r = x * (d - s);
-    else if constexpr (MODE == BWD_LOG_SOFTMAX) r = d - exp_like_forward<TI>(x) * s;
-    else r = (d * (w != nullptr ? (float)w[c] : 1.0f) - x * inv * mean) * inv;
-    orow[c] = (TO)r;
+  auto result = [&](float x, float d, float wv) -> TO {
+    if constexpr (MODE == BWD_SOFTMAX) return (TO)(x * (d - s));
+    else if constexpr (MODE == BWD_LOG_SOFTMAX) return (TO)(d - exp_like_forward<TI>(x) * s);
+    else return (TO)((d * wv - x * inv * mean) * inv);
+  };
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<TI, VEC> pa[UNROLL], pg[UNROLL], pw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        pa[u] = ld_pack_u<TI, VEC>(ar + p * VEC);
+        pg[u] = ld_pack_u<TI, VEC>(gr + p * VEC);
+        if (has_w) pw[u] = ld_pack_u<TI, VEC>(w + p * VEC);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        Pack<TO, VEC> po;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          po.v[e] = result((float)pa[u].v[e], (float)pg[u].v[e], has_w ? (float)pw[u].v[e] : 1.0f);
+        st_pack_u<TO, VEC>(orow + p * VEC, po);
+      }
+    }
+  }
+  if (t < N - tail0) {
+    const int64_t c = tail0 + t;
+    orow[c] = result((float)ar[c], (float)gr[c], has_w ? (float)w[c] : 1.0f);
+  }
+}
+
+// Short rows whose start is only element-aligned (N <= 512): one wave per row, element j * 64 + lane in
+// register j, no LDS and no barrier.  Softmax and log_softmax only.
+template <typename TI, typename TO, int MODE, int ITERS>
+__global__ __launch_bounds__(256) void bwd_short_kernel(const TI* __restrict__ a, const TI* __restrict__ g,
+                                                       TO* __restrict__ out, int64_t M, int N) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;  // the whole wave leaves
+  const TI* ar = a + row * (int64_t)N;
+  const TI* gr = g + row * (int64_t)N;
+  TO* orow = out + row * (int64_t)N;
+  float x[ITERS], d[ITERS];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    x[j] = c < N ? (float)ar[c] : 0.f;
+    d[j] = c < N ? (float)gr[c] : 0.f;
+    s += MODE == BWD_SOFTMAX ? x[j] * d[j] : d[j];
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    if (c < N) orow[c] = MODE == BWD_SOFTMAX ? (TO)(x[j] * (d[j] - s)) : (TO)(d[j] - exp_like_forward<TI>(x[j]) * s);
   }
 }
 
@@ -358,9 +442,22 @@ int bwd_rows_dispatch(const TI* a, const TI* g, TO* out, int64_t M, int64_t N, h
   const int64_t packs = vec_ok ? N / VEC : 0;
 #define FG_ROWS(ITERS, TPR) launch_rows<TI, TO, VEC, ITERS, TPR, MODE>(a, g, out, M, (int)N, st)
   // two input streams: one pack per thread from each, as in the fused add + norm forward
-  if (!vec_ok || packs > 4096) {
-    hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE>), dim3((unsigned)M), dim3(256), 0, st, a, g, (const TI*)nullptr,
-                       (const float*)nullptr, out, M, N);
+  if (!vec_ok && N <= 512) {  // from there on the two-sweep kernel with 256 threads measures faster
+#define FG_SHORT(ITERS)                                                                                                \
+  hipLaunchKernelGGL((bwd_short_kernel<TI, TO, MODE, ITERS>), dim3((unsigned)fg_cdiv(M, 4)), dim3(256), 0, st, a, g, out, \
+                     M, (int)N)
+    if (N <= 64) FG_SHORT(1);
+    else if (N <= 128) FG_SHORT(2);
+    else if (N <= 256) FG_SHORT(4);
+    else FG_SHORT(8);
+#undef FG_SHORT
+  } else if (!vec_ok || packs > 4096) {
+    if (N >= 2048)
+      hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE, 1024>), dim3((unsigned)M), dim3(1024), 0, st, a, g,
+                         (const TI*)nullptr, (const float*)nullptr, out, M, N);
+    else
+      hipLaunchKernelGGL((bwd_looped_kernel<TI, TO, MODE, 256>), dim3((unsigned)M), dim3(256), 0, st, a, g,
+                         (const TI*)nullptr, (const float*)nullptr, out, M, N);
   } else if (packs > 2048) {
     FG_ROWS(4, 1024);  // vocabulary-sized rows (32000 16-bit elements)
   } else if (packs <= 64) {
@@ -409,8 +506,12 @@ int rms_bwd_dispatch(const T* x, const T* dy, const T* w, const float* inv_rms, 
   // rows summed into one partial row: with partial_rows groups of that many rows all M rows are covered
   const int64_t rows_per_group = dw_partial != nullptr ? fg_cdiv(M, partial_rows) : 1;
   if (!vec_ok || packs > 2048) {
-    hipLaunchKernelGGL((bwd_looped_kernel<T, T, BWD_RMS>), dim3((unsigned)M), dim3(256), 0, st, x, dy, w, inv_rms, dx, M,
-                       N);
+    if (N >= 2048)
+      hipLaunchKernelGGL((bwd_looped_kernel<T, T, BWD_RMS, 1024>), dim3((unsigned)M), dim3(1024), 0, st, x, dy, w, inv_rms,
+                         dx, M, N);
+    else
+      hipLaunchKernelGGL((bwd_looped_kernel<T, T, BWD_RMS, 256>), dim3((unsigned)M), dim3(256), 0, st, x, dy, w, inv_rms,
+                         dx, M, N);
     if (dw_partial != nullptr)
       hipLaunchKernelGGL((rms_dw_partial_kernel<T>), dim3((unsigned)partial_rows, (unsigned)fg_cdiv(N, 256)), dim3(256),
                          0, st, x, dy, inv_rms, dw_partial, M, N, (int)rows_per_group);

@@ -81,6 +81,19 @@ __device__ __forceinline__ void st_pack_nt(T* p, const Pack<T, VEC>& v) {
   }
 }
 
+// Element-aligned variants: the address is a multiple of sizeof(T) only.  The compiler still emits one wide
+// access (the target handles unaligned vector-memory accesses), split by the hardware where it crosses a line.
+template <typename T, int VEC>
+__device__ __forceinline__ Pack<T, VEC> ld_pack_u(const T* p) {
+  Pack<T, VEC> v;
+  __builtin_memcpy(&v, p, sizeof(T) * VEC);
+  return v;
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void st_pack_u(T* p, const Pack<T, VEC>& v) {
+  __builtin_memcpy(p, &v, sizeof(T) * VEC);
+}
+
 // Waits until every vector-memory operation this wave has issued, stores included, has completed.
 // A workgroup-scope release fence does not emit this wait on gfx950 (the waves of a workgroup share
 // one L1, so the fence has nothing to order for them), and a device-scope release would write the

@@ -112,17 +112,6 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
 // running (max, sum) per thread, rescaled once per 16-byte pack; the second reads the row again (from L2 for all but
 // the longest rows), and writes.  Loads and stores are 16-byte accesses declared element-aligned; up to four of them
 // per thread are in flight.  The N % VEC elements behind the last full pack go one per thread.
-template <typename T, int VEC>
-__device__ __forceinline__ Pack<T, VEC> ld_pack_u(const T* p) {
-  Pack<T, VEC> v;
-  __builtin_memcpy(&v, p, sizeof(T) * VEC);
-  return v;
-}
-template <typename T, int VEC>
-__device__ __forceinline__ void st_pack_u(T* p, const Pack<T, VEC>& v) {
-  __builtin_memcpy(p, &v, sizeof(T) * VEC);
-}
-
 template <typename TI, typename TO, bool LOG, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void softmax_long_kernel(const TI* __restrict__ in, TO* __restrict__ out, int64_t M,
                                                             int64_t N) {

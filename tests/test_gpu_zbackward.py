@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", SOFTMAX_SHAPES + [(16, 2048), (7, 40999), (5, 33), (3, 16392), (64, 8192)])
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES + [(16, 2048), (7, 40999), (5, 33), (3, 16392), (64, 8192), (3, 70000), (2, 131072),
+                                                    (9, 1001), (4, 1500), (6, 100), (4, 300), (3, 500)])
 @pytest.mark.parametrize("neg_inf", [False, True])
 def test_softmax_backward(gpu, shape, dtype, neg_inf):
     torch.manual_seed(0)
@@ -30,7 +31,8 @@ def test_softmax_backward(gpu, shape, dtype, neg_inf):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(200, 2560, 3), (16, 2048), (5, 33), (8, 32000)])
+@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(200, 2560, 3), (16, 2048), (5, 33), (8, 32000), (3, 70001), (2, 151936),
+                                                      (9, 1001)])
 def test_log_softmax_backward(gpu, shape, dtype):
     torch.manual_seed(0)
     for dim in range(len(shape)):
@@ -71,7 +73,8 @@ def test_softmax_backward_through_autograd(gpu):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(64, 4096), (3, 5, 1024), (17, 8200), (130, 16392), (1000, 33)])
+@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(64, 4096), (3, 5, 1024), (17, 8200), (130, 16392), (1000, 33), (5, 40999),
+                                                      (3, 70000)])
 def test_rms_norm_backward(gpu, shape, dtype):
     np.random.seed(0)
     n = shape[-1]
