@@ -6,7 +6,8 @@
 // 64*VEC*sizeof(T) contiguous bytes (1 KiB at 16 B per lane).  Blocks are 256 threads, so
 // 256/TPR rows share a block when TPR < 256.  Rows too long for the register variant
 // (N > 1024*VEC*8) and rows that defeat vector access (N or strides not a multiple of VEC,
-// unaligned base) go through a looped two-pass kernel that re-reads the row from L2.
+// unaligned base) go through a two-pass kernel that re-reads the row from L2 (16-byte accesses
+// declared element-aligned, one workgroup per row), or, up to 512 elements, one wave per row.
 #include "fg_common.h"
 
 namespace {
@@ -96,37 +97,131 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
 }
 
 // Any N, any alignment: one 256-thread block per row, element-wise coalesced access, two passes.
-template <typename T, bool FUSED>
-__global__ __launch_bounds__(256) void rms_looped_kernel(const T* x, T* res,
-                                                        const T* __restrict__ w, T* y,
-                                                        float* __restrict__ inv_rms, int64_t M, int64_t N,
-                                                        int64_t xs, int64_t rs, int64_t ys, float eps) {
-  __shared__ float smem[4];
+// Short rows that defeat 16-byte access (N <= 512): one wave per row, element j * 64 + lane in register j.
+template <typename T, bool FUSED, int ITERS>
+__global__ __launch_bounds__(256) void rms_short_kernel(const T* x, T* res, const T* __restrict__ w, T* y,
+                                                       float* __restrict__ inv_rms, int64_t M, int N, int64_t xs,
+                                                       int64_t rs, int64_t ys, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;  // the whole wave leaves
+  const T* xr = x + row * xs;
+  T* rr = FUSED ? res + row * rs : nullptr;
+  T* yr = y + row * ys;
+  float v[ITERS];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    v[j] = c < N ? (float)xr[c] : 0.f;
+    if constexpr (FUSED) {
+      if (c < N) v[j] += (float)rr[c];
+    }
+    ss += v[j] * v[j];
+  }
+  ss = wave_sum(ss);
+  const float rrms = 1.0f / sqrtf(ss / (float)N + eps);
+  if constexpr (!FUSED) {
+    if (inv_rms != nullptr && lane == 0) inv_rms[row] = rrms;
+  }
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    if (c < N) {
+      if constexpr (FUSED) rr[c] = (T)v[j];
+      yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)w[c] : 1.0f));
+    }
+  }
+}
+
+template <typename T, bool FUSED, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void rms_looped_kernel(const T* x, T* res,
+                                                          const T* __restrict__ w, T* y,
+                                                          float* __restrict__ inv_rms, int64_t M, int64_t N,
+                                                          int64_t xs, int64_t rs, int64_t ys, float eps) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int UNROLL = FUSED ? 2 : 4;
+  __shared__ float smem[BLOCK / 64];
   const int64_t row = blockIdx.x;
   const T* xr = x + row * xs;
   T* rr = FUSED ? res + row * rs : nullptr;
   T* yr = y + row * ys;
+  const int64_t packs = N / VEC, tail0 = packs * VEC;
+  const int t = threadIdx.x;
+  // 16-byte accesses declared element-aligned; the N % VEC elements behind the last full pack go one per thread
   float ss = 0.f;
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
-    float v = (float)xr[c];
-    if constexpr (FUSED) v += (float)rr[c];
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<T, VEC> px[UNROLL], pr[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        px[u] = ld_pack_u<T, VEC>(xr + p * VEC);
+        if constexpr (FUSED) pr[u] = ld_pack_u<T, VEC>(rr + p * VEC);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      if (p0 + (int64_t)u * BLOCK < packs) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float v = (float)px[u].v[e];
+          if constexpr (FUSED) v += (float)pr[u].v[e];
+          ss += v * v;
+        }
+      }
+    }
+  }
+  if (t < N - tail0) {
+    float v = (float)xr[tail0 + t];
+    if constexpr (FUSED) v += (float)rr[tail0 + t];
     ss += v * v;
   }
-  ss = row_sum<256>(ss, smem, 0, threadIdx.x);
+  ss = row_sum<BLOCK>(ss, smem, 0, t);
   const float rrms = 1.0f / sqrtf(ss / (float)N + eps);
   if constexpr (!FUSED) {
-    if (inv_rms != nullptr && threadIdx.x == 0) inv_rms[row] = rrms;
+    if (inv_rms != nullptr && t == 0) inv_rms[row] = rrms;
   }
   // Second pass recomputes the fp32 sum from the still-unmodified inputs (each element is read
   // and then written by the same thread, so in-place operation is safe).
-  for (int64_t c = threadIdx.x; c < N; c += 256) {
+  for (int64_t p0 = t; p0 < packs; p0 += (int64_t)BLOCK * UNROLL) {
+    Pack<T, VEC> px[UNROLL], pr[UNROLL], pw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        px[u] = ld_pack_u<T, VEC>(xr + p * VEC);
+        if constexpr (FUSED) pr[u] = ld_pack_u<T, VEC>(rr + p * VEC);
+        if (w != nullptr) pw[u] = ld_pack_u<T, VEC>(w + p * VEC);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t p = p0 + (int64_t)u * BLOCK;
+      if (p < packs) {
+        Pack<T, VEC> po, ps;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float v = (float)px[u].v[e];
+          if constexpr (FUSED) {
+            v += (float)pr[u].v[e];
+            ps.v[e] = (T)v;
+          }
+          po.v[e] = (T)(v * rrms * (w != nullptr ? (float)pw[u].v[e] : 1.0f));
+        }
+        if constexpr (FUSED) st_pack_u<T, VEC>(rr + p * VEC, ps);
+        st_pack_u<T, VEC>(yr + p * VEC, po);
+      }
+    }
+  }
+  if (t < N - tail0) {
+    const int64_t c = tail0 + t;
     float v = (float)xr[c];
     if constexpr (FUSED) {
       v += (float)rr[c];
       rr[c] = (T)v;
     }
-    const float wv = w != nullptr ? (float)w[c] : 1.0f;
-    yr[c] = (T)(v * rrms * wv);
+    yr[c] = (T)(v * rrms * (w != nullptr ? (float)w[c] : 1.0f));
   }
 }
 
@@ -154,8 +249,21 @@ int rms_dispatch(const T* x, T* res, const T* w, T* y, float* inv_rms, int64_t M
   }
 #define FG_ROWS(ITERS, TPR) launch_rows<T, VEC, ITERS, TPR, FUSED>(x, res, w, y, inv_rms, M, (int)N, xs, rs, ys, eps, st)
   if (!vec_ok || packs > 1024 * 8) {
-    hipLaunchKernelGGL((rms_looped_kernel<T, FUSED>), dim3((unsigned)M), dim3(256), 0, st, x, res, w, y, inv_rms, M,
-                       N, xs, rs, ys, eps);
+    if (N <= 512) {  // from there on the two-pass kernel with 256 threads measures faster
+#define FG_SHORT(ITERS)                                                                                              \
+  hipLaunchKernelGGL((rms_short_kernel<T, FUSED, ITERS>), dim3((unsigned)fg_cdiv(M, 4)), dim3(256), 0, st, x, res, w, y, \
+                     inv_rms, M, (int)N, xs, rs, ys, eps)
+      if (N <= 64) FG_SHORT(1);
+      else if (N <= 128) FG_SHORT(2);
+      else if (N <= 256) FG_SHORT(4);
+      else FG_SHORT(8);
+#undef FG_SHORT
+    } else if (N >= 2048)
+      hipLaunchKernelGGL((rms_looped_kernel<T, FUSED, 1024>), dim3((unsigned)M), dim3(1024), 0, st, x, res, w, y, inv_rms,
+                         M, N, xs, rs, ys, eps);
+    else
+      hipLaunchKernelGGL((rms_looped_kernel<T, FUSED, 256>), dim3((unsigned)M), dim3(256), 0, st, x, res, w, y, inv_rms,
+                         M, N, xs, rs, ys, eps);
   } else if (FUSED) {
     // Two input streams: one pack per thread from each wherever a row fits 1024 threads.  Measured on
     // MI355X this beats fewer threads holding several packs (16384 x 4096 bf16: 84.8 us at 1 x 512

@@ -23,7 +23,8 @@ def g(name, dtype, dev):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(64, 4096), (3, 5, 1024), (17, 8200), (5, 65536)])
+@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(64, 4096), (3, 5, 1024), (17, 8200), (5, 65536), (5, 4099), (3, 70001),
+                                                      (2, 131072), (7, 1001), (9, 33), (6, 100), (4, 300), (3, 500)])
 def test_rms_norm(gpu, shape, dtype):
     np.random.seed(0)
     x = torch.from_numpy(np.random.uniform(-0.1, 0.1, shape).astype(np.float32)).to(dtype).to(gpu)
@@ -56,7 +57,7 @@ def test_rms_norm_schema_defaults_and_autograd(gpu):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(4096, 4096), (33, 1000)])
+@pytest.mark.parametrize("shape", REDUCTION_SHAPES + [(4096, 4096), (33, 1000), (5, 4099), (3, 70001), (2, 131072), (7, 1001), (9, 33), (4, 300)])
 def test_fused_add_rms_norm(gpu, shape, dtype):
     torch.manual_seed(0)
     x = torch.randn(shape, dtype=dtype, device=gpu); r = torch.randn(shape, dtype=dtype, device=gpu)
