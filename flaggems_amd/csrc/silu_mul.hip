@@ -2,8 +2,8 @@
 //
 // a, b and out are [rows, cols] with unit column stride and independent row strides, which covers
 // the two halves of a fused gate-up projection without a copy.  Packs of 16 bytes are numbered
-// row-major and dealt one per thread.  Rows that defeat 16-byte access are handled one element
-// per thread.
+// row-major and dealt one per thread.  Rows that defeat 16-byte alignment keep the scheme with accesses
+// declared element-aligned.
 #include "fg_common.h"
 
 namespace {
@@ -24,19 +24,42 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* a, const T* b, T
   st_pack_nt<T, VEC>(out + r * os + c, o);
 }
 
+// Rows that defeat 16-byte alignment (odd column count, row stride or base address): the same numbering with
+// ceil(cols / VEC) packs per row, 16-byte accesses declared element-aligned, the ragged last pack of a row element
+// by element.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void silu_mul_unaligned_kernel(const T* a, const T* b, T* out, int64_t rows, int64_t cols,
+                                                                int64_t as, int64_t bs, int64_t os) {
+  const int64_t ppr = (cols + VEC - 1) / VEC;
+  const int64_t item = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (item >= rows * ppr) return;
+  const int64_t r = item / ppr;
+  const int64_t c = (item - r * ppr) * VEC;
+  if (c + VEC <= cols) {
+    Pack<T, VEC> x = ld_pack_u<T, VEC>(a + r * as + c), y = ld_pack_u<T, VEC>(b + r * bs + c), o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.v[e] = (T)silu_mul((float)x.v[e], (float)y.v[e]);
+    st_pack_u<T, VEC>(out + r * os + c, o);
+  } else {
+    for (int64_t cc = c; cc < cols; ++cc)
+      out[r * os + cc] = (T)silu_mul((float)a[r * as + cc], (float)b[r * bs + cc]);
+  }
+}
+
 template <typename T>
 int silu_dispatch(const T* a, const T* b, T* out, int64_t rows, int64_t cols, int64_t as, int64_t bs, int64_t os,
                   hipStream_t st) {
   constexpr int VEC = 16 / sizeof(T);
   const bool vec_ok = cols % VEC == 0 && as % VEC == 0 && bs % VEC == 0 && os % VEC == 0 && fg_aligned(a, 16) &&
                       fg_aligned(b, 16) && fg_aligned(out, 16);
-  const int64_t items = vec_ok ? rows * (cols / VEC) : rows * cols;
+  const int64_t items = vec_ok ? rows * (cols / VEC) : rows * fg_cdiv(cols, VEC);
   const int64_t grid = fg_cdiv(items, 256);
   FG_REQUIRE(grid < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "silu_and_mul: problem too large for one launch");
   if (vec_ok)
     hipLaunchKernelGGL((silu_mul_kernel<T, VEC>), dim3((unsigned)grid), dim3(256), 0, st, a, b, out, rows, cols, as, bs, os);
   else
-    hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((unsigned)grid), dim3(256), 0, st, a, b, out, rows, cols, as, bs, os);
+    hipLaunchKernelGGL((silu_mul_unaligned_kernel<T, VEC>), dim3((unsigned)grid), dim3(256), 0, st, a, b, out, rows, cols, as,
+                       bs, os);
   return fg_check_launch("silu_and_mul");
 }
 

@@ -197,12 +197,15 @@ def test_rope_fused_qkv_views_and_table_layouts(gpu):
 
 
 @pytest.mark.parametrize("dtype", FLOAT_DTYPES)
-@pytest.mark.parametrize("shape", [(), (2, 19, 7), (1024, 1024), (16, 22016), (3, 4, 5, 6, 8)])
+@pytest.mark.parametrize("shape", [(), (2, 19, 7), (1024, 1024), (16, 22016), (3, 4, 5, 6, 8), (33, 4099), (5, 1), (7, 8206)])
 def test_silu_and_mul(gpu, shape, dtype):
     torch.manual_seed(0)
     if shape == (16, 22016):  # the two halves of a gate-up projection: strided rows, no copy
         gu = torch.randn(shape, dtype=dtype, device=gpu)
         a, b = gu[:, :11008], gu[:, 11008:]
+    elif shape == (7, 8206):  # halves with an odd split: element-aligned starts, ragged last pack
+        gu = torch.randn(shape, dtype=dtype, device=gpu)
+        a, b = gu[:, :4103], gu[:, 4103:]
     else:
         a = torch.randn(shape, dtype=dtype, device=gpu); b = torch.randn(shape, dtype=dtype, device=gpu)
     ref = O.silu_and_mul(a, b)
