@@ -765,6 +765,12 @@ int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
       }
     } else {
       switch (D) {
+        // head dims that are a multiple of 16 but fill their LDS rows only partly: the padding chunks are loaded
+        // with finite data and the output columns computed from them are never stored
+        case 32: return launch_async<T, 32, 128, 4, 2>(a, grid, st);
+        case 48: return launch_async<T, 48, 128, 4, 2>(a, grid, st);
+        case 80: return launch_async<T, 80, 256, 4, 2>(a, grid, st);
+        case 112: return launch_async<T, 112, 256, 4, 2>(a, grid, st);
         case 64: return launch_async<T, 64, 128, 4, 2>(a, grid, st);
         case 96: return launch_async<T, 96, 256, 4, 2>(a, grid, st);
         case 128: return launch_async<T, 128, 256, 4, 2>(a, grid, st);
@@ -898,11 +904,12 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.page_shift = -1;
   for (int sft = 0; sft < 31; ++sft)
     if ((1 << sft) == p.page_size) a.page_shift = sft;
-  // Kernel variant.  Head dims 64/96/128/192/256 take the asynchronous-tile kernel with 4 waves and
-  // two LDS stages (measured fastest; the 8-wave variants stay selectable for head dims <= 128);
+  // Kernel variant.  Head dims 32/48/64/80/96/112/128/192/256 take the asynchronous-tile kernel with 4 waves and
+  // two LDS stages (measured fastest; the 8-wave variants stay selectable for head dims 64, 96 and 128);
   // everything else the register-staged kernel.
   // FG_ATTN_KERNEL = "fast" | "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
-  a.use_async = (p.D == 64 || p.D == 96 || p.D == 128 || p.D == 192 || p.D == 256) ? 1 : 0;
+  a.use_async = (p.D == 32 || p.D == 48 || p.D == 64 || p.D == 80 || p.D == 96 || p.D == 112 || p.D == 128 || p.D == 192 ||
+                 p.D == 256) ? 1 : 0;
   a.nw = 4;
   a.nst = 2;
   // The lean kernel needs the 16 key rows a wave moves per tile inside one page, and keeps the page ids of
@@ -916,7 +923,7 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   if (const char* force = getenv("FG_ATTN_KERNEL")) {
     a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p');
     if (force[0] == 's') a.use_async = 0;
-    if (force[0] == 'w' && p.D <= 128) {
+    if (force[0] == 'w' && (p.D == 64 || p.D == 96 || p.D == 128)) {
       a.nw = force[1] == '8' ? 8 : 4;
       a.nst = (force[2] == 's' && force[3] == '3' && a.nw == 8) ? 3 : 2;
     }

@@ -61,7 +61,7 @@ def test_flash_attn_varlen_reference_grid(gpu, dtype, Hq, Hk, D, num_blocks, ali
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hk", [(6, 2), (3, 1), (32, 8)])
-@pytest.mark.parametrize("D", [64, 80, 96, 120])
+@pytest.mark.parametrize("D", [32, 48, 64, 72, 80, 96, 112, 120])
 def test_flash_attn_varlen_more_heads_and_dims(gpu, dtype, Hq, Hk, D):
     check(gpu, [(1, 1328), (5, 18), (129, 463), (70, 70)], Hq, Hk, D, 16, 512, dtype)
 
@@ -173,7 +173,7 @@ def _dense_inputs(dev, batch, heads, heads_k, sq, sk, d, dtype):
 
 
 @pytest.mark.parametrize("batch,heads,sq,sk", [(1, 1, 128, 2048), (4, 8, 1024, 128), (4, 8, 17, 1030)])
-@pytest.mark.parametrize("d", [64, 128, 192, 256])
+@pytest.mark.parametrize("d", [32, 64, 96, 128, 192, 256])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_flash_attention_forward_nonsquare(gpu, batch, heads, sq, sk, d, causal, dtype):
