@@ -99,6 +99,7 @@ _SIGNATURES = {
     "fg_rms_norm_backward_partial_rows": (c_i64, [c_i64, c_i64, c_int, c_int]),
     "fg_rms_norm_backward": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_vp]),
     "fg_rms_norm_backward_dw": (c_int, [c_vp, c_i64, c_i64, c_vp, c_int, c_vp]),
+    "fg_transpose2d": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
     "fg_gemm_workspace_bytes": (ctypes.c_size_t, [c_i64, c_i64, c_i64, c_int, c_int, c_int]),
     "fg_gemm": (
         c_int,

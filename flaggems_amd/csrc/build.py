@@ -19,6 +19,7 @@ SOURCES = [
     "norm.hip",
     "softmax.hip",
     "backward.hip",
+    "transpose.hip",
     "rope.hip",
     "kvcache.hip",
     "silu_mul.hip",

@@ -16,7 +16,26 @@ def _prepare(a, b):
     if b.stride(0) > 1 and b.stride(1) > 1:
         b = b.contiguous()
     assert a.shape[1] == b.shape[0], "incompatible dimensions"
+    # A column-major A (the X^T of a weight gradient) misses the direct-to-LDS and skinny kernels, which want
+    # A contiguous along K; one transposing copy of A (the library's own kernel) costs far less than the
+    # slower main loop once the output is 256 columns wide, or 64 when A has few rows.  Measured, bf16:
+    # 4096^3 209 -> 127 us, 65 x 4096 x 4096 195 -> 29 us, 16384 x 4096 x 11008 1954 -> 1393 us.
+    wide = b.shape[1] >= 256 or (b.shape[1] >= 64 and a.shape[0] <= 1024)
+    if (a.stride(0) == 1 and a.stride(1) > 1 and a.shape[0] > 1 and wide and a.is_cuda
+            and a.element_size() in (2, 4) and _C.supported_dtype(a.dtype)):
+        a = _transposed_copy(a)
     return a, b
+
+
+def _transposed_copy(a):
+    """Row-major copy of a column-major [M, K] matrix (memory [K, M]) with the library's transpose kernel."""
+    M, K = a.shape
+    out = torch.empty((M, K), dtype=a.dtype, device=a.device)
+    with _C.device_guard(a.device):
+        rc = _C.lib().fg_transpose2d(a.data_ptr(), out.data_ptr(), K, M, a.stride(1), K, a.element_size(),
+                                     _C.current_stream(a.device))
+    _C.check(rc, "fg_transpose2d")
+    return out
 
 
 def _kernel_covers(a, b):

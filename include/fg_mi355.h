@@ -107,6 +107,13 @@ int fg_rms_norm_backward(const void* x, const void* dy, const float* inv_rms, co
 int fg_rms_norm_backward_dw(const float* dw_partial, int64_t partial_rows, int64_t N, void* dw, int dtype,
                             void* stream);
 
+/* dst[c, r] = src[r, c] for a [rows, cols] source with unit column stride and a [cols, rows] destination with unit
+ * column stride (row strides in elements), elements of 2 or 4 bytes moved as bits.  No counterpart in the reference,
+ * whose Triton GEMMs read operands through any strides (src/flag_gems/ops/mm.py:54-134): the host side of mm uses
+ * it to turn a column-major A into the K-contiguous layout the fast GEMM kernels read. */
+int fg_transpose2d(const void* src, void* dst, int64_t rows, int64_t cols, int64_t src_row_stride,
+                   int64_t dst_row_stride, int elem_bytes, void* stream);
+
 /* Rotary embedding of q [n_tokens,Hq,D] and k [n_tokens,Hk,D] (element strides given as
  * {token, head, dim}); cos/sin [max_pos, D/2] with unit inner stride.  pos == NULL means
  * position = token_index % seq_len.  q_out/k_out may alias q/k (in-place).

@@ -334,3 +334,20 @@ def test_mm_unaligned_operands(gpu, M, N, K, dtype, a_col_major, b_col_major, sh
     bias = torch.randn(N, dtype=dtype, device=gpu)
     res = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
     gems_assert_close(res, O.addmm(bias, a, b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols,src_pad,dst_pad", [(64, 64, 0, 0), (4096, 1024, 0, 0), (1000, 130, 0, 0), (257, 511, 3, 5),
+                                                       (1, 7, 0, 0), (129, 1, 8, 8), (300, 200, 8, 16)])
+def test_transpose2d(gpu, rows, cols, src_pad, dst_pad, dtype):
+    """fg_transpose2d through the C ABI: bit-exact, ragged tiles, padded row strides, nothing written outside dst."""
+    from flaggems_amd import _C
+
+    torch.manual_seed(rows + cols)
+    src = torch.randn(rows, cols + src_pad, dtype=dtype, device=gpu)
+    dst = torch.full((cols, rows + dst_pad), 7.0, dtype=dtype, device=gpu)
+    rc = _C.lib().fg_transpose2d(src.data_ptr(), dst.data_ptr(), rows, cols, cols + src_pad, rows + dst_pad,
+                                 src.element_size(), _C.current_stream(src.device))
+    assert rc == 0, _C.last_error()
+    assert torch.equal(dst[:, :rows], src[:, :cols].t())
+    assert (dst[:, rows:] == 7.0).all()
