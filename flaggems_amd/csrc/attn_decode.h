@@ -29,6 +29,9 @@ struct DecodeArgs {
 };
 
 constexpr int kDecTile = 32;  // keys per wave tile
+// cache-policy bits of the K/V tile loads: non-temporal, every byte of the cache is read once per launch
+// (measured 5.4 -> 5.7-5.9 TB/s on 64 x 4096 keys, 5.7 -> 6.2 on 256 x 2048)
+constexpr int kDecLoadAux = 2;
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
@@ -123,16 +126,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
       const char* kp = kbase + (page * p.k_page_stride + (int64_t)slot * p.k_row_stride) * 2;
       const char* vp = vbase + (page * p.v_page_stride + (int64_t)slot * p.v_row_stride) * 2;
       if (full) {
-        __builtin_amdgcn_global_load_lds(FG_GLBP(kp + (krow_off + c16[j])), FG_LDSP(kdst + j * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(FG_GLBP(vp + (vrow_off + c16[j])), FG_LDSP(kdst + OPB + j * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(FG_GLBP(kp + (krow_off + c16[j])), FG_LDSP(kdst + j * 1024), 16, 0, kDecLoadAux);
+        __builtin_amdgcn_global_load_lds(FG_GLBP(vp + (vrow_off + c16[j])), FG_LDSP(kdst + OPB + j * 1024), 16, 0, kDecLoadAux);
       } else {
         // rows past the end read the last valid key instead (their scores are masked; stale cache contents
         // must not reach the accumulators)
         const bool valid = key + lane_key < k_len;
         const char* ks = valid ? kp + (krow_off + c16[j]) : klast + c16[j];
         const char* vs = valid ? vp + (vrow_off + c16[j]) : vlast + c16[j];
-        __builtin_amdgcn_global_load_lds(FG_GLBP(ks), FG_LDSP(kdst + j * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(FG_GLBP(vs), FG_LDSP(kdst + OPB + j * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(FG_GLBP(ks), FG_LDSP(kdst + j * 1024), 16, 0, kDecLoadAux);
+        __builtin_amdgcn_global_load_lds(FG_GLBP(vs), FG_LDSP(kdst + OPB + j * 1024), 16, 0, kDecLoadAux);
       }
     }
   };
