@@ -61,12 +61,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
   const int t_begin = split * a.tiles_per_split;
   int t_end = t_begin + a.tiles_per_split;
   t_end = t_end < tiles_total ? t_end : tiles_total;
-  const bool has_work = q_len > 0 && t_begin < t_end;
+  // exactly one query token: in a mixed batch the sequences with more belong to the prefill kernels
+  const bool has_work = q_len == 1 && t_begin < t_end;
 
   // ---- Q fragments: row r < G is query head kvh*G + r of this sequence's token; other rows are zero ---------
   Frag qf[KS];
   {
-    const bool row_ok = ql < G && q_len > 0;
+    const bool row_ok = ql < G && q_len == 1;
     const T* qp = (const T*)p.q + (int64_t)q_bos * p.q_row_stride + (int64_t)(kvh * G + (row_ok ? ql : 0)) * p.q_head_stride;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
         for (int e = 0; e < 4; ++e) osum[(wave * G + ql) * D + dt * 32 + g * 8 + half * 4 + e] = o_acc[dt][g * 4 + e] * my_scale;
   }
   __syncthreads();
-  if (q_len <= 0) return;
+  if (q_len != 1) return;
   // thread i sums element i of the [G][D] block over the waves
   for (int i = tid; i < G * D; i += 256) {
     const int r = i / D, d = i - r * D;
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(256) void attn_decode_combine_kernel(DecodeArgs a) 
   const int head = (int)(bh % p.Hq);
   const int b = (int)(bh / p.Hq);
   const int q_bos = p.cu_seqlens_q[b];
-  if (p.cu_seqlens_q[b + 1] - q_bos <= 0) return;
+  if (p.cu_seqlens_q[b + 1] - q_bos != 1) return;
   float m = -INFINITY;
   for (int s = 0; s < a.splits; ++s) m = fmaxf(m, a.part_ml[(((int64_t)s * p.batch + b) * p.Hq + head) * 2]);
   float l = 0.f, o = 0.f;

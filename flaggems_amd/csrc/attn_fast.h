@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_fast_kernel(AttnArgs a) {
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
   const int k_len = p.seqused_k[b];
   const int block_row0 = m_block * a.rows_per_block;
-  if (block_row0 >= q_len) return;
+  if (block_row0 >= q_len || (a.skip_single && q_len == 1)) return;
   // As the second pass behind the head-pair kernel: only blocks that kernel has marked (its blocks hold two
   // of these in the row direction).
   if (a.redo_rows != 0 &&

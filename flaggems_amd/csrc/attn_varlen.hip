@@ -68,6 +68,7 @@ struct AttnArgs {
   int* redo_flags;    // head-pair kernel: one flag per workgroup, set when the block has to be redone by the lean kernel
   int redo_rows;      // lean kernel as the second pass: query rows per flagged block (0: ordinary launch)
   int redo_grid_x;    // ... and the first grid dimension of the flagging launch
+  int skip_single;    // mixed batch: sequences with one query token are left to the single-token kernel
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_varlen_kernel(AttnArgs a) {
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
   const int k_len = p.seqused_k[b];
   const int block_row0 = m_block * a.rows_per_block;
-  if (block_row0 >= q_len) return;
+  if (block_row0 >= q_len || (a.skip_single && q_len == 1)) return;
 
   // wave -> (head, row block)
   const int waves_per_head = 4 / a.hpb;
@@ -411,7 +412,7 @@ __global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_asyn
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
   const int k_len = p.seqused_k[b];
   const int block_row0 = m_block * a.rows_per_block;
-  if (block_row0 >= q_len) return;
+  if (block_row0 >= q_len || (a.skip_single && q_len == 1)) return;
 
   const int waves_per_head = NW / a.hpb;
   const int head = hgroup * a.hpb + wave / waves_per_head;
@@ -798,8 +799,9 @@ int decode_num_cu() {
 }
 // Decides whether the single-token kernel takes these parameters and, if so, how the key ranges are cut.
 // Without a large enough workspace the ranges are not split beyond what the kernel itself requires.
-bool decode_setup(const FgFlashParams& p, DecodeArgs* d) {
-  if (p.max_seqlen_q != 1 || !(p.D == 64 || p.D == 128) || p.alibi_slopes != nullptr || p.softcap > 0.f) return false;
+// `mixed`: the batch may also hold sequences with more than one query token (they are skipped by the kernel).
+bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
+  if ((p.max_seqlen_q != 1 && !mixed) || !(p.D == 64 || p.D == 128) || p.alibi_slopes != nullptr || p.softcap > 0.f) return false;
   if (p.window_left >= 0 && p.window_left < p.max_seqlen_k) return false;
   if (p.Hk <= 0 || p.Hq % p.Hk != 0 || p.Hq / p.Hk > 32) return false;
   int shift = -1;
@@ -827,6 +829,15 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d) {
   d->tiles_per_split = tps;
   d->part_o = splits > 1 ? (float*)p.workspace : nullptr;
   d->part_ml = splits > 1 ? (float*)p.workspace + (size_t)splits * p.batch * p.Hq * p.D : nullptr;
+  return true;
+}
+// A batch of at least four sequences with max_seqlen_q > 1 is treated as mixed: the single-token kernel takes the
+// sequences with one query token (it streams K/V 2-3 times faster than the prefill kernels do for one row, and
+// splits long sequences), the prefill kernel skips them.  Both read the lengths on the device; a batch without
+// such sequences pays two launches of workgroups that leave at once.
+bool mixed_batch(const FgFlashParams& p) {
+  if (p.max_seqlen_q <= 1 || p.batch < 4) return false;
+  if (const char* e = getenv("FG_ATTN_MIXED")) return e[0] != '0';
   return true;
 }
 // Head-pair kernel: applicable?  If so, its block shape and the size of its flag array.
@@ -859,7 +870,7 @@ extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int dev
   p.workspace_bytes = INT64_MAX;
   (void)device;
   DecodeArgs d;
-  if (decode_setup(p, &d)) return decode_workspace_bytes(p, d.splits);
+  if (decode_setup(p, &d, mixed_batch(p))) return decode_workspace_bytes(p, d.splits);
   int hpb = 0, rows = 0;
   size_t flag_bytes = 0;
   if (pair_plan(p, &hpb, &rows, &flag_bytes)) return flag_bytes;
@@ -890,15 +901,21 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   FG_REQUIRE(p.batch < 65536 && p.Hq < 65536, FG_ERR_UNSUPPORTED, "flash_attn_varlen_fwd: batch/heads exceed the grid");
 
   hipStream_t st = (hipStream_t)stream;
+  bool skip_single = false;
   {
     DecodeArgs d;
-    if (decode_setup(p, &d)) {
-      if (p.dtype == FG_F16) return p.D == 64 ? launch_decode<f16_t, 64>(d, st) : launch_decode<f16_t, 128>(d, st);
-      return p.D == 64 ? launch_decode<bf16_t, 64>(d, st) : launch_decode<bf16_t, 128>(d, st);
+    const bool mixed = mixed_batch(p);
+    if (decode_setup(p, &d, mixed)) {
+      int rc;
+      if (p.dtype == FG_F16) rc = p.D == 64 ? launch_decode<f16_t, 64>(d, st) : launch_decode<f16_t, 128>(d, st);
+      else rc = p.D == 64 ? launch_decode<bf16_t, 64>(d, st) : launch_decode<bf16_t, 128>(d, st);
+      if (!mixed || rc != FG_OK) return rc;
+      skip_single = true;  // the prefill kernel below handles every other sequence
     }
   }
   AttnArgs a;
   a.p = p;
+  a.skip_single = skip_single ? 1 : 0;
   const int ratio = p.Hq / p.Hk;
   a.hpb = ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1);
   a.page_shift = -1;

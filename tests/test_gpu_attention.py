@@ -85,6 +85,27 @@ def test_flash_attn_varlen_edges(gpu):
     check(gpu, [(1, 17), (1, 1000), (1, 1), (1, 4096)], 32, 8, 128, 16, 2048, torch.bfloat16)
 
 
+# Mixed batches, as a serving engine with chunked prefill produces them: sequences with one query token go to the
+# single-token kernel (split key ranges), the rest to the prefill kernels, in one call.  Also: a batch of four or
+# more without any single-token sequence, one made of nothing else but with max_seqlen_q > 1 passed, empty
+# sequences in between, a non-causal batch, and the same batches with the routing switched off.
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hk,D,block_size", [(32, 8, 128, 16), (8, 8, 64, 32), (12, 4, 128, 64)])
+@pytest.mark.parametrize("mixed_env", [None, "0"])
+def test_flash_attn_mixed_batches(gpu, monkeypatch, dtype, Hq, Hk, D, block_size, mixed_env):
+    if mixed_env is None:
+        monkeypatch.delenv("FG_ATTN_MIXED", raising=False)
+    else:
+        monkeypatch.setenv("FG_ATTN_MIXED", mixed_env)
+    check(gpu, [(1, 700), (1, 33), (300, 300), (1, 4096), (64, 1000), (1, 1), (1, 2500), (17, 17)], Hq, Hk, D, block_size,
+          2048, dtype)
+    check(gpu, [(128, 128), (5, 900), (200, 1200), (33, 64)], Hq, Hk, D, block_size, 1024, dtype)
+    check(gpu, [(1, 100), (1, 2000), (1, 3), (1, 513), (1, 64)], Hq, Hk, D, block_size, 1024, dtype)
+    check(gpu, [(1, 40), (0, 0), (70, 70), (1, 0), (0, 50), (1, 900)], Hq, Hk, D, block_size, 512, dtype)
+    check(gpu, [(1, 300), (40, 300), (1, 1000), (2, 77)], Hq, Hk, D, block_size, 512, dtype, causal=False)
+    check(gpu, [(1, 300), (40, 300), (1, 1000), (2, 77)], Hq, Hk, D, block_size, 512, dtype, window=(128, 0))
+
+
 # The head-pair kernel (two heads of a KV group per wave, software-pipelined tiles; opt-in through the
 # environment): same oracle, same tolerances.  The last case feeds scores that keep growing along the keys, so
 # that rows leave the exponent headroom above their fixed softmax reference and the blocks are handed to the
