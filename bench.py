@@ -23,6 +23,7 @@ It is a reported baseline, never the thing optimised.
 import argparse
 import json
 import math
+import random
 import os
 import sys
 import time
@@ -308,6 +309,42 @@ def main():
                     workload="flash_attn_varlen_func decode: 64 seqs x 4096 keys, 1 query token each, 32q/8kv heads, D 128, page 16",
                     cpu=(cpu, 2 * S * Hk * D * 2, "oracle paged attention (torch CPU fp32) on one sequence"))
 
+    def wl_mixed():
+        # what a serving engine with chunked prefill sends in one call: many decoding sequences and a few prefill chunks
+        Hq, Hk, D, bs = 32, 8, 128, 16
+        rng = random.Random(0)
+        lens = [(1, rng.randint(2048, 4096)) for _ in range(60)] + [(512, 512 + 1024 * i) for i in range(4)]
+        qlens, klens = [l[0] for l in lens], [l[1] for l in lens]
+        nblk = sum((k + bs - 1) // bs for k in klens)
+        torch.manual_seed(0)
+        q = torch.randn(sum(qlens), Hq, D, device=dev).to(bf16)
+        kc = torch.randn(nblk, bs, Hk, D, device=dev).to(bf16)
+        vc = torch.randn(nblk, bs, Hk, D, device=dev).to(bf16)
+        cu = torch.tensor([0] + qlens, dtype=torch.int32).cumsum(0, dtype=torch.int32).to(dev)
+        sk = torch.tensor(klens, dtype=torch.int32, device=dev)
+        perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(0))
+        bt = torch.zeros(len(lens), (max(klens) + bs - 1) // bs, dtype=torch.int32)
+        o = 0
+        for i, k in enumerate(klens):
+            n = (k + bs - 1) // bs
+            bt[i, :n] = perm[o:o + n]
+            o += n
+        bt = bt.to(dev)
+
+        def run(i):
+            flag_gems.flash_attn_varlen_func(q, kc, vc, max(qlens), cu, max(klens), seqused_k=sk, causal=True, block_table=bt)
+
+        qc, kcc, vcc, btc = q[:1].cpu(), kc.cpu(), vc.cpu(), bt[:1].cpu()
+
+        def cpu():
+            O.paged_attention(qc, kcc, vcc, [1], [klens[0]], btc, D ** -0.5, compute_dtype=torch.float32)
+
+        kv_bytes = 2 * sum(klens) * Hk * D * 2  # every K and V row once per KV head
+        return dict(run=run, work=kv_bytes + 2 * sum(qlens) * Hq * D * 2, bound="hbm", dtype="bf16",
+                    workload="flash_attn_varlen_func mixed batch: 60 decoding sequences of 2048-4096 keys + 4 prefill chunks of "
+                             "512 tokens behind 0-3072 cached keys, 32q/8kv heads, D 128, page 16 (bytes: K/V once per KV head)",
+                    cpu=(cpu, 2 * klens[0] * Hk * D * 2, "oracle paged attention (torch CPU fp32) on the first sequence"))
+
     def wl_sdpa():
         # dense causal attention through scaled_dot_product_attention (the caller's (batch, heads, seq, d) tensors
         # are used in place as a virtual paged cache)
@@ -440,6 +477,7 @@ def main():
         "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
         "flash_attn_c4": wl_attn_c4,
         "flash_attn_decode": wl_decode,
+        "flash_attn_mixed": wl_mixed,
         "sdpa_dense": wl_sdpa,
         "decoder_layer_c5": wl_layer_c5,
         "mfma_ceiling_random": lambda: wl_mfma_ceiling(True),
