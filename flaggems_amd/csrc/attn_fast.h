@@ -51,7 +51,11 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_fast_kernel(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it is wave-uniform
   const int half = lane >> 5, ql = lane & 31;
-  const int m_block = gridDim.x - 1 - blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+  // Long (late) row blocks first, and the order rotated per (sequence, head group): workgroups go round-robin to the
+  // 8 XCDs by their linear id, so without the rotation a batch whose sequences have one row block each (and
+  // gridDim.x a multiple of 8) would put all of its work on one XCD.
+  const int b = blockIdx.y, hgroup = blockIdx.z;
+  const int m_block = (int)((gridDim.x - 1 - blockIdx.x + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;

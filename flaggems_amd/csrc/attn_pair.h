@@ -97,7 +97,9 @@ __global__ __launch_bounds__(256, 1) void attn_varlen_pair_kernel(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, ql = lane & 31;
-  const int m_block = gridDim.x - 1 - blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+  const int b = blockIdx.y, hgroup = blockIdx.z;
+  // long row blocks first, rotated per (sequence, head group) as in the lean kernel
+  const int m_block = (int)((gridDim.x - 1 - blockIdx.x + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;

@@ -88,7 +88,9 @@ __global__ __launch_bounds__(256) void attn_varlen_kernel(AttnArgs a) {
   const FgFlashParams& p = a.p;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, ql = lane & 31;
-  const int m_block = blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+  const int b = blockIdx.y, hgroup = blockIdx.z;
+  // rotated per (sequence, head group) so that sequences of one row block do not all land on one XCD
+  const int m_block = (int)((blockIdx.x + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
@@ -406,7 +408,11 @@ __global__ __launch_bounds__(NW * 64, (RB <= 256 ? 2 : 1)) void attn_varlen_asyn
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, ql = lane & 31;
   // long (late) row blocks first: they take the most steps under a causal mask
-  const int m_block = gridDim.x - 1 - blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+  // Long (late) row blocks first, and the order rotated per (sequence, head group): workgroups go round-robin to the
+  // 8 XCDs by their linear id, so without the rotation a batch whose sequences have one row block each (and
+  // gridDim.x a multiple of 8) would put all of its work on one XCD.
+  const int b = blockIdx.y, hgroup = blockIdx.z;
+  const int m_block = (int)((gridDim.x - 1 - blockIdx.x + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
