@@ -23,12 +23,24 @@ struct DecodeArgs {
   int page_shift;
   int group;             // query heads per KV head
   int splits;            // key ranges per sequence (grid x)
-  int tiles_per_split;   // 32-key tiles per range, a multiple of 4
+  int tiles_per_split;   // most 32-key tiles per range, a multiple of 4 (cut for max_seqlen_k)
+  int min_tiles;         // fewest 32-key tiles per range of a shorter sequence, a multiple of 4
   float* part_o;         // [splits][batch][Hq][D] fp32, unnormalised   (splits > 1)
   float* part_ml;        // [splits][batch][Hq][2] fp32: maximum (base 2), sum
 };
 
 constexpr int kDecTile = 32;  // keys per wave tile
+
+// Tiles per key range of one sequence.  The host cuts the ranges for max_seqlen_k, which it knows; a sequence
+// may be much shorter (a batch with one long sequence, or a caller that passes the model's limit), and with the
+// host's cut its keys would fill the first range or two and leave the other workgroups of the sequence without
+// work.  So each sequence spreads its own tiles over all `splits` ranges, down to `min_tiles` per range.
+__device__ inline int decode_range_tiles(const DecodeArgs& a, int tiles_total) {
+  int t = (tiles_total + a.splits - 1) / a.splits;
+  t = (t + 3) & ~3;
+  t = t < a.min_tiles ? a.min_tiles : t;
+  return t < a.tiles_per_split ? t : a.tiles_per_split;
+}
 // cache-policy bits of the K/V tile loads: non-temporal, every byte of the cache is read once per launch
 // (measured 5.4 -> 5.7-5.9 TB/s on 64 x 4096 keys, 5.7 -> 6.2 on 256 x 2048)
 constexpr int kDecLoadAux = 2;
@@ -51,18 +63,26 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, ql = lane & 31;
-  const int split = blockIdx.x, b = blockIdx.y, kvh = blockIdx.z;
+  const int b = blockIdx.y, kvh = blockIdx.z;
+  // Key range, rotated per (sequence, KV head): workgroups go round-robin to the 8 XCDs by their linear id, and a
+  // short sequence has work in range 0 only, so with 8 ranges every short sequence of a batch would land on one XCD.
+  const int split = (int)((blockIdx.x + (unsigned)(b * 5 + kvh * 3)) % gridDim.x);
   const int G = a.group;
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
   const int k_len = p.seqused_k[b];
   const int tiles_total = (k_len + kDecTile - 1) / kDecTile;
-  const int t_begin = split * a.tiles_per_split;
-  int t_end = t_begin + a.tiles_per_split;
+  const int range_tiles = decode_range_tiles(a, tiles_total);
+  const int t_begin = split * range_tiles;
+  int t_end = t_begin + range_tiles;
   t_end = t_end < tiles_total ? t_end : tiles_total;
   // exactly one query token: in a mixed batch the sequences with more belong to the prefill kernels
-  const bool has_work = q_len == 1 && t_begin < t_end;
+  if (q_len != 1) return;
+  // a key range past the end of this sequence: nothing to do, and the merge does not read its partial results
+  // (range 0 always reports, so that a sequence without keys still gets its zeros)
+  if (split > 0 && t_begin >= t_end) return;
+  const bool has_work = t_begin < t_end;
 
   // ---- Q fragments: row r < G is query head kvh*G + r of this sequence's token; other rows are zero ---------
   Frag qf[KS];
@@ -335,10 +355,15 @@ __global__ __launch_bounds__(256) void attn_decode_combine_kernel(DecodeArgs a) 
   const int b = (int)(bh / p.Hq);
   const int q_bos = p.cu_seqlens_q[b];
   if (p.cu_seqlens_q[b + 1] - q_bos != 1) return;
+  // key ranges that hold keys of this sequence (the others were not written)
+  const int tiles_total = (p.seqused_k[b] + kDecTile - 1) / kDecTile;
+  const int range_tiles = decode_range_tiles(a, tiles_total);
+  int ns = (tiles_total + range_tiles - 1) / range_tiles;
+  ns = ns < 1 ? 1 : (ns > a.splits ? a.splits : ns);
   float m = -INFINITY;
-  for (int s = 0; s < a.splits; ++s) m = fmaxf(m, a.part_ml[(((int64_t)s * p.batch + b) * p.Hq + head) * 2]);
+  for (int s = 0; s < ns; ++s) m = fmaxf(m, a.part_ml[(((int64_t)s * p.batch + b) * p.Hq + head) * 2]);
   float l = 0.f, o = 0.f;
-  for (int s = 0; s < a.splits; ++s) {
+  for (int s = 0; s < ns; ++s) {
     const int64_t row = ((int64_t)s * p.batch + b) * p.Hq + head;
     const float ms = a.part_ml[row * 2];
     if (ms == -INFINITY) continue;
@@ -358,7 +383,12 @@ inline void decode_plan(const FgFlashParams& p, int page_shift, int num_cu, int*
   const int64_t range_cap = (int64_t)256 << page_shift < 4096 ? (int64_t)256 << page_shift : 4096;  // keys
   int64_t need = fg_cdiv(max_k, range_cap);
   const int64_t wgs = (int64_t)p.batch * p.Hk;
-  int64_t want = fg_cdiv((int64_t)2 * num_cu, wgs > 0 ? wgs : 1);
+  int per_cu = 2;
+  if (const char* e = getenv("FG_DECODE_WG_PER_CU")) {
+    const int v = atoi(e);
+    if (v >= 1 && v <= 64) per_cu = v;
+  }
+  int64_t want = fg_cdiv((int64_t)per_cu * num_cu, wgs > 0 ? wgs : 1);
   const int64_t most = max_k / 512 > 1 ? max_k / 512 : 1;
   if (want > most) want = most;
   int64_t s = need > want ? need : want;

@@ -833,6 +833,11 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
   d->group = p.Hq / p.Hk;
   d->splits = splits;
   d->tiles_per_split = tps;
+  d->min_tiles = 16;
+  if (const char* e = getenv("FG_DECODE_MIN_TILES")) {
+    const int v = atoi(e);
+    if (v >= 4 && v % 4 == 0) d->min_tiles = v;
+  }
   d->part_o = splits > 1 ? (float*)p.workspace : nullptr;
   d->part_ml = splits > 1 ? (float*)p.workspace + (size_t)splits * p.batch * p.Hq * p.D : nullptr;
   return true;

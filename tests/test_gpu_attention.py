@@ -183,6 +183,32 @@ def test_flash_attn_decode_variants(gpu):
     torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
 
 
+# max_seqlen_k is an upper bound, not the longest length present (a caller may pass the model's limit, and one long
+# sequence sets it for a whole batch): each sequence cuts its own key ranges from its own length on the device,
+# and the merge must read exactly the ranges that sequence wrote.
+@pytest.mark.parametrize("max_k", [4096, 32768, 131072])
+@pytest.mark.parametrize("min_tiles", [None, "4", "64"])
+def test_flash_attn_decode_max_seqlen_k_above_lengths(gpu, monkeypatch, max_k, min_tiles):
+    if min_tiles is not None:
+        monkeypatch.setenv("FG_DECODE_MIN_TILES", min_tiles)
+    lens = [(1, n) for n in (2048, 1, 0, 31, 129, 511, 513, 2047, 2049, 3000, 4096, 640)] + [(1, 700 + 61 * i) for i in range(24)]
+    q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16)
+    wide = torch.zeros(bt.shape[0], max_k // 16, dtype=bt.dtype, device=bt.device)
+    wide[:, :bt.shape[1]] = bt
+    out, lse = flag_gems.ops.flash_attn_varlen_func(q, kc, vc, 1, cu, max_k, seqused_k=sk, causal=True, block_table=wide,
+                                                    return_softmax_lse=True)
+    ref, rlse = O.paged_attention(q, kc, vc, qlens, klens, bt, 128 ** -0.5, causal=True, compute_dtype=torch.float32,
+                                  return_lse=True)
+    torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
+    lse = lse.cpu()
+    fin = torch.isfinite(rlse)
+    torch.testing.assert_close(lse[fin], rlse[fin], atol=1e-2, rtol=1e-3)
+    assert (lse[~fin] == float("inf")).all()  # the sequence without keys: out = 0, lse = +inf
+    # the same batch with one sequence that really is that long (bounded so the oracle stays quick)
+    if max_k == 32768:
+        check(gpu, lens[:8] + [(1, 32768)], 32, 8, 128, 16, 4096, torch.bfloat16)
+
+
 # Dense attention through the same kernel: aten::_flash_attention_forward and scaled_dot_product_attention
 # (reference: tests/test_attention_ops.py:540-575 test_flash_fwd_nonsquare_qk, :578-640 GQA and alibi, :296-330 sdpa).
 def _dense_inputs(dev, batch, heads, heads_k, sq, sk, d, dtype):
