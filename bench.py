@@ -115,6 +115,14 @@ def main():
         ts.sort()
         return ts[len(ts) // 2]
 
+    # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs scaled by what the
+    # same counters read for a plain 512 MiB copy (profiles/hbm_traffic_*.txt hold the runs and their commands)
+    TRAFFIC = {
+        "softmax_c2": 1073780000,
+        "mm_c3a_8192": 1771500000,
+        "flash_attn_c4": 1835830000,
+    }
+
     cores = torch.get_num_threads()
     from oracle import torch_ref as O  # the checker, used here only for the cpu_baseline leg
 
@@ -142,16 +150,18 @@ def main():
 
         # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
         # read for a plain 512 MiB copy (profiles/hbm_traffic_softmax_mm_attention.txt)
-        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=1073780000,
+        return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=TRAFFIC.get("softmax_c2"),
                     workload="softmax dim=-1 [131072,2048] bf16, N(0,4) with 1% -inf (BASELINE.json configs[1])",
                     cpu=(cpu, 2 * 32768 * N * 2, "oracle softmax (torch CPU, fp64 upcast) on the first 32768 rows"))
 
-    def wl_fused_add_rms_norm_c1():
+    def wl_fused_add_rms_norm_c1(dt=bf16):
         torch.manual_seed(0)
-        M, N, sets = 4096, 4096, 6  # 6 x 64 MiB of x+residual: rotates through more than the 256 MB cache
-        xs = [torch.randn(M, N).to(bf16).to(dev) for _ in range(sets)]
-        rs = [torch.randn(M, N).to(bf16).to(dev) for _ in range(sets)]
-        w = (torch.rand(N) + 0.5).to(bf16).to(dev)
+        eb = 2 if dt is bf16 else 4
+        M, N = 4096, 4096
+        sets = 6 if dt is bf16 else 3  # 6 x 64 MiB (3 x 128 MiB) of x+residual: rotates through more than the 256 MB cache
+        xs = [torch.randn(M, N).to(dt).to(dev) for _ in range(sets)]
+        rs = [torch.randn(M, N).to(dt).to(dev) for _ in range(sets)]
+        w = (torch.rand(N) + 0.5).to(dt).to(dev)
 
         def run(i):
             flag_gems.fused_add_rms_norm(xs[i % sets], rs[i % sets], [N], w, 1e-6)
@@ -161,8 +171,10 @@ def main():
         def cpu():
             O.fused_add_rms_norm(xc, rc, wc, 1e-6)
 
-        return dict(run=run, work=4 * M * N * 2 + N * 2, bound="hbm", dtype="bf16",
-                    workload="fused_add_rms_norm [4096,4096] bf16, eps 1e-6 (configs[0] shape)",
+        return dict(run=run, work=4 * M * N * eb + N * eb, bound="hbm", dtype="bf16" if dt is bf16 else "f32",
+                    traffic={2: TRAFFIC.get("fused_add_rms_norm_c1"), 4: TRAFFIC.get("fused_add_rms_norm_c1_fp32")}[eb],
+                    workload="fused_add_rms_norm [4096,4096] %s, eps 1e-6 (configs[0]%s)"
+                             % ("bf16" if dt is bf16 else "fp32", " shape" if dt is bf16 else ", its stated precision"),
                     cpu=(cpu, 4 * M * N * 4 + N * 4, "oracle fused_add_rms_norm (torch CPU, fp32 in / fp64 math) on the full [4096,4096]"))
 
     def wl_softmax_backward():
@@ -206,17 +218,24 @@ def main():
                              "(one kernel + the sum of its partial rows)",
                     cpu=(cpu, 3 * 2048 * N * 2, "oracle rms_norm_grads (torch CPU autograd, fp64) on the first 2048 rows"))
 
-    def wl_mm(M, N, K, name, b_t=False, bias=False, bound="mfma"):
+    def wl_mm(M, N, K, name, b_t=False, bias=False, bound="mfma", key=None):
         def make():
             torch.manual_seed(0)
             a = (torch.randn(M, K) / math.sqrt(K)).to(bf16).to(dev)
             b = ((torch.randn(N, K) / math.sqrt(K)).to(bf16).to(dev).t() if b_t
                  else (torch.randn(K, N) / math.sqrt(K)).to(bf16).to(dev))
+            # a bandwidth-bound problem streams its weights: rotate through copies of B that together exceed
+            # the 256 MB last-level cache, so the rate is an HBM rate (what a decoding model sees)
+            copies = 1
+            if bound == "hbm":
+                copies = max(3, -(-320 * 2 ** 20 // (N * K * 2)))
+            bs_ = [b] + [b.clone() if not b_t else b.t().clone().t() for _ in range(copies - 1)]
             bi = (torch.randn(N) * 0.02).to(bf16).to(dev) if bias else None
             state = {}
 
             def run(i):
-                state["c"] = flag_gems.addmm(bi, a, b) if bias else flag_gems.mm(a, b)
+                bb = bs_[i % copies]
+                state["c"] = flag_gems.addmm(bi, a, bb) if bias else flag_gems.mm(a, bb)
 
             rows = min(M, 512)
             ac, bc = a[:rows].cpu().float(), b.cpu().float()
@@ -233,8 +252,9 @@ def main():
             d = dict(run=run, work=work, bound=bound, dtype="bf16", workload=name,
                      cpu=(cpu, cw, "torch.mm on the host in fp32, first %d rows of A" % rows))
             d["post"] = lambda: {"schedule": {1: "data-parallel", 2: "stream-K"}.get(_gemm.last_schedule())}
-            if (M, N, K) == (8192, 8192, 8192) and not b_t and not bias:
-                d["traffic"] = 1771500000  # measured as for softmax; 6x the compulsory A + B + C because of L2 misses
+            d["traffic"] = TRAFFIC.get(key)
+            if copies > 1:
+                d["workload"] += " [B rotated through %d copies = %d MB]" % (copies, copies * N * K * 2 // 2 ** 20)
             return d
         return make
 
@@ -281,7 +301,7 @@ def main():
         def cpu():
             O.paged_attention(qc, kcc, vcc, [ls], [ls], btc, D ** -0.5, compute_dtype=torch.float32)
 
-        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=1835830000,
+        return dict(run=run, work=flops, bound="mfma", dtype="bf16", traffic=TRAFFIC.get("flash_attn_c4"),
                     workload="flash_attn_varlen_func causal GQA prefill, 16 seqs U[512,4096] (sum 35846), 32q/8kv heads, D 128, page 16 (configs[3])",
                     cpu=(cpu, 4 * D * Hq * ls * (ls + 1) // 2, "oracle paged attention (torch CPU fp32) on the shortest sequence (%d tokens)" % ls))
 
@@ -306,6 +326,7 @@ def main():
             O.paged_attention(qc, kcc, vcc, [1], [S], btc, D ** -0.5, compute_dtype=torch.float32)
 
         return dict(run=run, work=2 * B * S * Hk * D * 2 + 2 * B * Hq * D * 2, bound="hbm", dtype="bf16",
+                    traffic=TRAFFIC.get("flash_attn_decode"),
                     workload="flash_attn_varlen_func decode: 64 seqs x 4096 keys, 1 query token each, 32q/8kv heads, D 128, page 16",
                     cpu=(cpu, 2 * S * Hk * D * 2, "oracle paged attention (torch CPU fp32) on one sequence"))
 
@@ -413,20 +434,50 @@ def main():
 
         lin = 2 * T * Hd * (3 * Hd + Hd + 2 * F + F)
         att = B * 4 * D * H * S * (S + 1) // 2
+        e2 = 2  # bytes per element
+        # algorithmic work of every operator of the layer: (bound, flop or bytes)
+        op_work = {
+            "rms_norm": ("hbm", 2 * T * Hd * e2 + Hd * e2),
+            "mm_qkv": ("mfma", 2 * T * Hd * 3 * Hd),
+            "rope": ("hbm", 2 * 2 * T * Hd * e2),
+            "reshape_and_cache_flash": ("hbm", 2 * 2 * T * Hd * e2),
+            "flash_attn_varlen": ("mfma", att),
+            "mm_o": ("mfma", 2 * T * Hd * Hd),
+            "fused_add_rms_norm(+clone)": ("hbm", (4 + 2) * T * Hd * e2 + Hd * e2),
+            "mm_gate_up": ("mfma", 2 * T * Hd * 2 * F),
+            "silu_and_mul": ("hbm", 3 * T * F * e2),
+            "mm_down": ("mfma", 2 * T * F * Hd),
+            "residual_add": ("hbm", 3 * T * Hd * e2),
+        }
 
         def post():
-            rec = []
-            run(0, rec)
-            torch.cuda.synchronize()
-            ops = {}
-            for (n0, e0), (n1_, e1) in zip(rec[:-1], rec[1:]):
-                ops[n1_] = round(e0.elapsed_time(e1), 4)
+            reps = 3
+            acc = {}
+            for _ in range(reps):
+                rec = []
+                run(0, rec)
+                torch.cuda.synchronize()
+                for (n0, e0), (n1_, e1) in zip(rec[:-1], rec[1:]):
+                    acc.setdefault(n1_, []).append(e0.elapsed_time(e1))
+            ops = {n: round(sorted(v)[len(v) // 2], 4) for n, v in acc.items()}
+            per_op = {n: roofline(op_work[n][0], op_work[n][1], ms) for n, ms in ops.items()}
             lib._destroy()
-            return {"per_op_ms": ops, "linear_flop": lin, "attention_flop": att}
+            return {"per_op_ms": ops, "per_op_roofline": per_op, "linear_flop": lin, "attention_flop": att}
 
+        # CPU baseline: the fp32 layer oracle on the first 256 tokens of one sequence
+        cs = 256
+        hc, posc = h[:cs].cpu(), pos[:cs].cpu()
+        wc = [w.cpu() for w in (wqkv, wo, wgu, wd, n1, n2)]
+        cosc, sinc = cos.cpu(), sin.cpu()
+
+        def cpu():
+            O.decoder_layer(hc, wc[0], wc[1], wc[2], wc[3], wc[4], wc[5], posc, cosc, sinc, 1e-5, H)
+
+        cwork = 2 * cs * Hd * (3 * Hd + Hd + 2 * F + F) + 4 * D * H * cs * (cs + 1) // 2
         return dict(run=run, work=lin + att, bound="mfma", dtype="bf16",
                     workload="Llama-2-7B decoder layer forward under flag_gems.enable(), 8 x 2048-token prefill, paged KV (configs[4])",
-                    cpu=None, post=post)
+                    cpu=(cpu, cwork, "layer oracle (torch CPU fp32, per-operator bf16 rounding) on the first %d tokens of one sequence" % cs),
+                    post=post)
 
     def wl_copy_ref():
         # plain device copy of known size (torch's elementwise copy kernel): the yardstick the
@@ -463,18 +514,21 @@ def main():
     workloads = {
         "softmax_c2": wl_softmax_c2,
         "fused_add_rms_norm_c1": wl_fused_add_rms_norm_c1,
+        "fused_add_rms_norm_c1_fp32": lambda: wl_fused_add_rms_norm_c1(torch.float32),
         "softmax_backward": wl_softmax_backward,
         "rms_norm_backward": wl_rms_norm_backward,
-        "mm_c3a_8192": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B row-major (configs[2]a)"),
+        "mm_c3a_8192": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B row-major (configs[2]a)", key="mm_c3a_8192"),
         "mm_c3a_8192_nt": wl_mm(8192, 8192, 8192, "mm bf16 M=N=K=8192, B = W^T column-major (configs[2]a, weight layout)", b_t=True),
-        "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm"),
+        "mm_c3b_skinny": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, stream-K (configs[2]b)", bound="hbm",
+                               key="mm_c3b_skinny"),
         "mm_c3b_skinny_nt": wl_mm(16, 4096, 14336, "mm bf16 M=16 N=4096 K=14336, B = W^T of a [N, K] weight, stream-K",
                                   b_t=True, bound="hbm"),
         "mm_chunk_1024_nt": wl_mm(1024, 12288, 4096, "mm bf16 M=1024 N=12288 K=4096, B = W^T (a 1024-token prefill chunk "
                                   "through a fused QKV weight: less than one round of 256x256 tiles)", b_t=True),
         "mm_chunk_512_nt": wl_mm(512, 4096, 4096, "mm bf16 M=512 N=4096 K=4096, B = W^T (half a round of 128x128 tiles: "
                                  "each tile cut in two)", b_t=True),
-        "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True),
+        "addmm_c3c": wl_mm(4096, 11008, 4096, "addmm bf16 M=4096 N=11008 K=4096 + bias (configs[2]c)", bias=True,
+                           key="addmm_c3c"),
         "flash_attn_c4": wl_attn_c4,
         "flash_attn_decode": wl_decode,
         "flash_attn_mixed": wl_mixed,

@@ -100,6 +100,9 @@ _SIGNATURES = {
     "fg_rms_norm_backward": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_vp]),
     "fg_rms_norm_backward_dw": (c_int, [c_vp, c_i64, c_i64, c_vp, c_int, c_vp]),
     "fg_transpose2d": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
+    "fg_reload_options": (None, []),
+    "fg_gemm_workspace_layout": (c_int, [c_int, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
+    "fg_stream_capture_id": (c_int, [c_vp, ctypes.POINTER(ctypes.c_ulonglong)]),
     "fg_gemm_workspace_bytes": (ctypes.c_size_t, [c_i64, c_i64, c_i64, c_int, c_int, c_int]),
     "fg_gemm": (
         c_int,

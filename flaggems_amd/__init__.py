@@ -11,6 +11,7 @@ import logging
 import torch
 
 from . import config  # noqa: F401
+from . import custom_ops  # noqa: F401  (defines torch.ops.flag_gems.*)
 from . import runtime  # noqa: F401
 from . import testing  # noqa: F401
 from . import fused, ops  # noqa: F401

@@ -3,7 +3,8 @@
 The reference distinguishes a pure-Python (Triton) path from an optional C extension.  Here the
 native library is the only implementation, so `has_c_extension` reports whether it is built and
 `use_c_extension` stays False: the Python wrappers call the C ABI themselves rather than routing
-through torch.ops.flag_gems, and nothing is patched from C++ at import time.
+through torch.ops.flag_gems, and nothing is patched from C++ at import time.  The torch.ops.flag_gems
+namespace itself is defined (custom_ops.py) for callers that use it directly.
 """
 import os
 

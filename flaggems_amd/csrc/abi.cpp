@@ -1,4 +1,6 @@
 // Host-only part of libfg_mi355.so: error channel, device facts, stream-K partition arithmetic.
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include "fg_common.h"
 
@@ -20,6 +22,51 @@ int fg_check_launch(const char* what) {
     return FG_ERR_LAUNCH;
   }
   return FG_OK;
+}
+
+namespace {
+FgOptions g_opt;
+std::once_flag g_opt_once;
+void load_options() {
+  FgOptions o = {};
+  o.gemm_no_dma = getenv("FG_GEMM_NO_DMA") != nullptr;
+  o.gemm_sk_even = getenv("FG_GEMM_SK_EVEN") != nullptr;
+  if (const char* e = getenv("FG_GEMM_TILE")) {
+    int a = 0, b = 0;
+    char c = 0;
+    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && a > 0 && b > 0) {
+      o.gemm_tile_bm = a; o.gemm_tile_bn = b; o.gemm_tile_deep = c != 's';
+    }
+  }
+  o.skinny_no_lds = getenv("FG_SKINNY_NO_LDS") != nullptr;
+  o.skinny_rows64 = getenv("FG_SKINNY_ROWS64") != nullptr;
+  if (const char* e = getenv("FG_SKINNY_TILE")) {
+    const int v = atoi(e);
+    o.skinny_tile = v == 32 ? 32 : v == 16 ? 16 : 0;
+  }
+  if (const char* e = getenv("FG_ATTN_KERNEL")) strncpy(o.attn_kernel, e, sizeof(o.attn_kernel) - 1);
+  o.attn_mixed = -1;
+  if (const char* e = getenv("FG_ATTN_MIXED")) o.attn_mixed = e[0] != '0' ? 1 : 0;
+  if (const char* e = getenv("FG_DECODE_MIN_TILES")) {
+    const int v = atoi(e);
+    if (v >= 4 && v % 4 == 0) o.decode_min_tiles = v;
+  }
+  if (const char* e = getenv("FG_DECODE_WG_PER_CU")) {
+    const int v = atoi(e);
+    if (v >= 1 && v <= 64) o.decode_wg_per_cu = v;
+  }
+  g_opt = o;
+}
+}  // namespace
+
+const FgOptions& fg_options() {
+  std::call_once(g_opt_once, load_options);
+  return g_opt;
+}
+
+extern "C" void fg_reload_options(void) {
+  std::call_once(g_opt_once, [] {});
+  load_options();
 }
 
 extern "C" const char* fg_last_error(void) { return g_err; }

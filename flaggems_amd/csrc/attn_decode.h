@@ -384,10 +384,7 @@ inline void decode_plan(const FgFlashParams& p, int page_shift, int num_cu, int*
   int64_t need = fg_cdiv(max_k, range_cap);
   const int64_t wgs = (int64_t)p.batch * p.Hk;
   int per_cu = 2;
-  if (const char* e = getenv("FG_DECODE_WG_PER_CU")) {
-    const int v = atoi(e);
-    if (v >= 1 && v <= 64) per_cu = v;
-  }
+  if (fg_options().decode_wg_per_cu > 0) per_cu = fg_options().decode_wg_per_cu;
   int64_t want = fg_cdiv((int64_t)per_cu * num_cu, wgs > 0 ? wgs : 1);
   const int64_t most = max_k / 512 > 1 ? max_k / 512 : 1;
   if (want > most) want = most;

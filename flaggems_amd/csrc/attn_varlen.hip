@@ -814,7 +814,7 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
   for (int sft = 0; sft < 31; ++sft)
     if ((1 << sft) == p.page_size) shift = sft;
   if (shift < 4) return false;
-  if (const char* force = getenv("FG_ATTN_KERNEL")) {
+  if (const char* force = fg_options().attn_kernel; force[0] != 0) {
     if (force[0] != 'd') return false;
   }
   int splits = 1, tps = 4;
@@ -834,10 +834,7 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
   d->splits = splits;
   d->tiles_per_split = tps;
   d->min_tiles = 16;
-  if (const char* e = getenv("FG_DECODE_MIN_TILES")) {
-    const int v = atoi(e);
-    if (v >= 4 && v % 4 == 0) d->min_tiles = v;
-  }
+  if (fg_options().decode_min_tiles > 0) d->min_tiles = fg_options().decode_min_tiles;
   d->part_o = splits > 1 ? (float*)p.workspace : nullptr;
   d->part_ml = splits > 1 ? (float*)p.workspace + (size_t)splits * p.batch * p.Hq * p.D : nullptr;
   return true;
@@ -848,7 +845,7 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
 // such sequences pays two launches of workgroups that leave at once.
 bool mixed_batch(const FgFlashParams& p) {
   if (p.max_seqlen_q <= 1 || p.batch < 4) return false;
-  if (const char* e = getenv("FG_ATTN_MIXED")) return e[0] != '0';
+  if (fg_options().attn_mixed >= 0) return fg_options().attn_mixed != 0;
   return true;
 }
 // Head-pair kernel: applicable?  If so, its block shape and the size of its flag array.
@@ -862,8 +859,7 @@ bool pair_plan(const FgFlashParams& p, int* hpb, int* rows, size_t* flag_bytes) 
       p.alibi_slopes != nullptr || p.softcap > 0.f)
     return false;
   // Measured on MI355X the lean kernel is still ahead (see the header of attn_pair.h): opt-in for now.
-  const char* force = getenv("FG_ATTN_KERNEL");
-  if (force == nullptr || force[0] != 'p') return false;
+  if (fg_options().attn_kernel[0] != 'p') return false;
   *hpb = ratio % 4 == 0 ? 4 : 2;
   *rows = (8 / *hpb) * 32;
   *flag_bytes = (size_t)fg_cdiv(p.max_seqlen_q, *rows) * (size_t)p.batch * (size_t)(p.Hq / *hpb) * sizeof(int);
@@ -948,7 +944,7 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.redo_flags = nullptr;
   a.redo_rows = 0;
   a.redo_grid_x = 0;
-  if (const char* force = getenv("FG_ATTN_KERNEL")) {
+  if (const char* force = fg_options().attn_kernel; force[0] != 0) {
     a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p');
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && (p.D == 64 || p.D == 96 || p.D == 128)) {

@@ -20,6 +20,23 @@ int fg_check_launch(const char* what);
     }                               \
   } while (0)
 
+// Measurement and test switches, read from the environment once (first use) and again only when
+// fg_reload_options() is called; no entry point calls getenv().
+struct FgOptions {
+  bool gemm_no_dma;       // FG_GEMM_NO_DMA: keep 16-bit GEMMs off the direct-to-LDS kernels
+  bool gemm_sk_even;      // FG_GEMM_SK_EVEN: stream-K always in equal shares
+  int gemm_tile_bm, gemm_tile_bn;  // FG_GEMM_TILE=256x128[s]: forced direct-to-LDS tile (bm == 0: not forced)
+  bool gemm_tile_deep;    // ... false with the "s" suffix (two LDS stages)
+  bool skinny_no_lds;     // FG_SKINNY_NO_LDS
+  bool skinny_rows64;     // FG_SKINNY_ROWS64
+  int skinny_tile;        // FG_SKINNY_TILE=16|32 (0: not set)
+  char attn_kernel[8];    // FG_ATTN_KERNEL ("" when not set)
+  int attn_mixed;         // FG_ATTN_MIXED: 0 / 1 (-1: not set)
+  int decode_min_tiles;   // FG_DECODE_MIN_TILES (0: not set)
+  int decode_wg_per_cu;   // FG_DECODE_WG_PER_CU (0: not set)
+};
+const FgOptions& fg_options();
+
 static inline bool fg_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 static inline int64_t fg_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -1,5 +1,4 @@
 // Host side of fg_gemm: validation, load-mode and tile selection, schedule selection, launches.
-#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 #include "gemm_tile.h"
@@ -117,7 +116,7 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
   if constexpr (sizeof(T) == 2) {
     // Aligned operands with K a multiple of 64 take the direct-to-LDS kernel, on the tile size that fills
     // the machine best (even a lone 128x128 workgroup per CU runs twice as fast as the register-staged kernel).
-    if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && getenv("FG_GEMM_NO_DMA") == nullptr) {
+    if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && !fg_options().gemm_no_dma) {
       int bm = 256, bn = 256;
       bool deep = false;
       dma_pick_tile(g.M, g.N, g.K, num_cu, &bm, &bn, &deep);
@@ -169,6 +168,27 @@ extern "C" size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int a
   size_t a = skinny_workspace_bytes(M, N, K, cu);
   size_t b = streamk_workspace_bytes(M, N, K, ab_dtype, cu);
   return a > b ? a : b;
+}
+
+extern "C" int fg_gemm_workspace_layout(int device, size_t* max_bytes, size_t* header_bytes) {
+  // the largest request of either stream-K family: header + two fp32 128x128 partial tiles per CU
+  const int cu = num_cus(device);
+  if (max_bytes) *max_bytes = kPartialOffset + (size_t)(cu < kMaxWorkers ? cu : kMaxWorkers) * 2 * 128 * 128 * sizeof(float);
+  if (header_bytes) *header_bytes = kPartialOffset;
+  return FG_OK;
+}
+
+extern "C" int fg_stream_capture_id(void* stream, unsigned long long* id) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long cid = 0;
+  const hipError_t e = hipStreamGetCaptureInfo((hipStream_t)stream, &status, &cid);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    fg_set_error("stream_capture_id: %s", hipGetErrorString(e));
+    return FG_ERR_INVALID;
+  }
+  if (id) *id = status == hipStreamCaptureStatusActive ? (cid != 0 ? cid : ~0ull) : 0;
+  return FG_OK;
 }
 
 extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
@@ -226,7 +246,7 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
           // sharing up to half a wave of tiles; for the direct-to-LDS one the two duration models decide.
           const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
           const int64_t iters = fg_cdiv(K, 64);
-          const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && getenv("FG_GEMM_NO_DMA") == nullptr;
+          const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && !fg_options().gemm_no_dma;
           if (dma) {
             int bm, bn, workers;
             bool deep;
@@ -251,7 +271,7 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
   }
   if (use_streamk) {
     if (schedule_used) *schedule_used = FG_SCHED_STREAM_K;
-    if (amode != LOAD_GEN && dma_supported(g, eb) && getenv("FG_GEMM_NO_DMA") == nullptr)
+    if (amode != LOAD_GEN && dma_supported(g, eb) && !fg_options().gemm_no_dma)
       return dma_streamk_launch(g, ab_dtype, workspace, workspace_bytes, cu, st);
     return streamk_launch(g, ab_dtype, amode, bmode, workspace, workspace_bytes, cu, st);
   }

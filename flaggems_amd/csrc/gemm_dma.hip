@@ -72,13 +72,10 @@ static bool dma_tile_exists(int bm, int bn) {
 
 // Tile choice: the candidate the model above finishes first.  Returns its estimated duration.
 double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep) {
-  if (const char* e = getenv("FG_GEMM_TILE")) {  // measurement aid: one of the tiles above as "256x128"; "s" appended = two stages
-    int a = 0, b = 0;
-    char c = 0;
-    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && dma_tile_exists(a, b)) {
-      *bm = a; *bn = b; *deep = c != 's';
-      return 0.0;
-    }
+  const FgOptions& opt = fg_options();  // measurement aid: one of the tiles above forced
+  if (opt.gemm_tile_bm > 0 && dma_tile_exists(opt.gemm_tile_bm, opt.gemm_tile_bn)) {
+    *bm = opt.gemm_tile_bm; *bn = opt.gemm_tile_bn; *deep = opt.gemm_tile_deep;
+    return 0.0;
   }
   double best = 0.0;
   bool have = false;
@@ -103,7 +100,7 @@ double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, in
   const bool aligned = total % w == 0 && ((total / w) % iters_per_tile == 0 || iters_per_tile % (total / w) == 0);
   double best = aligned ? 20.0 + 0.42 * (double)(total / w) : 27.0 + 0.6 * (double)fg_cdiv(total, w);
   *workers = (int)w;
-  if (getenv("FG_GEMM_SK_EVEN") != nullptr) return best;  // measurement and test aid: always equal shares
+  if (fg_options().gemm_sk_even) return best;  // measurement and test aid: always equal shares
   for (int64_t s = 1; s <= iters_per_tile && sk_tiles * s <= num_cu; ++s) {
     if (iters_per_tile % s != 0) continue;
     const double c = (s == 1 ? 10.0 : 20.0) + 0.42 * (double)(iters_per_tile / s);

@@ -552,9 +552,9 @@ int skinny_supported(const GemmArgs& g, int dtype, int amode, int bmode) {
   // kernels cannot fill the machine (narrow outputs) and, up to 32 rows, for outputs of moderate width; measured
   // against those kernels on 4096..32000 columns with K = 4096..14336.
   if (g.M > 16) {
-    if (bmode != LOAD_K || g.K % kcStepK != 0 || getenv("FG_SKINNY_NO_LDS") != nullptr) return 0;
+    if (bmode != LOAD_K || g.K % kcStepK != 0 || fg_options().skinny_no_lds) return 0;
     const bool pays = g.N <= 8192 || (g.M <= 32 && g.N <= 24576);
-    return pays || getenv("FG_SKINNY_ROWS64") != nullptr ? 2 : 0;
+    return pays || fg_options().skinny_rows64 ? 2 : 0;
   }
   if (bmode == LOAD_K) return 2;
   if (bmode == LOAD_MN) return 1;
@@ -574,10 +574,10 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
   SkinnyArgs a;
   a.g = g;
   // K-contiguous B with K a multiple of 64: the kernel that stages B through LDS, on 16-column tiles
-  const bool kc = b_kind == 2 && g.K % kcStepK == 0 && getenv("FG_SKINNY_NO_LDS") == nullptr;
+  const bool kc = b_kind == 2 && g.K % kcStepK == 0 && !fg_options().skinny_no_lds;
   // 32-column tiles once they still give every CU a tile of its own (measurement aid: FG_SKINNY_TILE=16|32)
   int kc_tile = g.N >= 32 * (int64_t)num_cu ? 32 : 16;
-  if (const char* e = getenv("FG_SKINNY_TILE")) kc_tile = atoi(e) == 32 ? 32 : atoi(e) == 16 ? 16 : kc_tile;
+  if (fg_options().skinny_tile != 0) kc_tile = fg_options().skinny_tile;
   if (g.M > 32) kc_tile = 32;
   a.tiles_n = (int)fg_cdiv(g.N, kc ? kc_tile : kTileN);
   a.ksteps = (int)fg_cdiv(g.K, kc ? kcStepK : kStepK);

@@ -22,20 +22,40 @@ def get_higher_dtype(a, b):
             return a
 
 
-# One scratch buffer per (device, stream): stream-K partial tiles and their flags.  The reference
-# allocates these per call (src/flag_gems/ops/mm_streamk.py:488-491); launches on one stream are
-# ordered, so a buffer per stream can be reused without a hazard.
+# One scratch buffer per (device, stream): stream-K partial tiles behind a header of ticket counters.  The
+# reference allocates these per call (src/flag_gems/ops/mm_streamk.py:488-491); launches on one stream are
+# ordered, so a buffer per stream is reused without a hazard.  The buffer has the largest size any problem can
+# ask for on the device and is never replaced: a HIP graph that recorded its address stays valid whatever runs
+# later.  Only the header has to read zero when a launch starts, and the kernels return it to zero.  It is
+# cleared when the buffer is made and, once per graph capture that uses the buffer, by a fill kernel recorded
+# into that graph, so that every replay starts from a cleared header whichever graph of the stream ran (or was
+# only recorded) before it.
 _workspaces = {}
+_layouts = {}
+_capture_id = ctypes.c_ulonglong(0)
 
 
-def _workspace(device, stream, nbytes):
+def _workspace(device, stream):
+    lib = _C.lib()
     key = (device.index, stream)
-    buf = _workspaces.get(key)
-    if buf is None or buf.numel() < nbytes:
-        # zero-filled once: the kernels return their ticket counters to zero after every launch
-        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = buf
-    return buf
+    entry = _workspaces.get(key)
+    _C.check(lib.fg_stream_capture_id(stream, ctypes.byref(_capture_id)), "fg_stream_capture_id")
+    capture = _capture_id.value
+    if entry is None:
+        layout = _layouts.get(device.index)
+        if layout is None:
+            total, header = ctypes.c_size_t(0), ctypes.c_size_t(0)
+            _C.check(lib.fg_gemm_workspace_layout(device.index, ctypes.byref(total), ctypes.byref(header)),
+                     "fg_gemm_workspace_layout")
+            layout = _layouts[device.index] = (total.value, header.value)
+        buf = torch.empty(layout[0], dtype=torch.uint8, device=device)
+        buf[:layout[1]].zero_()
+        entry = _workspaces[key] = [buf, capture, layout[1]]
+    elif capture != entry[1]:
+        if capture != 0:
+            entry[0][:entry[2]].zero_()
+        entry[1] = capture
+    return entry[0]
 
 
 _last_schedule = ctypes.c_int(0)
@@ -56,7 +76,7 @@ def gemm(a, b, bias, c, alpha=1.0, beta=0.0, schedule=_C.SCHED_AUTO):
         stream = _C.current_stream(dev)
         ab = _C.dtype_id(a.dtype)
         ws_bytes = lib.fg_gemm_workspace_bytes(M, N, K, ab, schedule, dev.index)
-        ws = _workspace(dev, stream, ws_bytes) if ws_bytes else None
+        ws = _workspace(dev, stream) if ws_bytes else None
         if bias is not None:
             bptr, sim, sin_, bdt = bias.data_ptr(), bias.stride(0), bias.stride(1), _C.dtype_id(bias.dtype)
         else:

@@ -41,6 +41,10 @@ const char* fg_last_error(void);
 /* ABI version of this header (bumped on any signature change). */
 int fg_abi_version(void);
 
+/* Re-reads the FG_* measurement and test switches from the environment.  The library reads them once, on first
+ * use; no entry point consults the environment per call.  No counterpart in the reference. */
+void fg_reload_options(void);
+
 /* Device facts the host-side heuristics use (CU count stands in for the reference's
  * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530). */
 int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
@@ -163,6 +167,18 @@ enum { FG_SCHED_AUTO = 0, FG_SCHED_DATA_PARALLEL = 1, FG_SCHED_STREAM_K = 2 };
  * Stands in for the per-call `locks`/`P` allocation of src/flag_gems/ops/mm_streamk.py:488-491. */
 size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, int schedule,
                                int device);
+
+/* The largest value fg_gemm_workspace_bytes can return on `device` (a function of its CU count only), and the
+ * size of the buffer's header: the part that must read zero when a launch starts (the ticket counters, which
+ * the kernels return to zero).  A caller that sizes one buffer per stream to *max_bytes never has to replace
+ * it, so pointers recorded in HIP graphs stay valid.  Stands in for the per-call allocation of
+ * src/flag_gems/ops/mm_streamk.py:488-491. */
+int fg_gemm_workspace_layout(int device, size_t* max_bytes /*host*/, size_t* header_bytes /*host*/);
+
+/* *id = 0 when `stream` is not capturing into a HIP graph, otherwise a non-zero number unique to the capture in
+ * progress.  Host code uses it to record one clearing of the workspace header per captured graph.  No counterpart
+ * in the reference (its Triton launches allocate and clear per call). */
+int fg_stream_capture_id(void* stream, unsigned long long* id /*host*/);
 
 /* C[M,N] = alpha * (A[M,K] . B[K,N]) + beta * bias (bias == NULL: C = A.B), fp32 accumulate.
  * A, B, C and bias are addressed through (row, col) element strides; bias strides may be 0

@@ -286,3 +286,49 @@ def gems_tolerance(dtype, reduce_dim=1, atol=1e-4):
     """(atol, rtol) of src/flag_gems/testing/__init__.py:41-49."""
     rtol = {torch.float16: 1e-3, torch.bfloat16: 0.016, torch.float32: 1.3e-6, torch.float64: 1e-7}[dtype]
     return atol * reduce_dim, rtol
+
+
+def decoder_layer(h, wqkv, wo, wgu, wd, n1, n2, positions, cos, sin, eps, heads, q_rows=None):
+    """One Llama-style decoder layer over ONE causal sequence, evaluated on the host in fp32 from the operator
+    oracles above, with every operator's result rounded to the input dtype where the device path stores a
+    tensor (so that a comparison sees one rounding per operator, not an accumulation of them):
+    rms_norm -> x.Wqkv^T -> rotary (neox) on q, k -> causal attention over the sequence's own keys ->
+    .Wo^T -> fused_add_rms_norm with the layer input as residual -> .Wgu^T -> silu_and_mul -> .Wd^T -> + residual.
+    The chain is the layer the benchmark configuration runs (hidden = heads * head_dim, MHA); it follows the
+    reference's module layer, src/flag_gems/modules/{normalization,rotary_embedding,activation}.py, and the
+    operator tests cited above for each step.  `q_rows` (a LongTensor of token indices) restricts everything
+    behind the key/value projection to those query tokens; keys and values are always computed for the whole
+    sequence.  Returns a dict of the intermediate tensors (fp32), restricted to q_rows where that applies."""
+    dt = h.dtype
+    rnd = lambda t: t.to(dt).float()
+    h = to_reference(h)
+    S, hidden = h.shape
+    D = hidden // heads
+    wqkv, wo, wgu, wd = (to_reference(w).float() for w in (wqkv, wo, wgu, wd))
+    n1, n2 = to_reference(n1), to_reference(n2)
+    cos, sin, positions = to_reference(cos), to_reference(sin), to_reference(positions)
+    rows = torch.arange(S) if q_rows is None else to_reference(q_rows).long()
+    x = rms_norm(h, n1, eps).float()                                   # [S, hidden], rounded by the oracle itself
+    kv = rnd(x @ wqkv[hidden:].t())                                    # keys and values of every token
+    k = kv[:, :hidden].view(S, heads, D)
+    v = kv[:, hidden:].view(S, heads, D)
+    q = rnd(x[rows] @ wqkv[:hidden].t()).view(len(rows), heads, D)
+    q, _ = apply_rotary_pos_emb(q, q, cos, sin, positions[rows], False)
+    k, _ = apply_rotary_pos_emb(k, k, cos, sin, positions, False)
+    q, k = rnd(q), rnd(k)
+    scale = D ** -0.5
+    att = torch.empty(len(rows), heads, D)
+    for i, r in enumerate(rows.tolist()):                              # causal: token r sees keys 0..r
+        s = torch.einsum("hd,khd->hk", q[i] * scale, k[: r + 1])
+        p = torch.softmax(s, dim=-1)
+        att[i] = torch.einsum("hk,khd->hd", p, v[: r + 1])
+    att = rnd(att)
+    o = rnd(att.reshape(len(rows), hidden) @ wo.t())
+    y, resid = fused_add_rms_norm(o, h[rows].float(), n2.float(), eps)
+    y, resid = rnd(y), rnd(resid)
+    gu = rnd(y @ wgu.t())
+    F_ = wgu.shape[0] // 2
+    act = rnd(silu_and_mul(gu[:, :F_], gu[:, F_:]))
+    out = rnd(rnd(act @ wd.t()) + resid)
+    return {"x": x, "k": k, "v": v, "q": q, "attn": att, "o": o, "y": y, "residual": resid, "gate_up": gu,
+            "act": act, "out": out}

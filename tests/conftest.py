@@ -22,3 +22,41 @@ def gpu():
 
     _C.lib()  # raises if libfg_mi355.so is not built
     return torch.device("cuda:0")
+
+
+class _FgEnv:
+    """Sets or removes FG_* switches and has the library read them again (it reads the environment
+    once, not per call)."""
+
+    def __init__(self):
+        self._saved = {}
+
+    def _reload(self):
+        from flaggems_amd import _C
+
+        _C.lib().fg_reload_options()
+
+    def setenv(self, name, value):
+        self._saved.setdefault(name, os.environ.get(name))
+        os.environ[name] = value
+        self._reload()
+
+    def delenv(self, name, raising=False):
+        self._saved.setdefault(name, os.environ.get(name))
+        os.environ.pop(name, None)
+        self._reload()
+
+    def restore(self):
+        for name, old in self._saved.items():
+            if old is None:
+                os.environ.pop(name, None)
+            else:
+                os.environ[name] = old
+        self._reload()
+
+
+@pytest.fixture
+def fg_env():
+    env = _FgEnv()
+    yield env
+    env.restore()

@@ -92,11 +92,11 @@ def test_flash_attn_varlen_edges(gpu):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hk,D,block_size", [(32, 8, 128, 16), (8, 8, 64, 32), (12, 4, 128, 64)])
 @pytest.mark.parametrize("mixed_env", [None, "0"])
-def test_flash_attn_mixed_batches(gpu, monkeypatch, dtype, Hq, Hk, D, block_size, mixed_env):
+def test_flash_attn_mixed_batches(gpu, fg_env, dtype, Hq, Hk, D, block_size, mixed_env):
     if mixed_env is None:
-        monkeypatch.delenv("FG_ATTN_MIXED", raising=False)
+        fg_env.delenv("FG_ATTN_MIXED", raising=False)
     else:
-        monkeypatch.setenv("FG_ATTN_MIXED", mixed_env)
+        fg_env.setenv("FG_ATTN_MIXED", mixed_env)
     check(gpu, [(1, 700), (1, 33), (300, 300), (1, 4096), (64, 1000), (1, 1), (1, 2500), (17, 17)], Hq, Hk, D, block_size,
           2048, dtype)
     check(gpu, [(128, 128), (5, 900), (200, 1200), (33, 64)], Hq, Hk, D, block_size, 1024, dtype)
@@ -112,8 +112,8 @@ def test_flash_attn_mixed_batches(gpu, monkeypatch, dtype, Hq, Hk, D, block_size
 # lean kernel by the second pass.
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hk", [(8, 2), (4, 2), (6, 3)])
-def test_flash_attn_head_pair_kernel(gpu, monkeypatch, dtype, Hq, Hk):
-    monkeypatch.setenv("FG_ATTN_KERNEL", "pair")
+def test_flash_attn_head_pair_kernel(gpu, fg_env, dtype, Hq, Hk):
+    fg_env.setenv("FG_ATTN_KERNEL", "pair")
     check(gpu, [(1, 1328), (5, 18), (129, 463), (70, 70)], Hq, Hk, 128, 16, 512, dtype)
     check(gpu, [(200, 200), (64, 64), (65, 65), (300, 1000)], Hq, Hk, 128, 32, 1024, dtype)
     check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=False)
@@ -124,8 +124,8 @@ def test_flash_attn_head_pair_kernel(gpu, monkeypatch, dtype, Hq, Hk):
 
 
 @pytest.mark.parametrize("dtype,grow", [(torch.bfloat16, 0.02), (torch.float16, 0.004), (torch.bfloat16, 0.05)])
-def test_flash_attn_head_pair_second_pass(gpu, monkeypatch, dtype, grow):
-    monkeypatch.setenv("FG_ATTN_KERNEL", "pair")
+def test_flash_attn_head_pair_second_pass(gpu, fg_env, dtype, grow):
+    fg_env.setenv("FG_ATTN_KERNEL", "pair")
     dev, Hq, Hk, D, bs, nblk = gpu, 8, 2, 128, 16, 512
     qlens, klens = [300, 64], [300, 700]
     torch.manual_seed(5)
@@ -188,9 +188,9 @@ def test_flash_attn_decode_variants(gpu):
 # and the merge must read exactly the ranges that sequence wrote.
 @pytest.mark.parametrize("max_k", [4096, 32768, 131072])
 @pytest.mark.parametrize("min_tiles", [None, "4", "64"])
-def test_flash_attn_decode_max_seqlen_k_above_lengths(gpu, monkeypatch, max_k, min_tiles):
+def test_flash_attn_decode_max_seqlen_k_above_lengths(gpu, fg_env, max_k, min_tiles):
     if min_tiles is not None:
-        monkeypatch.setenv("FG_DECODE_MIN_TILES", min_tiles)
+        fg_env.setenv("FG_DECODE_MIN_TILES", min_tiles)
     lens = [(1, n) for n in (2048, 1, 0, 31, 129, 511, 513, 2047, 2049, 3000, 4096, 640)] + [(1, 700 + 61 * i) for i in range(24)]
     q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, lens, 32, 8, 128, 16, 1024, torch.bfloat16)
     wide = torch.zeros(bt.shape[0], max_k // 16, dtype=bt.dtype, device=bt.device)

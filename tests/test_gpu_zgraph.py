@@ -78,3 +78,93 @@ def test_decode_step_in_hip_graph(gpu):
         assert torch.equal(got, want), f"replay {step} differs from the eager step"
         assert torch.equal(got_r, want_r)
         assert torch.equal(kc_after, kc) and torch.equal(vc_after, vc)
+
+
+def _fresh_stream(gpu):
+    """A side stream that has no GEMM workspace yet (torch hands streams out of a small pool)."""
+    from flaggems_amd.ops import _gemm
+
+    for _ in range(64):
+        s = torch.cuda.Stream()
+        if (gpu.index, s.cuda_stream) not in _gemm._workspaces:
+            return s
+    raise AssertionError("no unused stream left in torch's pool")
+
+
+def _streamk_mm(a, b):
+    from flaggems_amd import _C
+    from flaggems_amd.ops import _gemm
+
+    out = torch.empty(a.shape[0], b.shape[1], dtype=a.dtype, device=a.device)
+    _gemm.gemm(a, b, None, out, schedule=_C.SCHED_STREAM_K)
+    assert _gemm.last_schedule() == 2
+    return out
+
+
+def _sk_inputs(gpu, M, N, K, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    a = (torch.randn(M, K, generator=g) / 8).to(torch.bfloat16).to(gpu)
+    w = (torch.randn(N, K, generator=g) / 8).to(torch.bfloat16).to(gpu)
+    return a, w
+
+
+def test_workspace_survives_a_larger_eager_gemm_after_capture(gpu):
+    """A captured decode GEMM (skinny stream-K, small share of the workspace), then an eager stream-K tile GEMM on
+    the same stream that needs far more of it, then replays: the graph's recorded workspace address must still be
+    the live buffer, so the replays equal the eager results."""
+    from flaggems_amd.ops import _gemm
+
+    a, w = _sk_inputs(gpu, 8, 512, 4096, 1)
+    big_a, big_w = _sk_inputs(gpu, 384, 4096, 4096, 2)
+    want = _streamk_mm(a, w.t())
+    side = _fresh_stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        got = _streamk_mm(a, w.t())
+    key = (gpu.index, side.cuda_stream)
+    buf = _gemm._workspaces[key][0]
+    with torch.cuda.stream(side):
+        big = _streamk_mm(big_a, big_w.t())  # eager, same stream: 128x128 stream-K tiles
+    torch.cuda.synchronize()
+    assert _gemm._workspaces[key][0] is buf and buf.data_ptr() == _gemm._workspaces[key][0].data_ptr()
+    for _ in range(3):
+        got.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        with torch.cuda.stream(side):
+            again = _streamk_mm(big_a, big_w.t())
+        torch.cuda.synchronize()
+        assert torch.equal(again, big)
+    from oracle import torch_ref as O
+    from helpers import gems_assert_close
+    gems_assert_close(big[:16], O.mm(big_a[:16], big_w.t()), torch.bfloat16, reduce_dim=4096)
+
+
+def test_two_graphs_on_one_stream_replayed_out_of_order(gpu):
+    """The workspace of a stream is first made during a capture (its clearing is only recorded there); a second
+    graph captured on the same stream is replayed BEFORE the first ever ran.  Each graph clears the ticket header
+    itself, so both produce the eager result in either order."""
+    from flaggems_amd.ops import _gemm
+
+    a1, w1 = _sk_inputs(gpu, 16, 1024, 4096, 3)
+    a2, w2 = _sk_inputs(gpu, 4, 768, 8192, 4)
+    want1 = _streamk_mm(a1, w1.t())
+    want2 = _streamk_mm(a2, w2.t())
+    torch.cuda.synchronize()
+    side = _fresh_stream(gpu)
+    g1, g2 = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1, stream=side):
+        got1 = _streamk_mm(a1, w1.t())
+    with torch.cuda.graph(g2, stream=side):
+        got2 = _streamk_mm(a2, w2.t())
+    # poison the header the way stale memory would: a replay that did not clear it would mis-count its tickets
+    entry = _gemm._workspaces[(gpu.index, side.cuda_stream)]
+    entry[0][:entry[2]].fill_(0xFF)
+    torch.cuda.synchronize()
+    for order in ((g2, g1), (g1, g2), (g2, g2, g1)):
+        got1.zero_(); got2.zero_()
+        for g in order:
+            g.replay()
+            torch.cuda.synchronize()
+        assert torch.equal(got1, want1) and torch.equal(got2, want2)

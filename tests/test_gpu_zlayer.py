@@ -1,0 +1,101 @@
+"""The Llama-2-7B-shaped decoder layer of the benchmark configuration at its full size (8 sequences x 2048
+tokens, hidden 4096, 32 heads x 128, FFN 11008, paged KV with page 16) under flag_gems.enable() semantics.
+Every operator boundary is checked on sampled tokens against the CPU oracle fed with the device path's own
+inputs to that operator (the reference's per-operator tolerance rule), the cache scatter bit-exactly over all
+tokens, and the layer output end to end for sampled tokens of one sequence against the fp32 layer oracle."""
+import pytest
+import torch
+
+import flag_gems
+from helpers import gems_assert_close
+from oracle import torch_ref as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_decoder_layer_full_size(gpu):
+    torch.manual_seed(0)
+    Hd, H, D, F, bs, B, S = 4096, 32, 128, 11008, 16, 8, 2048
+    T = B * S
+    bf16 = torch.bfloat16
+    wqkv = (torch.randn(3 * Hd, Hd) * 0.02).to(bf16).to(gpu)
+    wo = (torch.randn(Hd, Hd) * 0.02).to(bf16).to(gpu)
+    wgu = (torch.randn(2 * F, Hd) * 0.02).to(bf16).to(gpu)
+    wd = (torch.randn(Hd, F) * 0.02).to(bf16).to(gpu)
+    n1 = (torch.rand(Hd) + 0.5).to(bf16).to(gpu)
+    n2 = (torch.rand(Hd) + 0.5).to(bf16).to(gpu)
+    h = torch.randn(T, Hd).to(bf16).to(gpu)
+    pos = torch.arange(S).repeat(B).to(gpu)
+    cos, sin = O.rope_cos_sin(S, D, device=gpu)
+    nblk = T // bs
+    bt = torch.randperm(nblk).view(B, S // bs).int().to(gpu)
+    t = torch.arange(S, device=gpu)
+    slots = torch.cat([bt[i][t // bs].long() * bs + t % bs for i in range(B)])
+    kc = torch.zeros(nblk, bs, H, D, dtype=bf16, device=gpu)
+    vc = torch.zeros_like(kc)
+    cu = torch.arange(0, T + 1, S, dtype=torch.int32, device=gpu)
+    sk = torch.full((B,), S, dtype=torch.int32, device=gpu)
+    with flag_gems.use_gems():
+        x = torch.nn.functional.rms_norm(h, [Hd], n1, 1e-5)
+        qkv = torch.mm(x, wqkv.t())
+        qkv_pre = qkv.clone()
+        q, k, v = (qkv[:, i * Hd:(i + 1) * Hd].view(T, H, D) for i in range(3))
+        flag_gems.apply_rotary_pos_emb(q, k, cos, sin, pos, False, inplace=True)
+        flag_gems.reshape_and_cache_flash(k, v, kc, vc, slots, "auto", None, None)
+        attn = flag_gems.flash_attn_varlen_func(q, kc, vc, S, cu, S, seqused_k=sk, causal=True, block_table=bt)
+        o = torch.mm(attn.view(T, Hd), wo.t())
+        o_pre = o.clone()
+        y, resid = flag_gems.fused_add_rms_norm(o, h.clone(), [Hd], n2, 1e-5)
+        gu = torch.mm(y, wgu.t())
+        act = flag_gems.silu_and_mul(gu[:, :F], gu[:, F:])
+        down = torch.mm(act, wd.t())
+        out = down + resid
+    torch.cuda.synchronize()
+
+    g = torch.Generator().manual_seed(1)
+    rows = torch.cat([torch.tensor([0, 1, S - 1, S, T - 1]), torch.randint(0, T, (11,), generator=g)]).to(gpu)
+    # rms_norm, the four projections, silu_and_mul, fused_add_rms_norm: sampled token rows, oracle on the device
+    # path's own operands
+    gems_assert_close(x[rows], O.rms_norm(h[rows], n1, 1e-5), bf16)
+    gems_assert_close(qkv_pre[rows], O.mm(x[rows], wqkv.t()), bf16, reduce_dim=Hd)
+    gems_assert_close(o_pre[rows], O.mm(attn.view(T, Hd)[rows], wo.t()), bf16, reduce_dim=Hd)
+    ry, rr = O.fused_add_rms_norm(o_pre[rows], h[rows], n2, 1e-5)
+    gems_assert_close(y[rows], ry, bf16)
+    gems_assert_close(resid[rows], rr, bf16)
+    gems_assert_close(gu[rows], O.mm(y[rows], wgu.t()), bf16, reduce_dim=Hd)
+    gems_assert_close(act[rows], O.silu_and_mul(gu[rows, :F], gu[rows, F:]), bf16)
+    gems_assert_close(down[rows], O.mm(act[rows], wd.t()), bf16, reduce_dim=F)
+    cols = torch.tensor([0, 255, 256, 4095, 4096, 8191, 8192, 12287], device=gpu)  # whole columns of the widest GEMM
+    gems_assert_close(qkv_pre[:, cols], O.mm(x, wqkv.t()[:, cols]), bf16, reduce_dim=Hd)
+    # rotary embedding: q and k of the sampled tokens, from the values the GEMM left
+    qp, kp = (qkv_pre[:, i * Hd:(i + 1) * Hd].view(T, H, D)[rows] for i in range(2))
+    rq, rk = O.apply_rotary_pos_emb(qp, kp, cos, sin, pos[rows], False)
+    gems_assert_close(q[rows], rq, bf16)
+    gems_assert_close(k[rows], rk, bf16)
+    assert torch.equal(v, qkv_pre[:, 2 * Hd:].view(T, H, D))  # values are not rotated
+    # cache scatter: every token row sits, bit for bit, in the slot the mapping names (gather on the device with
+    # torch indexing), and the oracle scatter agrees on two whole sequences' pages
+    assert torch.equal(kc.view(-1, H, D)[slots], k) and torch.equal(vc.view(-1, H, D)[slots], v)
+    for b in (0, B - 1):
+        pages = bt[b].long().cpu()
+        ek = torch.zeros(nblk, bs, H, D, dtype=bf16); ev = torch.zeros_like(ek)
+        sl = slice(b * S, (b + 1) * S)
+        ek, ev = O.reshape_and_cache_flash(k[sl], v[sl], ek, ev, slots[sl])
+        assert torch.equal(kc[pages.to(gpu)].cpu(), ek[pages]) and torch.equal(vc[pages.to(gpu)].cpu(), ev[pages])
+    # attention: query tokens of three sequences against the paged-attention oracle over the device's own cache
+    kc_h, vc_h = kc.cpu(), vc.cpu()
+    for b, lo, hi in ((0, 0, 5), (3, 1021, 1029), (B - 1, S - 6, S)):
+        qs = q[b * S + lo:b * S + hi]
+        ref = O.paged_attention(qs, kc_h, vc_h, [hi - lo], [hi], bt[b:b + 1], D ** -0.5, compute_dtype=torch.float32)
+        torch.testing.assert_close(attn[b * S + lo:b * S + hi].float().cpu(), ref, atol=2e-2, rtol=1e-2)
+    # end to end: sampled tokens of one sequence through the fp32 layer oracle
+    b = 5
+    sl = slice(b * S, (b + 1) * S)
+    q_rows = torch.tensor([0, 1, 15, 16, 777, 1024, S - 2, S - 1])
+    ref = O.decoder_layer(h[sl], wqkv, wo, wgu, wd, n1, n2, pos[sl], cos, sin, 1e-5, H, q_rows=q_rows)
+    idx = (b * S + q_rows).to(gpu)
+    torch.testing.assert_close(out[idx].float().cpu(), ref["out"], atol=5e-2, rtol=5e-2)
+    torch.testing.assert_close(attn[idx].float().cpu(), ref["attn"], atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(k[sl].float().cpu(), ref["k"], atol=3e-2, rtol=2e-2)
+    err = (out[idx].float().cpu() - ref["out"]).abs().max().item()
+    print(f"decoder layer, 8 x 2048 tokens: end-to-end max |err| on sampled tokens = {err:.4f}")

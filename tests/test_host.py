@@ -211,3 +211,44 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(base, f)).read()
                 assert "oracle" not in text.replace("the oracle", ""), f"{f} mentions the oracle package"
+
+
+def test_custom_op_namespace_schemas():
+    """torch.ops.flag_gems.* carries the reference's schemas for the operators of this path
+    (src/flag_gems/csrc/cstub.cpp:26-90), each with a kernel on the CUDA key."""
+    from flaggems_amd import custom_ops
+
+    want = {
+        "mm", "addmm", "bmm", "softmax", "softmax_backward", "rms_norm", "fused_add_rms_norm",
+        "rotary_embedding", "rotary_embedding_inplace", "reshape_and_cache_flash", "flash_attn_varlen_func",
+    }
+    assert set(custom_ops.op_names()) == want
+    for name in want:
+        op = getattr(torch.ops.flag_gems, name).default
+        assert "custom_ops.py" in _cuda_kernel_of("flag_gems::" + name), name
+        assert op._schema.name == "flag_gems::" + name
+    s = torch.ops.flag_gems.fused_add_rms_norm.default._schema
+    assert [a.name for a in s.arguments] == ["input", "residual", "weight", "epsilon"]
+    assert s.arguments[0].alias_info.is_write and s.arguments[1].alias_info.is_write and len(s.returns) == 0
+    s = torch.ops.flag_gems.rms_norm.default._schema
+    assert [a.name for a in s.arguments] == ["input", "weight", "epsilon"]
+    s = torch.ops.flag_gems.reshape_and_cache_flash.default._schema
+    assert [a.name for a in s.arguments] == [
+        "key", "value", "key_cache", "value_cache", "slot_mapping", "kv_cache_dtype", "k_scale", "v_scale"]
+    assert s.arguments[2].alias_info.is_write and s.arguments[3].alias_info.is_write and len(s.returns) == 0
+    s = torch.ops.flag_gems.flash_attn_varlen_func.default._schema
+    assert [a.name for a in s.arguments] == [
+        "q", "k", "v", "max_seqlen_q", "cu_seqlens_q", "max_seqlen_k", "cu_seqlens_k", "seqused_k", "q_v", "dropout_p",
+        "softmax_scale", "causal", "window_size", "softcap", "alibi_slopes", "deterministic", "return_attn_probs",
+        "block_table", "return_softmax_lse", "out", "scheduler_metadata", "q_descale", "k_descale", "v_descale",
+        "fa_version"]
+    assert len(s.returns) == 2
+    s = torch.ops.flag_gems.addmm.default._schema
+    assert [(a.name, a.kwarg_only) for a in s.arguments] == [
+        ("self", False), ("mat1", False), ("mat2", False), ("beta", True), ("alpha", True)]
+    s = torch.ops.flag_gems.rotary_embedding_inplace.default._schema
+    assert s.arguments[0].alias_info.is_write and s.arguments[1].alias_info.is_write and len(s.returns) == 0
+    assert len(torch.ops.flag_gems.rotary_embedding.default._schema.returns) == 2
+    # a CPU tensor finds no kernel: the namespace is served on the CUDA key only, as in the reference
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.flag_gems.mm(torch.ones(2, 2), torch.ones(2, 2))

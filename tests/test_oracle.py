@@ -481,3 +481,44 @@ def test_streamk_partition_rule_and_abi_agreement():
         pb = (ctypes.c_int64 * workers)(); pe = (ctypes.c_int64 * workers)()
         assert _C.lib().fg_streamk_partition(tiles, iters, workers, ctypes.byref(sk), pb, pe) == 0
         assert sk.value == coop and list(pb) == b.tolist() and list(pe) == e.tolist()
+
+
+def test_decoder_layer_pinned():
+    """The layer oracle against an independent composition of library routines (F.rms_norm,
+    F.scaled_dot_product_attention, F.silu, the textbook rotation written with complex numbers) in fp32, where
+    the oracle's per-operator rounding is the identity; and its q_rows restriction against the full result."""
+    import torch.nn.functional as F
+
+    torch.manual_seed(0)
+    S, heads, D, Fd = 11, 4, 16, 40
+    hid = heads * D
+    h = torch.randn(S, hid)
+    wqkv, wo = torch.randn(3 * hid, hid) / 8, torch.randn(hid, hid) / 8
+    wgu, wd = torch.randn(2 * Fd, hid) / 8, torch.randn(hid, Fd) / 8
+    n1, n2 = torch.rand(hid) + 0.5, torch.rand(hid) + 0.5
+    pos = torch.arange(3, 3 + S)
+    cos, sin = O.rope_cos_sin(64, D)
+    got = O.decoder_layer(h, wqkv, wo, wgu, wd, n1, n2, pos, cos, sin, 1e-5, heads)
+
+    def rope(t):  # pairs (i, i + D/2) rotated by pos * base^(-2i/D): complex multiplication
+        ang = pos[:, None].double() * (1.0 / 10000 ** (torch.arange(0, D, 2).double() / D))[None, :]
+        z = torch.complex(t[..., : D // 2].double(), t[..., D // 2:].double()) * torch.polar(torch.ones_like(ang), ang)[:, None, :]
+        return torch.cat([z.real, z.imag], -1).float()
+
+    x = F.rms_norm(h, [hid], n1, 1e-5)
+    qkv = x @ wqkv.t()
+    q, k, v = (qkv[:, i * hid:(i + 1) * hid].view(S, heads, D) for i in range(3))
+    q, k = rope(q), rope(k)
+    att = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                         is_causal=True)[0].transpose(0, 1).reshape(S, hid)
+    r = att @ wo.t() + h
+    y = F.rms_norm(r, [hid], n2, 1e-5)
+    gu = y @ wgu.t()
+    want = (F.silu(gu[:, :Fd]) * gu[:, Fd:]) @ wd.t() + r
+    torch.testing.assert_close(got["out"], want, atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(got["k"], k, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(got["attn"].reshape(S, hid), att, atol=1e-5, rtol=1e-4)
+    rows = torch.tensor([0, 4, 10])
+    part = O.decoder_layer(h, wqkv, wo, wgu, wd, n1, n2, pos, cos, sin, 1e-5, heads, q_rows=rows)
+    for name in ("q", "attn", "o", "y", "residual", "gate_up", "act", "out"):
+        torch.testing.assert_close(part[name], got[name][rows], atol=1e-6, rtol=1e-6)
