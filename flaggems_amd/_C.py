@@ -109,6 +109,11 @@ _SIGNATURES = {
         [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
          c_f32, c_f32, c_int, c_int, c_int, c_int, c_vp, ctypes.c_size_t, ctypes.POINTER(c_int), c_vp],
     ),
+    "fg_gemm_skinny_static": (
+        c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+         c_f32, c_f32, c_int, c_int, c_int, c_vp],
+    ),
     "fg_bmm": (
         c_int,
         [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,

@@ -603,3 +603,99 @@ int skinny_launch(const GemmArgs& g, int dtype, int b_kind, void* workspace, siz
 }
 
 }  // namespace fgk
+
+// ---------------------------------------------------------------------------------------------
+// fg_gemm_skinny_static: the skinny stream-K GEMM for callers that cannot allocate device memory
+// (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  Same kernels
+// as above; the partial tiles and ticket counters live in a file-scope device array instead of a
+// caller-provided workspace.  Every GPU holds its own copy of the array until the process ends;
+// all calls on a GPU share it, so calls that overlap on one GPU (two streams) race.
+// ---------------------------------------------------------------------------------------------
+namespace fgk {
+int pick_mode(const void* base, int64_t rows, int64_t K, int64_t s_row, int64_t s_k, int elem_bytes);  // gemm.hip
+int num_cus(int device);                                                                                // gemm.hip
+}
+
+namespace {
+constexpr int kStaticMaxCu = 256;  // MI355X; a device with more CUs is turned away
+constexpr size_t kStaticScratchBytes = fgk::kPartialOffset + (size_t)kStaticMaxCu * 2 * 16 * 128 * sizeof(float);
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];  // 4 198 656 bytes
+
+namespace {
+__global__ void clear_tickets_kernel(unsigned* tickets, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) tickets[i] = 0u;
+}
+
+// Device address of this GPU's copy of `scratch`, looked up once per device with that device current.
+// In host code the array's name is only a handle for this lookup, never an address to hand to a kernel.
+int static_scratch(unsigned char** out) {
+  static std::mutex mu;
+  static unsigned char* ptr[64] = {nullptr};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64) {
+    fg_set_error("gemm_skinny_static: cannot identify the current device: %s", hipGetErrorString(e));
+    return FG_ERR_INVALID;
+  }
+  std::lock_guard<std::mutex> lk(mu);
+  if (ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      fg_set_error("gemm_skinny_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return FG_ERR_LAUNCH;
+    }
+    ptr[dev] = (unsigned char*)p;
+  }
+  *out = ptr[dev];
+  return FG_OK;
+}
+}  // namespace
+
+extern "C" int fg_gemm_skinny_static(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                                     int64_t K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim,
+                                     int64_t sin_, int64_t scm, int64_t scn, float alpha, float beta, int ab_dtype,
+                                     int c_dtype, int bias_dtype, void* stream) {
+  using namespace fgk;
+  FG_REQUIRE(M >= 0 && N >= 0 && K >= 0, FG_ERR_INVALID, "gemm_skinny_static: negative size");
+  FG_REQUIRE(ab_dtype == FG_F16 || ab_dtype == FG_BF16, FG_ERR_UNSUPPORTED,
+             "gemm_skinny_static: 16-bit inputs only (dtype %d)", ab_dtype);
+  FG_REQUIRE(c_dtype == ab_dtype && (bias == nullptr || bias_dtype == ab_dtype), FG_ERR_UNSUPPORTED,
+             "gemm_skinny_static: output and bias must have the input dtype");
+  if (M == 0 || N == 0) return FG_OK;
+  FG_REQUIRE(M <= 64, FG_ERR_UNSUPPORTED,
+             "gemm_skinny_static: %lld rows exceed the maximum of 64 the static scratch buffer is sized for; use fg_gemm",
+             (long long)M);
+  FG_REQUIRE(A && B && C, FG_ERR_INVALID, "gemm_skinny_static: null pointer");
+  FG_REQUIRE(N < ((int64_t)1 << 31) && K < ((int64_t)1 << 31), FG_ERR_UNSUPPORTED, "gemm_skinny_static: extent exceeds 2^31");
+  GemmArgs g = {};
+  g.A = A; g.B = B; g.bias = bias; g.C = C;
+  g.M = M; g.N = N; g.K = K;
+  g.sam = sam; g.sak = sak; g.sbk = sbk; g.sbn = sbn; g.sim = sim; g.sin = sin_; g.scm = scm; g.scn = scn;
+  g.alpha = alpha; g.beta = beta;
+  const int amode = pick_mode(A, M, K, sam, sak, 2);
+  const int bmode = pick_mode(B, N, K, sbn, sbk, 2);
+  const int kind = skinny_supported(g, ab_dtype, amode, bmode);
+  FG_REQUIRE(kind != 0, FG_ERR_UNSUPPORTED,
+             "gemm_skinny_static: not a problem of the skinny stream-K kernels (K >= 1024, 16-byte aligned A with unit "
+             "K stride, B row-major or K-contiguous; 17..64 rows only with a K-contiguous B); use fg_gemm");
+  const int cu = num_cus(-1);
+  const size_t need = skinny_workspace_bytes(M, N, K, cu);
+  FG_REQUIRE(need <= kStaticScratchBytes, FG_ERR_UNSUPPORTED,
+             "gemm_skinny_static: this device (%d CUs) needs %zu bytes of scratch, the static buffer holds %zu", cu, need,
+             kStaticScratchBytes);
+  unsigned char* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != FG_OK) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  // The array keeps what the last call left.  The ticket counters must read zero when the kernel starts: cleared
+  // by a small kernel (a memset node would not be safe to record into a caller's graph).
+  hipLaunchKernelGGL(clear_tickets_kernel, dim3(kMaxWorkers / 256), dim3(256), 0, st, (unsigned*)(ws + kTicketOffset),
+                     kMaxWorkers);
+  return skinny_launch(g, ab_dtype, kind, ws, kStaticScratchBytes, cu, st);
+}
+

@@ -192,6 +192,19 @@ int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, 
             int c_dtype, int bias_dtype, int schedule, void* workspace, size_t workspace_bytes,
             int* schedule_used, void* stream);
 
+/* fg_gemm for skinny problems WITHOUT a caller-provided workspace and without any device allocation: the
+ * stream-K partial tiles and ticket counters live in a static device array of 4 198 656 bytes inside the library
+ * (one copy per GPU, held until the process ends).  No counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Accepts what the skinny stream-K kernels accept: 16-bit inputs, M <= 64, K >= 1024, A with unit K stride and
+ * 16-byte aligned rows, B row-major (M <= 16) or K-contiguous; anything else returns FG_ERR_UNSUPPORTED with a
+ * message (use fg_gemm).  Results are bit-identical to fg_gemm's stream-K schedule.  All calls on one GPU share
+ * the array: calls that overlap on one GPU (different streams) race; calls on one stream are safe. */
+int fg_gemm_skinny_static(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
+                          int64_t K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim,
+                          int64_t sin_, int64_t scm, int64_t scn, float alpha, float beta, int ab_dtype,
+                          int c_dtype, int bias_dtype, void* stream);
+
 /* C[b] = A[b] . B[b] for b in [0, batch), fp32 accumulate, every operand addressed through
  * (matrix, row, col) element strides (a matrix stride of 0 broadcasts one operand).  Matrix b is
  * one data-parallel fg_gemm launch; the launches follow each other on the stream.
