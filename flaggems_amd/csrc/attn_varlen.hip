@@ -69,6 +69,7 @@ struct AttnArgs {
   int redo_rows;      // lean kernel as the second pass: query rows per flagged block (0: ordinary launch)
   int redo_grid_x;    // ... and the first grid dimension of the flagging launch
   int skip_single;    // mixed batch: sequences with one query token are left to the single-token kernel
+  int use_pipe;       // lean kernel's cases on its software-pipelined variant
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -754,6 +755,7 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
 }
 
 #include "attn_fast.h"
+#include "attn_pipe.h"
 #include "attn_pair.h"
 #include "attn_decode.h"
 
@@ -761,6 +763,7 @@ template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
   if (a.use_pair) return launch_pair<T, 128>(a, grid, st);
+  if (a.use_fast && a.use_pipe) return D == 64 ? launch_pipe<T, 64>(a, grid, st) : launch_pipe<T, 128>(a, grid, st);
   if (a.use_fast) return D == 64 ? launch_fast<T, 64>(a, grid, st) : launch_fast<T, 128>(a, grid, st);
   if (a.use_async) {
     if (a.nw == 8) {
@@ -941,11 +944,13 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.max_seqlen_k <= 128 * 64 && p.alibi_slopes == nullptr &&
                !(p.softcap > 0.f);
   a.use_pair = 0;
+  a.use_pipe = 0;
   a.redo_flags = nullptr;
   a.redo_rows = 0;
   a.redo_grid_x = 0;
   if (const char* force = fg_options().attn_kernel; force[0] != 0) {
-    a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p');
+    a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p' || force[0] == 'x');
+    a.use_pipe = force[0] == 'x';
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && (p.D == 64 || p.D == 96 || p.D == 128)) {
       a.nw = force[1] == '8' ? 8 : 4;
