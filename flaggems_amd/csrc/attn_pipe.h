@@ -23,12 +23,22 @@
 // slot; at the top of step 2t+1, K(t) is no longer read (its second half was scored in step 2t) and K(t+2)
 // is requested.  Two K and two V slots: 64 KB for head dim 128, two workgroups per CU.
 //
+// The vector ALU's issue port, not the matrix pipe, is the scarce resource (an exponential holds it ~8 cycles,
+// any other vector instruction 4, an MFMA 8): so the per-score work is one exponential, an addition, half a
+// convert and half a three-way maximum, and nothing else (measured: two exponentials and three to four plain
+// instructions fit behind one MFMA of the same wave; v_dot2 instructions do not, they queue behind the MFMA).  The softmax scale is folded into Q
+// once (Q * scale * log2(e), rounded to the input type: an error of ~2^-9 per element of Q that averages to
+// ~1e-3 in a base-2 score, well below the rounding of P itself), and the row's reference m is subtracted by
+// the matrix pipe: one extra MFMA per step multiplies a fragment of ones with a fragment holding -m split in
+// three 16-bit pieces, so the accumulator leaves the pipe as S*scale - m.  The reference moves only when a
+// lane finds a score more than 2^8 above it (a lane-local test, no exchange on the common path); then the
+// waiting scores, O and the row sum are shifted once.
+//
 // Every wave runs every step of its workgroup in the same form: half tiles that lie wholly outside a wave's
 // mask bounds are scored and masked to -inf like the partly masked ones (P = 0 adds nothing to O) instead of
 // being branched around.  Variants of the step body that merge again cost this compiler a second copy of the
 // accumulators (80 registers of moves per step); the waves that would skip are not the ones the workgroup
-// waits for.  The slot a tile sits in alternates at run time: the lane's fragment addresses are moved from one
-// slot to the other once per tile (16 additions), so the loop body is one tile = two steps, unrolled once.
+// waits for.  The loop body is two tiles = four steps, so that ring slots and buffers are instruction immediates.
 // This header is included by attn_varlen.hip inside its unnamed namespace, behind attn_fast.h.
 
 template <int N, typename V>
@@ -39,24 +49,6 @@ template <int N, typename V>
 __device__ __forceinline__ void lds_wait_n2(V& r0, V& r1) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(r0), "+v"(r1) : "i"(N));
 }
-
-template <typename T> struct PipeDot2;
-template <> struct PipeDot2<bf16_t> {
-  typedef bf16_t V2 __attribute__((ext_vector_type(2)));
-  typedef short S2 __attribute__((ext_vector_type(2)));
-  // acc + a.x + a.y, on the rounded values that the PV MFMA will use
-  static __device__ __forceinline__ float add_pair(V2 a, float acc) {
-    const S2 ones = {(short)0x3f80, (short)0x3f80};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(V2, a), __builtin_bit_cast(V2, ones), acc, false);
-  }
-};
-template <> struct PipeDot2<f16_t> {
-  typedef f16_t V2 __attribute__((ext_vector_type(2)));
-  static __device__ __forceinline__ float add_pair(V2 a, float acc) {
-    const V2 ones = {(f16_t)1.0f, (f16_t)1.0f};
-    return __builtin_amdgcn_fdot2(a, ones, acc, false);
-  }
-};
 
 template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
@@ -120,8 +112,19 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 v = {0u, 0u, 0u, 0u};
       if (row_ok) v = *reinterpret_cast<const u32x4*>(qp + ks * 16 + half * 8);
-      qf[ks] = __builtin_bit_cast(Frag, v);
+      Frag f = __builtin_bit_cast(Frag, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (T)((float)f[e] * a.scale_log2);  // scores leave the MFMA in base-2 units
+      qf[ks] = f;
     }
+  }
+  // the reference m enters the scores through the matrix pipe: ones_f (k-slots 0..2 of the lower half-wave) times
+  // m_f (-m as three 16-bit pieces in the same slots of the lane that owns the row)
+  Frag ones_f, m_f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    ones_f[e] = (T)((half == 0 && e < 3) ? 1.0f : 0.0f);
+    m_f[e] = (T)0.0f;
   }
   f32x16 o_acc[DT];
 #pragma unroll
@@ -210,7 +213,6 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     v_addr1[dt] = lds0 + 2 * OPB + (v_key0 + 4) * RB + v_byte + (((dt * 4) ^ vx1) * 16);
   }
 
-  const float sc = a.scale_log2;
   // visible keys of this lane's row, relative to the first key of the workgroup: [col_lo, col_hi]
   const int col_hi = (a.has_right ? (qrow + shift + a.right_off_w < k_len - 1 ? qrow + shift + a.right_off_w : k_len - 1)
                                   : k_len - 1) - key_base - half * 8;
@@ -218,37 +220,37 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
 
   f32x16 s_buf[2];      // S(h) in buffer h & 1
   Frag pf[2];           // P(h) as the B operand of the PV MFMAs (2 x 16 keys)
-  float m_use = 0.f;    // reference of the scores waiting in s_buf (0 for a row that has seen no key)
   float psum = 0.f;
   float tmax_a = -INFINITY, tmax_b = -INFINITY;
   u32x4 kring[RING];
   u32x2 vring[RING][2];
 
-  // fragment read for MFMA `i` of phase A (key sub-tile KT of the K slot k_addr points into) or of phase B (the keys
-  // of sub-tile KT in the V slot v_addr points into)
-  auto read_k = [&](auto i_c, auto kt_c) {
-    constexpr int i = decltype(i_c)::value, KT = decltype(kt_c)::value;
-    kring[i % RING] = lds_read_b128_imm<KT * 32 * RB>(k_addr[i]);
+  // fragment read for MFMA `i` of phase A (key sub-tile KT of K slot SK) or of phase B (the keys of sub-tile KT in
+  // V slot SV)
+  auto read_k = [&](auto i_c, auto sk_c, auto kt_c) {
+    constexpr int i = decltype(i_c)::value, SK = decltype(sk_c)::value, KT = decltype(kt_c)::value;
+    kring[i % RING] = lds_read_b128_imm<SK * OPB + KT * 32 * RB>(k_addr[i]);
   };
-  auto read_v = [&](auto i_c, auto kt_c) {
-    constexpr int i = decltype(i_c)::value, KT = decltype(kt_c)::value;
+  auto read_v = [&](auto i_c, auto sv_c, auto kt_c) {
+    constexpr int i = decltype(i_c)::value, SV = decltype(sv_c)::value, KT = decltype(kt_c)::value;
     constexpr int dt = i / 2, t4 = KT * 2 + i % 2;
-    vring[i % RING][0] = lds_read_tr_b64_imm<t4 * 16 * RB>(v_addr0[dt]);
-    vring[i % RING][1] = lds_read_tr_b64_imm<t4 * 16 * RB>(v_addr1[dt]);
+    vring[i % RING][0] = lds_read_tr_b64_imm<SV * OPB + t4 * 16 * RB>(v_addr0[dt]);
+    vring[i % RING][1] = lds_read_tr_b64_imm<SV * OPB + t4 * 16 * RB>(v_addr1[dt]);
   };
 
-  // Phase A of the step whose scores S(h) sit in buffer CUR.  QK: S(h+1) -> buffer CUR^1 from key sub-tile
-  // CUR^1 of the K slot k_addr points into.  EXP: P(h) = exp2(S(h) * sc - m_use) and its row sum; the last RING
-  // slots then start the V fragment reads of the phase B that follows.
-  auto phase_a = [&](auto cur_c, auto qk_c, auto exp_c) {
+  // Phase A of the step whose scores S(h) sit in buffer CUR.  QK: S(h+1) = K.Q^T - m -> buffer CUR^1, from key
+  // sub-tile CUR^1 of K slot SK.  EXP: P(h) = exp2(S(h)) and its row sum; the last RING slots then start the V
+  // fragment reads of the phase B that follows (V slot SV).
+  auto phase_a = [&](auto cur_c, auto sk_c, auto sv_c, auto qk_c, auto exp_c) {
     constexpr int CUR = decltype(cur_c)::value;
     constexpr bool QK = decltype(qk_c)::value != 0, EXP = decltype(exp_c)::value != 0;
     constexpr bool PRE_V = EXP;
     constexpr int NXT = CUR ^ 1;
     if constexpr (QK) {
+      a_static_for<0, RING>([&](auto ic) { read_k(ic, sk_c, AInt<NXT>{}); });
 #pragma unroll
       for (int e = 0; e < 16; ++e) s_buf[NXT][e] = 0.f;
-      a_static_for<0, RING>([&](auto ic) { read_k(ic, AInt<NXT>{}); });
+      s_buf[NXT] = AttnMfma<T>::mma(ones_f, m_f, s_buf[NXT]);  // -m, while the first K fragments arrive
     }
     if constexpr (EXP) psum = 0.f;
     a_static_for<0, KS>([&](auto ic) {
@@ -260,10 +262,10 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
         constexpr int y3 = (RING > 3) ? ((i + 3 < KS) ? 1 : (PRE_V ? 2 : 0)) : 0;
         lds_wait_n<y1 + y2 + y3>(kring[i % RING]);
         s_buf[NXT] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, kring[i % RING]), qf[i], s_buf[NXT]);
-        if constexpr (i + RING < KS) read_k(AInt<i + RING>{}, AInt<NXT>{});
-        else if constexpr (PRE_V) read_v(AInt<i + RING - KS>{}, cur_c);
+        if constexpr (i + RING < KS) read_k(AInt<i + RING>{}, sk_c, AInt<NXT>{});
+        else if constexpr (PRE_V) read_v(AInt<i + RING - KS>{}, sv_c, cur_c);
       } else if constexpr (PRE_V) {
-        if constexpr (i + RING >= KS) read_v(AInt<i + RING - KS>{}, cur_c);
+        if constexpr (i + RING >= KS) read_v(AInt<i + RING - KS>{}, sv_c, cur_c);
       }
       if constexpr (EXP) {
         // 8 score pairs over KS slots: elements 2w, 2w+1 of half t2 -> word w of pf[t2]
@@ -272,11 +274,11 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
           constexpr int pi = i * per + decltype(jc)::value;
           if constexpr (pi < 8) {
             constexpr int t2 = pi / 4, w = pi % 4;
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(s_buf[CUR][t2 * 8 + 2 * w], sc, -m_use));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(s_buf[CUR][t2 * 8 + 2 * w + 1], sc, -m_use));
+            const float p0 = __builtin_amdgcn_exp2f(s_buf[CUR][t2 * 8 + 2 * w]);
+            const float p1 = __builtin_amdgcn_exp2f(s_buf[CUR][t2 * 8 + 2 * w + 1]);
             typedef T T2 __attribute__((ext_vector_type(2)));
             const T2 pk = {(T)p0, (T)p1};
-            psum = PipeDot2<T>::add_pair(pk, psum);
+            psum += p0 + p1;  // (dot-product instructions would halve this, but they wait for the matrix pipe)
             u32x4 words = __builtin_bit_cast(u32x4, pf[t2]);
             words[w] = __builtin_bit_cast(uint32_t, pk);
             pf[t2] = __builtin_bit_cast(Frag, words);
@@ -288,9 +290,10 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     if constexpr (EXP) l_run += xhalf_sum(psum);
   };
 
-  // Phase B.  PV: O += V(keys of sub-tile CUR)^T.P (the first RING fragment pairs were requested by phase A).
-  // MAX: running maximum over S(h+1) in buffer CUR^1 (redone by mask_and_max where the half tile needs a mask).
-  auto phase_b = [&](auto cur_c, auto max_c) {
+  // Phase B.  PV: O += V(keys of sub-tile CUR of V slot SV)^T.P (the first RING fragment pairs were requested by
+  // phase A).  MAX: the lane's maximum over S(h+1) in buffer CUR^1 (redone by mask_and_max where the half tile
+  // needs a mask); it starts two MFMAs into the phase, when the last scores have left the matrix pipe.
+  auto phase_b = [&](auto cur_c, auto sv_c, auto max_c) {
     constexpr int CUR = decltype(cur_c)::value;
     constexpr bool MAX = decltype(max_c)::value != 0;
     constexpr int NXT = CUR ^ 1;
@@ -301,22 +304,24 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
       lds_wait_n2<2 * ahead>(vring[i % RING][0], vring[i % RING][1]);
       const u32x4 both = {vring[i % RING][0][0], vring[i % RING][0][1], vring[i % RING][1][0], vring[i % RING][1][1]};
       o_acc[i / 2] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[i % 2], o_acc[i / 2]);
-      if constexpr (i + RING < NPV) read_v(AInt<i + RING>{}, cur_c);
-      if constexpr (MAX) {
-        constexpr int per = 8 / NPV > 0 ? 8 / NPV : 1;
+      if constexpr (i + RING < NPV) read_v(AInt<i + RING>{}, sv_c, cur_c);
+      if constexpr (MAX && i >= 2) {
+        // the 8 score pairs over the slots from the third on
+        constexpr int per = (8 + NPV - 3) / (NPV - 2);
         a_static_for<0, per>([&](auto jc) {
-          constexpr int pi = i * per + decltype(jc)::value;
+          constexpr int pi = (i - 2) * per + decltype(jc)::value;
           if constexpr (pi < 8) {
             if constexpr (pi % 2 == 0) tmax_a = fmaxf(fmaxf(tmax_a, s_buf[NXT][2 * pi]), s_buf[NXT][2 * pi + 1]);
             else tmax_b = fmaxf(fmaxf(tmax_b, s_buf[NXT][2 * pi]), s_buf[NXT][2 * pi + 1]);
           }
         });
+        if constexpr (i == NPV - 1) asm volatile("" : "+v"(tmax_a), "+v"(tmax_b));  // keeps the maxima inside their slots
       }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
 
-  // masks on the raw scores of half tile h (in buffer BUF), then their maximum (diagonal, window edge and last tiles)
+  // masks on the scores of half tile h (in buffer BUF), then their maximum (diagonal, window edge and last tiles)
   auto mask_and_max = [&](int h, auto buf_c) {
     constexpr int BUF = decltype(buf_c)::value;
     // element e is key key_base + h*32 + half*8 + (e>>3)*16 + (e&7)
@@ -339,66 +344,65 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     return (key0 + kHB > k_len) || (a.has_right && key0 + kHB - 1 > row0 + shift + a.right_off_w) ||
            (a.has_left && key0 < wave_row_last + shift - a.left_off_w);
   };
-  // the maximum of the half tile just scored joins the running reference; O and the row sum follow when it moves
-  auto new_reference = [&]() {
-    float tmax = fmaxf(tmax_a, tmax_b) * sc;  // scale > 0, so the maximum commutes with it
-    tmax = xhalf_max(tmax);
-    // the reference moves only when exceeded by more than 2^8: any reference gives the same result as long as
-    // P and the running sum use the same one
-    const bool moved = tmax > m_run + 8.0f;
-    const float m_new = moved ? tmax : m_run;
-    m_use = m_new == -INFINITY ? 0.f : m_new;
-    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
-      const float alpha = moved ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.0f;
+  // The scores in buffer BUF are relative to the reference m_run they were scored with.  Where a lane finds one
+  // more than 2^8 above it (or the row has no reference yet and sees its first key), the row's reference moves to
+  // the new maximum: the waiting scores, O and the row sum are shifted by the difference and -m is split anew.
+  // Any reference gives the same result as long as P and the running sum use the same one.
+  auto new_reference = [&](auto buf_c) {
+    constexpr int BUF = decltype(buf_c)::value;
+    const float tl = fmaxf(tmax_a, tmax_b);
+    const bool fresh = m_run == -INFINITY;
+    if (__builtin_amdgcn_ballot_w64(tl > 8.0f || (fresh && tl > -INFINITY)) == 0) return;
+    const float tmax = xhalf_max(tl);
+    const bool moved = tmax > 8.0f || (fresh && tmax > -INFINITY);
+    const float delta = moved ? tmax : 0.f;
+    const float alpha = __builtin_amdgcn_exp2f(-delta);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int e = 0; e < 16; ++e) s_buf[BUF][e] -= delta;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
-      l_run *= alpha;
-    }
-    m_run = m_new;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
+    l_run *= alpha;
+    if (moved) m_run = (fresh ? 0.f : m_run) + delta;
+    // -m_run as three pieces of the input type (their sum is exact to ~2^-24 of m), in k-slots 0..2 of the lane
+    // of the lower half-wave that owns the row
+    const float mm = (m_run == -INFINITY || half != 0) ? 0.f : -m_run;
+    const T hi = (T)mm;
+    const float r1 = mm - (float)hi;
+    const T mid = (T)r1;
+    const T lo = (T)(r1 - (float)mid);
+    m_f[0] = hi;
+    m_f[1] = mid;
+    m_f[2] = lo;
   };
 
-  // Step h = 2t + KT: S(h) sits in buffer KT and V(t) in the slot v_addr points into; S(h+1) comes from the second
-  // half of K(t) (KT = 0) or the first half of K(t+1) (KT = 1), which is where k_addr points.  LAST: the final step
-  // of the workgroup, which has no S(h+1) to score.
-  auto step = [&](int t, auto kt_c, auto last_c) {
-    constexpr int KT = decltype(kt_c)::value;
+  // Step h = 2t + KT of a tile t of parity PAR: S(h) sits in buffer KT, V(t) in V slot PAR; S(h+1) comes from the
+  // second half of K(t) (KT = 0: K slot PAR) or the first half of K(t+1) (KT = 1: K slot PAR^1).  LAST: the final
+  // step of the workgroup, which has no S(h+1) to score.
+  auto step = [&](int t, auto par_c, auto kt_c, auto last_c) {
+    constexpr int PAR = decltype(par_c)::value, KT = decltype(kt_c)::value;
     constexpr bool LAST = decltype(last_c)::value != 0;
+    constexpr int SK = KT == 0 ? PAR : (PAR ^ 1);
     const int h = 2 * t + KT;
     // landed: V(t) (KT = 0) or K(t+1) (KT = 1); the request behind it, K(t+1) resp. V(t+1), exists iff t+1 < T_
     if (t + 1 < T_) FG_WAIT_VM(IPW);
     else FG_WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
     if constexpr (KT == 0) {
-      if (t + 1 < T_) issue_op(t + 1, (t + 1) & 1, AInt<1>{});  // V(t-1) is no longer read
+      if (t + 1 < T_) issue_op(t + 1, PAR ^ 1, AInt<1>{});  // V(t-1) is no longer read
     } else {
-      if (t + 2 < T_) issue_op(t + 2, t & 1, AInt<0>{});        // K(t) is no longer read
+      if (t + 2 < T_) issue_op(t + 2, PAR, AInt<0>{});      // K(t) is no longer read
     }
     if constexpr (!LAST) {
-      phase_a(kt_c, AInt<1>{}, AInt<1>{});
-      phase_b(kt_c, AInt<1>{});
+      phase_a(kt_c, AInt<SK>{}, par_c, AInt<1>{}, AInt<1>{});
+      phase_b(kt_c, par_c, AInt<1>{});
       if (needs_mask(h + 1)) mask_and_max(h + 1, AInt<KT ^ 1>{});
-      new_reference();
+      new_reference(AInt<KT ^ 1>{});
     } else {
-      phase_a(kt_c, AInt<0>{}, AInt<1>{});
-      phase_b(kt_c, AInt<0>{});
+      phase_a(kt_c, AInt<SK>{}, par_c, AInt<0>{}, AInt<1>{});
+      phase_b(kt_c, par_c, AInt<0>{});
     }
-  };
-  // the lane's fragment addresses move to the other slot of their ring
-  int k_flip = OPB, v_flip = OPB;
-  auto flip_k = [&]() {
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_addr[ks] += (uint32_t)k_flip;
-    k_flip = -k_flip;
-  };
-  auto flip_v = [&]() {
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      v_addr0[dt] += (uint32_t)v_flip;
-      v_addr1[dt] += (uint32_t)v_flip;
-    }
-    v_flip = -v_flip;
   };
 
   if (T_ > 0) {
@@ -409,17 +413,26 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     if (1 < T_) FG_WAIT_VM(2 * IPW);
     else FG_WAIT_VM(IPW);
     __builtin_amdgcn_s_barrier();
-    phase_a(AInt<1>{}, AInt<1>{}, AInt<0>{});
+    phase_a(AInt<1>{}, AInt<0>{}, AInt<0>{}, AInt<1>{}, AInt<0>{});
     mask_and_max(0, AInt<0>{});
-    new_reference();
-    for (int t = 0; t + 1 < T_; ++t) {
-      step(t, AInt<0>{}, AInt<0>{});
-      flip_k();
-      step(t, AInt<1>{}, AInt<0>{});
-      flip_v();
+    new_reference(AInt<0>{});
+    // every step but the last, two tiles per trip
+    int t = 0;
+    for (; t + 2 < T_; t += 2) {
+      step(t, AInt<0>{}, AInt<0>{}, AInt<0>{});
+      step(t, AInt<0>{}, AInt<1>{}, AInt<0>{});
+      step(t + 1, AInt<1>{}, AInt<0>{}, AInt<0>{});
+      step(t + 1, AInt<1>{}, AInt<1>{}, AInt<0>{});
     }
-    step(T_ - 1, AInt<0>{}, AInt<0>{});
-    step(T_ - 1, AInt<1>{}, AInt<1>{});
+    if (t + 2 == T_) {
+      step(t, AInt<0>{}, AInt<0>{}, AInt<0>{});
+      step(t, AInt<0>{}, AInt<1>{}, AInt<0>{});
+      step(t + 1, AInt<1>{}, AInt<0>{}, AInt<0>{});
+      step(t + 1, AInt<1>{}, AInt<1>{}, AInt<1>{});
+    } else {
+      step(t, AInt<0>{}, AInt<0>{}, AInt<0>{});
+      step(t, AInt<0>{}, AInt<1>{}, AInt<1>{});
+    }
   }
 
   // ---- epilogue --------------------------------------------------------------------------------------
