@@ -15,7 +15,7 @@
 // MFMA formulation, LDS row layout (swz) and the base-2 online softmax are those of the prefill
 // kernels.  Conditions (checked on the host): head dim 64 or 128, page size a power of two >= 16,
 // max_seqlen_q == 1, G <= 32, no ALiBi, no soft-cap, no left window.
-// This header is included by attn_varlen.hip inside its unnamed namespace, after attn_fast.h.
+// This header is included by attn_varlen.hip inside its unnamed namespace, after attn_pipe.h.
 
 struct DecodeArgs {
   FgFlashParams p;

@@ -1,16 +1,23 @@
-// Paged varlen attention forward, software-pipelined variant of the lean kernel (attn_fast.h) for the same
-// cases: head dim 64 or 128, page size a power of two >= 16, at most 8192 keys per sequence, no ALiBi, no
-// soft-cap.  Same work split (4 waves x 32 query rows, a GQA group's heads per workgroup), MFMA formulation
-// (S^T = K.Q^T, O^T = V^T.P^T, MFMA 32x32x16), swizzled LDS tiles filled by global_load_lds, and lazily
-// re-referenced base-2 online softmax.  What differs is the order of work inside a wave.
+// Paged varlen attention forward, the lean kernel for the common case: head dim 64 or 128, page size a power of
+// two >= 16, no ALiBi, no soft-cap.  Same work split (4 waves x 32 query rows, a GQA group's heads per
+// workgroup), MFMA formulation (S^T = K.Q^T, O^T = V^T.P^T, MFMA 32x32x16) and swizzled LDS tiles filled by
+// global_load_lds as attn_varlen_async_kernel; what differs is that nothing address-like is recomputed per
+// tile on the vector ALU, and the order of work inside a wave:
+//   * A wave moves 16 consecutive key rows of every tile, which lie in one page.  So the page id and the row base
+//     are wave-uniform: the ids of 128 tiles sit in two registers (a lane each) and become a 64-bit scalar base;
+//     each lane adds a 32-bit offset fixed for the whole kernel.  The window of 128 ids is re-read when a
+//     sequence runs past it.  The last, partial tile of a sequence clamps keys per lane and looks its pages up
+//     per lane; that path runs once per sequence.
+//   * Stage, sub-tile and k-step offsets of every fragment read are instruction immediates on top of lane-constant
+//     registers.
 //
-// Measured on gfx950, one wave issues a plain vector instruction every ~6 cycles and an exponential every
-// ~17, and it cannot issue anything while it waits for a matrix result; a vector instruction placed between
-// two MFMAs of the same wave that do not need its result costs nothing while the matrix pipe is busy (32
-// cycles per MFMA).  The lean kernel runs QK^T, softmax and PV of a tile one after the other, so the matrix
-// pipe idles through ~1200 cycles of softmax per tile and wave, and two waves per SIMD do not mesh well
-// enough to fill the gap.  Here the work is cut into half tiles of 32 keys (one 32x32 score block per wave),
-// and the softmax of half tile h is split in two, each part in the shadow of the MFMAs of a neighbour:
+// Measured on gfx950, one wave issues a plain vector instruction every ~5 cycles and an exponential every ~9,
+// and it cannot issue anything while it waits for a matrix result; a vector instruction placed between two
+// MFMAs of the same wave that do not need its result costs nothing while the matrix pipe is busy (32 cycles per
+// MFMA).  Running QK^T, softmax and PV of a tile one after the other leaves the matrix pipe idle through ~1200
+// cycles of softmax per tile and wave, and two waves per SIMD do not mesh well enough to fill the gap.  So the
+// work is cut into half tiles of 32 keys (one 32x32 score block per wave), and the softmax of half tile h is
+// split in two, each part in the shadow of the MFMAs of a neighbour:
 //
 //   phase A of step h:  S(h+1) = K(h+1).Q^T   D/16 MFMAs  ||  P(h) = exp2(S(h)*scale - m), row sums
 //   phase B of step h:  O     += V(h)^T.P(h)  D/16 MFMAs  ||  running max over S(h+1)
@@ -23,7 +30,7 @@
 // slot; at the top of step 2t+1, K(t) is no longer read (its second half was scored in step 2t) and K(t+2)
 // is requested.  Two K and two V slots: 64 KB for head dim 128, two workgroups per CU.
 //
-// The vector ALU's issue port, not the matrix pipe, is the scarce resource (an exponential holds it ~8 cycles,
+// The vector ALU's issue port is as scarce as the matrix pipe (an exponential holds it ~8 cycles,
 // any other vector instruction 4, an MFMA 8): so the per-score work is one exponential, an addition, half a
 // convert and half a three-way maximum, and nothing else (measured: two exponentials and three to four plain
 // instructions fit behind one MFMA of the same wave; v_dot2 instructions do not, they queue behind the MFMA).  The softmax scale is folded into Q
@@ -39,7 +46,31 @@
 // being branched around.  Variants of the step body that merge again cost this compiler a second copy of the
 // accumulators (80 registers of moves per step); the waves that would skip are not the ones the workgroup
 // waits for.  The loop body is two tiles = four steps, so that ring slots and buffers are instruction immediates.
-// This header is included by attn_varlen.hip inside its unnamed namespace, behind attn_fast.h.
+//
+// RBW = query row blocks of 32 per wave.  Only RBW = 1 is built (two workgroups per CU).  With RBW = 2 every K or
+// V fragment read from LDS feeds two MFMAs and the per-step costs are shared by twice the work, but the ~370
+// registers mean one wave per SIMD, and this compiler then keeps the score accumulators in the AGPR half of the
+// register file and moves every score to a VGPR before the vector ALU can touch it: measured 2.4 to 3.5 times
+// slower, so it is not instantiated.
+// This header is included by attn_varlen.hip inside its unnamed namespace.
+
+template <int OFF> __device__ __forceinline__ u32x4 lds_read_b128_imm(uint32_t addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return v;
+}
+template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr_b64_imm(uint32_t addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+  return v;
+}
+template <int I> struct AInt { static constexpr int value = I; };
+template <int B, int E, typename F> __device__ __forceinline__ void a_static_for(F&& f) {
+  if constexpr (B < E) {
+    f(AInt<B>{});
+    a_static_for<B + 1, E>(f);
+  }
+}
 
 template <int N, typename V>
 __device__ __forceinline__ void lds_wait_n(V& r) {
@@ -50,29 +81,45 @@ __device__ __forceinline__ void lds_wait_n2(V& r0, V& r1) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(r0), "+v"(r1) : "i"(N));
 }
 
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
+template <typename T, int D, int RBW>
+__global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kernel(AttnArgs a) {
   typedef typename AttnMfma<T>::Frag Frag;
   constexpr int RB = 2 * D;            // bytes per key row in LDS
   constexpr int CPR = RB / 16;         // 16-byte chunks per row
-  constexpr int KS = D / 16;           // MFMA k-steps over the head dim = MFMAs of phase A
+  constexpr int KS = D / 16;           // MFMA k-steps over the head dim = fragment reads of phase A
   constexpr int DT = D / 32;           // 32-row output sub-tiles over the head dim
-  constexpr int NPV = 2 * DT;          // MFMAs of phase B
+  constexpr int NPV = 2 * DT;          // fragment reads of phase B
   constexpr int OPB = kBN * RB;        // one operand tile
   constexpr int KPI = 1024 / RB;       // key rows per DMA instruction
   constexpr int IPW = kBN / KPI / 4;   // DMA instructions per wave, operand and tile
-  constexpr int RING = KS < 4 ? KS : 4;  // fragment reads run this many MFMAs ahead
+  constexpr int RING = KS < 4 ? KS : 4;  // fragment reads run this many slots ahead
   constexpr int kHB = kBN / 2;         // keys per half tile
-  static_assert(KS == NPV && KS >= RING, "both phases issue the same number of MFMAs");
+  constexpr int WROWS = kRW * RBW;     // query rows per wave
+  static_assert(KS == NPV && KS >= RING, "both phases read the same number of fragments");
   extern __shared__ __attribute__((aligned(16))) char lds[];  // K slot 0, K slot 1, V slot 0, V slot 1
 
   const FgFlashParams& p = a.p;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, ql = lane & 31;
-  // long (late) row blocks first, order rotated per (sequence, head group): see attn_fast.h
-  const int b = blockIdx.y, hgroup = blockIdx.z;
-  const int m_block = (int)((gridDim.x - 1 - blockIdx.x + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
+  // Workgroups go to the 8 XCDs round-robin by their linear id, and every XCD has its own L2.  The id is therefore
+  // re-read as (XCD, turn) and XCD k works through the k-th eighth of the (head group, sequence, row block) order:
+  // all row blocks of a sequence and KV head run on one XCD, next to each other in time, so that its K and V are
+  // fetched into one L2 instead of eight.  Within a sequence, long (late) row blocks first; the order is rotated
+  // per (sequence, head group) so that sequences of one row block do not all start in the same turn.
+  int bx = blockIdx.x, b = blockIdx.y, hgroup = blockIdx.z;
+  if (a.xcd_remap) {
+    const unsigned total = gridDim.x * gridDim.y * gridDim.z;
+    const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const unsigned per = total / 8;
+    if (lin < per * 8) {  // (a ragged tail keeps its place)
+      const unsigned idx = (lin % 8) * per + lin / 8;
+      bx = (int)(idx % gridDim.x);
+      b = (int)((idx / gridDim.x) % gridDim.y);
+      hgroup = (int)(idx / (gridDim.x * gridDim.y));
+    }
+  }
+  const int m_block = (int)((gridDim.x - 1 - bx + (unsigned)(b * 5 + hgroup * 3)) % gridDim.x);
 
   const int q_bos = p.cu_seqlens_q[b];
   const int q_len = p.cu_seqlens_q[b + 1] - q_bos;
@@ -82,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
 
   const int waves_per_head = 4 / a.hpb;
   const int head = hgroup * a.hpb + wave / waves_per_head;
-  const int row0 = block_row0 + (wave % waves_per_head) * kRW;
+  const int row0 = block_row0 + (wave % waves_per_head) * WROWS;
   const int kv_head = head / (p.Hq / p.Hk);
 
   // ---- key tiles of the workgroup: [n_min, n_max) ----------------------------------------------------------
@@ -100,12 +147,12 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   }
   const int T_ = n_max > n_min ? n_max - n_min : 0;  // tiles of the workgroup
   const int key_base = n_min * kBN;
-  const int wave_row_last = (row0 + kRW - 1 < q_len ? row0 + kRW - 1 : q_len - 1);
 
-  // ---- Q fragments ---------------------------------------------------------------------------------
-  const int qrow = row0 + ql;
-  Frag qf[KS];
-  {
+  // ---- Q fragments, scaled: scores leave the MFMA in base-2 units -------------------------------------------
+  Frag qf[RBW][KS];
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb) {
+    const int qrow = row0 + rb * kRW + ql;
     const bool row_ok = qrow < q_len;
     const T* qp = (const T*)p.q + (int64_t)(q_bos + (row_ok ? qrow : 0)) * p.q_row_stride + (int64_t)head * p.q_head_stride;
 #pragma unroll
@@ -114,24 +161,30 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
       if (row_ok) v = *reinterpret_cast<const u32x4*>(qp + ks * 16 + half * 8);
       Frag f = __builtin_bit_cast(Frag, v);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = (T)((float)f[e] * a.scale_log2);  // scores leave the MFMA in base-2 units
-      qf[ks] = f;
+      for (int e = 0; e < 8; ++e) f[e] = (T)((float)f[e] * a.scale_log2);
+      qf[rb][ks] = f;
     }
   }
   // the reference m enters the scores through the matrix pipe: ones_f (k-slots 0..2 of the lower half-wave) times
   // m_f (-m as three 16-bit pieces in the same slots of the lane that owns the row)
-  Frag ones_f, m_f;
+  Frag ones_f, m_f[RBW];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     ones_f[e] = (T)((half == 0 && e < 3) ? 1.0f : 0.0f);
-    m_f[e] = (T)0.0f;
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb) m_f[rb][e] = (T)0.0f;
   }
-  f32x16 o_acc[DT];
+  f32x16 o_acc[RBW][DT];
+  float m_run[RBW], l_run[RBW];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int rb = 0; rb < RBW; ++rb) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) o_acc[dt][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[rb][dt][e] = 0.f;
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
+  }
 
   // ---- DMA geometry (as in the lean kernel: one page id per wave and tile, kept in two registers) ------
   const int32_t* btab = p.block_table + (int64_t)b * p.block_table_stride;
@@ -145,15 +198,18 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   const uint32_t lane_row_k = (uint32_t)(lane_key * (int)p.k_row_stride * 2);
   const uint32_t lane_row_v = (uint32_t)(lane_key * (int)p.v_row_stride * 2);
   const int last_page = k_len > 0 ? (k_len - 1) >> page_shift : 0;
-  int pg_cache0, pg_cache1;
-  {
-    int pg0 = ((n_min + lane) * kBN + wave * (IPW * KPI)) >> page_shift;
-    int pg1 = ((n_min + 64 + lane) * kBN + wave * (IPW * KPI)) >> page_shift;
+  // page ids of this wave's rows in tiles pg_base + l (pg_cache0) and pg_base + 64 + l (pg_cache1), lane l
+  int pg_cache0, pg_cache1, pg_base;
+  auto load_page_window = [&](int first_tile) {
+    pg_base = first_tile;
+    int pg0 = ((n_min + first_tile + lane) * kBN + wave * (IPW * KPI)) >> page_shift;
+    int pg1 = ((n_min + first_tile + 64 + lane) * kBN + wave * (IPW * KPI)) >> page_shift;
     pg0 = pg0 < last_page ? pg0 : last_page;
     pg1 = pg1 < last_page ? pg1 : last_page;
     pg_cache0 = btab[pg0];
     pg_cache1 = btab[pg1];
-  }
+  };
+  load_page_window(0);
   // one operand tile (K: is_v = 0, V: is_v = 1) of key tile n_min + t into `slot` of its ring
   auto issue_op = [&](int t, int slot, auto is_v_c) {
     constexpr bool IS_V = decltype(is_v_c)::value != 0;
@@ -164,7 +220,10 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     const int64_t row_stride = IS_V ? p.v_row_stride : p.k_row_stride;
     if (nb * kBN + kBN <= k_len) {
       // full tile: every key exists; one scalar row base per instruction, one 32-bit lane offset
-      const int tl = t < 127 ? t : 127;
+      // tiles are requested in the order V(1), K(2), V(2), K(3), ...: a window that starts one tile below the
+      // request that overran it still holds the V tile that follows
+      if (t - pg_base >= 128) load_page_window(t - 1);
+      const int tl = t - pg_base;
       const int64_t page = __builtin_amdgcn_readlane(tl < 64 ? pg_cache0 : pg_cache1, tl & 63);
       const int key = nb * kBN + wave * (IPW * KPI);
       const int slot_in_page = key & page_mask;
@@ -213,19 +272,24 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     v_addr1[dt] = lds0 + 2 * OPB + (v_key0 + 4) * RB + v_byte + (((dt * 4) ^ vx1) * 16);
   }
 
-  // visible keys of this lane's row, relative to the first key of the workgroup: [col_lo, col_hi]
-  const int col_hi = (a.has_right ? (qrow + shift + a.right_off_w < k_len - 1 ? qrow + shift + a.right_off_w : k_len - 1)
-                                  : k_len - 1) - key_base - half * 8;
-  const int col_lo = (a.has_left ? qrow + shift - a.left_off_w : 0) - key_base - half * 8;
+  // visible keys of this lane's rows, relative to the first key of the workgroup and the lane's half: [col_lo, col_hi]
+  int col_hi[RBW], col_lo[RBW];
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb) {
+    const int qrow = row0 + rb * kRW + ql;
+    col_hi[rb] = (a.has_right ? (qrow + shift + a.right_off_w < k_len - 1 ? qrow + shift + a.right_off_w : k_len - 1)
+                              : k_len - 1) - key_base - half * 8;
+    col_lo[rb] = (a.has_left ? qrow + shift - a.left_off_w : 0) - key_base - half * 8;
+  }
 
-  f32x16 s_buf[2];      // S(h) in buffer h & 1
-  Frag pf[2];           // P(h) as the B operand of the PV MFMAs (2 x 16 keys)
-  float psum = 0.f;
-  float tmax_a = -INFINITY, tmax_b = -INFINITY;
+  f32x16 s_buf[RBW][2];   // S(h) in buffer h & 1
+  Frag pf[RBW][2];        // P(h) as the B operand of the PV MFMAs (2 x 16 keys)
+  float psum[RBW];
+  float tmax_a[RBW], tmax_b[RBW];
   u32x4 kring[RING];
   u32x2 vring[RING][2];
 
-  // fragment read for MFMA `i` of phase A (key sub-tile KT of K slot SK) or of phase B (the keys of sub-tile KT in
+  // fragment read for slot `i` of phase A (key sub-tile KT of K slot SK) or of phase B (the keys of sub-tile KT in
   // V slot SV)
   auto read_k = [&](auto i_c, auto sk_c, auto kt_c) {
     constexpr int i = decltype(i_c)::value, SK = decltype(sk_c)::value, KT = decltype(kt_c)::value;
@@ -233,14 +297,15 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   };
   auto read_v = [&](auto i_c, auto sv_c, auto kt_c) {
     constexpr int i = decltype(i_c)::value, SV = decltype(sv_c)::value, KT = decltype(kt_c)::value;
-    constexpr int dt = i / 2, t4 = KT * 2 + i % 2;
+    constexpr int dt = (i / 2) % DT, t4 = KT * 2 + i % 2;
     vring[i % RING][0] = lds_read_tr_b64_imm<SV * OPB + t4 * 16 * RB>(v_addr0[dt]);
     vring[i % RING][1] = lds_read_tr_b64_imm<SV * OPB + t4 * 16 * RB>(v_addr1[dt]);
   };
 
   // Phase A of the step whose scores S(h) sit in buffer CUR.  QK: S(h+1) = K.Q^T - m -> buffer CUR^1, from key
   // sub-tile CUR^1 of K slot SK.  EXP: P(h) = exp2(S(h)) and its row sum; the last RING slots then start the V
-  // fragment reads of the phase B that follows (V slot SV).
+  // fragment reads of the phase B that follows (V slot SV).  Per slot: one K fragment, one MFMA and one score pair
+  // per row block.
   auto phase_a = [&](auto cur_c, auto sk_c, auto sv_c, auto qk_c, auto exp_c) {
     constexpr int CUR = decltype(cur_c)::value;
     constexpr bool QK = decltype(qk_c)::value != 0, EXP = decltype(exp_c)::value != 0;
@@ -249,10 +314,16 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     if constexpr (QK) {
       a_static_for<0, RING>([&](auto ic) { read_k(ic, sk_c, AInt<NXT>{}); });
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s_buf[NXT][e] = 0.f;
-      s_buf[NXT] = AttnMfma<T>::mma(ones_f, m_f, s_buf[NXT]);  // -m, while the first K fragments arrive
+      for (int rb = 0; rb < RBW; ++rb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_buf[rb][NXT][e] = 0.f;
+        s_buf[rb][NXT] = AttnMfma<T>::mma(ones_f, m_f[rb], s_buf[rb][NXT]);  // -m, while the first K fragments arrive
+      }
     }
-    if constexpr (EXP) psum = 0.f;
+    if constexpr (EXP) {
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) psum[rb] = 0.f;
+    }
     a_static_for<0, KS>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       if constexpr (QK) {
@@ -261,88 +332,106 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
         constexpr int y2 = (RING > 2) ? ((i + 2 < KS) ? 1 : (PRE_V ? 2 : 0)) : 0;
         constexpr int y3 = (RING > 3) ? ((i + 3 < KS) ? 1 : (PRE_V ? 2 : 0)) : 0;
         lds_wait_n<y1 + y2 + y3>(kring[i % RING]);
-        s_buf[NXT] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, kring[i % RING]), qf[i], s_buf[NXT]);
-        if constexpr (i + RING < KS) read_k(AInt<i + RING>{}, sk_c, AInt<NXT>{});
-        else if constexpr (PRE_V) read_v(AInt<i + RING - KS>{}, sv_c, cur_c);
-      } else if constexpr (PRE_V) {
-        if constexpr (i + RING >= KS) read_v(AInt<i + RING - KS>{}, sv_c, cur_c);
       }
-      if constexpr (EXP) {
-        // 8 score pairs over KS slots: elements 2w, 2w+1 of half t2 -> word w of pf[t2]
-        constexpr int per = 8 / KS > 0 ? 8 / KS : 1;
-        a_static_for<0, per>([&](auto jc) {
-          constexpr int pi = i * per + decltype(jc)::value;
-          if constexpr (pi < 8) {
-            constexpr int t2 = pi / 4, w = pi % 4;
-            const float p0 = __builtin_amdgcn_exp2f(s_buf[CUR][t2 * 8 + 2 * w]);
-            const float p1 = __builtin_amdgcn_exp2f(s_buf[CUR][t2 * 8 + 2 * w + 1]);
-            typedef T T2 __attribute__((ext_vector_type(2)));
-            const T2 pk = {(T)p0, (T)p1};
-            psum += p0 + p1;  // (dot-product instructions would halve this, but they wait for the matrix pipe)
-            u32x4 words = __builtin_bit_cast(u32x4, pf[t2]);
-            words[w] = __builtin_bit_cast(uint32_t, pk);
-            pf[t2] = __builtin_bit_cast(Frag, words);
-          }
-        });
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      a_static_for<0, RBW>([&](auto rc) {
+        constexpr int rb = decltype(rc)::value;
+        if constexpr (QK)
+          s_buf[rb][NXT] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, kring[i % RING]), qf[rb][i], s_buf[rb][NXT]);
+        if constexpr (rb == RBW - 1) {
+          if constexpr (QK && i + RING < KS) read_k(AInt<i + RING>{}, sk_c, AInt<NXT>{});
+          else if constexpr (PRE_V && i + RING >= KS) read_v(AInt<i + RING - KS>{}, sv_c, cur_c);
+        }
+        if constexpr (EXP) {
+          // 8 score pairs over KS slots: elements 2w, 2w+1 of half t2 -> word w of pf[t2]
+          constexpr int per = 8 / KS > 0 ? 8 / KS : 1;
+          a_static_for<0, per>([&](auto jc) {
+            constexpr int pi = i * per + decltype(jc)::value;
+            if constexpr (pi < 8) {
+              constexpr int t2 = pi / 4, w = pi % 4;
+              const float p0 = __builtin_amdgcn_exp2f(s_buf[rb][CUR][t2 * 8 + 2 * w]);
+              const float p1 = __builtin_amdgcn_exp2f(s_buf[rb][CUR][t2 * 8 + 2 * w + 1]);
+              typedef T T2 __attribute__((ext_vector_type(2)));
+              const T2 pk = {(T)p0, (T)p1};
+              psum[rb] += p0 + p1;  // (dot-product instructions would halve this, but they wait for the matrix pipe)
+              u32x4 words = __builtin_bit_cast(u32x4, pf[rb][t2]);
+              words[w] = __builtin_bit_cast(uint32_t, pk);
+              pf[rb][t2] = __builtin_bit_cast(Frag, words);
+            }
+          });
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
     });
-    if constexpr (EXP) l_run += xhalf_sum(psum);
+    if constexpr (EXP) {
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) l_run[rb] += xhalf_sum(psum[rb]);
+    }
   };
 
   // Phase B.  PV: O += V(keys of sub-tile CUR of V slot SV)^T.P (the first RING fragment pairs were requested by
   // phase A).  MAX: the lane's maximum over S(h+1) in buffer CUR^1 (redone by mask_and_max where the half tile
-  // needs a mask); it starts two MFMAs into the phase, when the last scores have left the matrix pipe.
+  // needs a mask); it starts two slots into the phase, when the last scores have left the matrix pipe.
   auto phase_b = [&](auto cur_c, auto sv_c, auto max_c) {
     constexpr int CUR = decltype(cur_c)::value;
     constexpr bool MAX = decltype(max_c)::value != 0;
     constexpr int NXT = CUR ^ 1;
-    if constexpr (MAX) tmax_a = tmax_b = -INFINITY;
+    if constexpr (MAX) {
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) tmax_a[rb] = tmax_b[rb] = -INFINITY;
+    }
     a_static_for<0, NPV>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       constexpr int ahead = (i + RING - 1 < NPV) ? RING - 1 : (NPV - 1 - i);
       lds_wait_n2<2 * ahead>(vring[i % RING][0], vring[i % RING][1]);
       const u32x4 both = {vring[i % RING][0][0], vring[i % RING][0][1], vring[i % RING][1][0], vring[i % RING][1][1]};
-      o_acc[i / 2] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[i % 2], o_acc[i / 2]);
-      if constexpr (i + RING < NPV) read_v(AInt<i + RING>{}, sv_c, cur_c);
-      if constexpr (MAX && i >= 2) {
-        // the 8 score pairs over the slots from the third on
-        constexpr int per = (8 + NPV - 3) / (NPV - 2);
-        a_static_for<0, per>([&](auto jc) {
-          constexpr int pi = (i - 2) * per + decltype(jc)::value;
-          if constexpr (pi < 8) {
-            if constexpr (pi % 2 == 0) tmax_a = fmaxf(fmaxf(tmax_a, s_buf[NXT][2 * pi]), s_buf[NXT][2 * pi + 1]);
-            else tmax_b = fmaxf(fmaxf(tmax_b, s_buf[NXT][2 * pi]), s_buf[NXT][2 * pi + 1]);
-          }
-        });
-        if constexpr (i == NPV - 1) asm volatile("" : "+v"(tmax_a), "+v"(tmax_b));  // keeps the maxima inside their slots
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      a_static_for<0, RBW>([&](auto rc) {
+        constexpr int rb = decltype(rc)::value;
+        o_acc[rb][i / 2] = AttnMfma<T>::mma(__builtin_bit_cast(Frag, both), pf[rb][i % 2], o_acc[rb][i / 2]);
+        if constexpr (rb == RBW - 1 && i + RING < NPV) read_v(AInt<i + RING>{}, sv_c, cur_c);
+        if constexpr (MAX && i >= 2) {
+          // the 8 score pairs over the slots from the third on
+          constexpr int per = (8 + NPV - 3) / (NPV - 2);
+          a_static_for<0, per>([&](auto jc) {
+            constexpr int pi = (i - 2) * per + decltype(jc)::value;
+            if constexpr (pi < 8) {
+              if constexpr (pi % 2 == 0)
+                tmax_a[rb] = fmaxf(fmaxf(tmax_a[rb], s_buf[rb][NXT][2 * pi]), s_buf[rb][NXT][2 * pi + 1]);
+              else
+                tmax_b[rb] = fmaxf(fmaxf(tmax_b[rb], s_buf[rb][NXT][2 * pi]), s_buf[rb][NXT][2 * pi + 1]);
+            }
+          });
+          if constexpr (i == NPV - 1) asm volatile("" : "+v"(tmax_a[rb]), "+v"(tmax_b[rb]));  // keeps the maxima in their slots
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
     });
   };
 
-  // masks on the scores of half tile h (in buffer BUF), then their maximum (diagonal, window edge and last tiles)
-  auto mask_and_max = [&](int h, auto buf_c) {
-    constexpr int BUF = decltype(buf_c)::value;
+  // masks on the scores of half tile h of row block RBI (in buffer BUF), then their maximum (diagonal, window edge
+  // and last tiles)
+  auto mask_and_max = [&](int h, auto rb_c, auto buf_c) {
+    constexpr int BUF = decltype(buf_c)::value, rb = decltype(rb_c)::value;
     // element e is key key_base + h*32 + half*8 + (e>>3)*16 + (e&7)
-    const int hi_rel = col_hi - h * kHB, lo_rel = col_lo - h * kHB;
+    const int hi_rel = col_hi[rb] - h * kHB, lo_rel = col_lo[rb] - h * kHB;
     float tm = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int rel = (e >> 3) * 16 + (e & 7);
-      float s = s_buf[BUF][e];
+      float s = s_buf[rb][BUF][e];
       s = rel > hi_rel ? -INFINITY : s;
       if (a.has_left) s = rel < lo_rel ? -INFINITY : s;
-      s_buf[BUF][e] = s;
+      s_buf[rb][BUF][e] = s;
       tm = fmaxf(tm, s);
     }
-    tmax_a = tm;
-    tmax_b = -INFINITY;
+    tmax_a[rb] = tm;
+    tmax_b[rb] = -INFINITY;
   };
-  auto needs_mask = [&](int h) {
+  auto needs_mask = [&](int h, int rb) {
     const int key0 = key_base + h * kHB;
-    return (key0 + kHB > k_len) || (a.has_right && key0 + kHB - 1 > row0 + shift + a.right_off_w) ||
-           (a.has_left && key0 < wave_row_last + shift - a.left_off_w);
+    const int r_first = row0 + rb * kRW;
+    const int r_last = (r_first + kRW - 1 < q_len ? r_first + kRW - 1 : q_len - 1);
+    return (key0 + kHB > k_len) || (a.has_right && key0 + kHB - 1 > r_first + shift + a.right_off_w) ||
+           (a.has_left && key0 < r_last + shift - a.left_off_w);
   };
   // The scores in buffer BUF are relative to the reference m_run they were scored with.  Where a lane finds one
   // more than 2^8 above it (or the row has no reference yet and sees its first key), the row's reference moves to
@@ -350,31 +439,46 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   // Any reference gives the same result as long as P and the running sum use the same one.
   auto new_reference = [&](auto buf_c) {
     constexpr int BUF = decltype(buf_c)::value;
-    const float tl = fmaxf(tmax_a, tmax_b);
-    const bool fresh = m_run == -INFINITY;
-    if (__builtin_amdgcn_ballot_w64(tl > 8.0f || (fresh && tl > -INFINITY)) == 0) return;
-    const float tmax = xhalf_max(tl);
-    const bool moved = tmax > 8.0f || (fresh && tmax > -INFINITY);
-    const float delta = moved ? tmax : 0.f;
-    const float alpha = __builtin_amdgcn_exp2f(-delta);
+    float tl[RBW];
+    bool any = false;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) s_buf[BUF][e] -= delta;
+    for (int rb = 0; rb < RBW; ++rb) {
+      tl[rb] = fmaxf(tmax_a[rb], tmax_b[rb]);
+      any = any || tl[rb] > 8.0f || (m_run[rb] == -INFINITY && tl[rb] > -INFINITY);
+    }
+    if (__builtin_amdgcn_ballot_w64(any) == 0) return;
+    a_static_for<0, RBW>([&](auto rc) {
+      constexpr int rb = decltype(rc)::value;
+      const bool fresh = m_run[rb] == -INFINITY;
+      const float tmax = xhalf_max(tl[rb]);
+      const bool moved = tmax > 8.0f || (fresh && tmax > -INFINITY);
+      if (__builtin_amdgcn_ballot_w64(moved) == 0) return;
+      const float delta = moved ? tmax : 0.f;
+      const float alpha = __builtin_amdgcn_exp2f(-delta);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int e = 0; e < 16; ++e) s_buf[rb][BUF][e] -= delta;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[dt][e] *= alpha;
-    l_run *= alpha;
-    if (moved) m_run = (fresh ? 0.f : m_run) + delta;
-    // -m_run as three pieces of the input type (their sum is exact to ~2^-24 of m), in k-slots 0..2 of the lane
-    // of the lower half-wave that owns the row
-    const float mm = (m_run == -INFINITY || half != 0) ? 0.f : -m_run;
-    const T hi = (T)mm;
-    const float r1 = mm - (float)hi;
-    const T mid = (T)r1;
-    const T lo = (T)(r1 - (float)mid);
-    m_f[0] = hi;
-    m_f[1] = mid;
-    m_f[2] = lo;
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o_acc[rb][dt][e] *= alpha;
+      l_run[rb] *= alpha;
+      if (moved) m_run[rb] = (fresh ? 0.f : m_run[rb]) + delta;
+      // -m_run as three pieces of the input type (their sum is exact to ~2^-24 of m), in k-slots 0..2 of the lane
+      // of the lower half-wave that owns the row
+      const float mm = (m_run[rb] == -INFINITY || half != 0) ? 0.f : -m_run[rb];
+      const T hi = (T)mm;
+      const float r1 = mm - (float)hi;
+      const T mid = (T)r1;
+      const T lo = (T)(r1 - (float)mid);
+      m_f[rb][0] = hi;
+      m_f[rb][1] = mid;
+      m_f[rb][2] = lo;
+    });
+  };
+  auto mask_where_needed = [&](int h, auto buf_c) {
+    a_static_for<0, RBW>([&](auto rc) {
+      if (needs_mask(h, decltype(rc)::value)) mask_and_max(h, rc, buf_c);
+    });
   };
 
   // Step h = 2t + KT of a tile t of parity PAR: S(h) sits in buffer KT, V(t) in V slot PAR; S(h+1) comes from the
@@ -397,7 +501,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     if constexpr (!LAST) {
       phase_a(kt_c, AInt<SK>{}, par_c, AInt<1>{}, AInt<1>{});
       phase_b(kt_c, par_c, AInt<1>{});
-      if (needs_mask(h + 1)) mask_and_max(h + 1, AInt<KT ^ 1>{});
+      mask_where_needed(h + 1, AInt<KT ^ 1>{});
       new_reference(AInt<KT ^ 1>{});
     } else {
       phase_a(kt_c, AInt<SK>{}, par_c, AInt<0>{}, AInt<1>{});
@@ -414,7 +518,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     else FG_WAIT_VM(IPW);
     __builtin_amdgcn_s_barrier();
     phase_a(AInt<1>{}, AInt<0>{}, AInt<0>{}, AInt<1>{}, AInt<0>{});
-    mask_and_max(0, AInt<0>{});
+    a_static_for<0, RBW>([&](auto rc) { mask_and_max(0, rc, AInt<0>{}); });
     new_reference(AInt<0>{});
     // every step but the last, two tiles per trip
     int t = 0;
@@ -436,34 +540,38 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   }
 
   // ---- epilogue --------------------------------------------------------------------------------------
-  if (qrow >= q_len) return;
-  const bool empty = l_run == 0.f || l_run != l_run;
-  const float inv = empty ? 1.f : 1.f / l_run;
-  if (p.lse != nullptr && half == 0) {
-    p.lse[(int64_t)head * p.total_q + q_bos + qrow] = empty ? INFINITY : m_run * 0.6931471805599453f + logf(l_run);
-  }
-  T* op = (T*)p.out + (int64_t)(q_bos + qrow) * p.o_row_stride + (int64_t)head * p.o_head_stride;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int d = dt * 32 + g * 8 + half * 4;
-      Pack<T, 4> o;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o.v[e] = (T)(o_acc[dt][g * 4 + e] * inv);
-      st_pack<T, 4>(op + d, o);
+  for (int rb = 0; rb < RBW; ++rb) {
+    const int qrow = row0 + rb * kRW + ql;
+    if (qrow >= q_len) continue;
+    const bool empty = l_run[rb] == 0.f || l_run[rb] != l_run[rb];
+    const float inv = empty ? 1.f : 1.f / l_run[rb];
+    if (p.lse != nullptr && half == 0) {
+      p.lse[(int64_t)head * p.total_q + q_bos + qrow] = empty ? INFINITY : m_run[rb] * 0.6931471805599453f + logf(l_run[rb]);
     }
+    T* op = (T*)p.out + (int64_t)(q_bos + qrow) * p.o_row_stride + (int64_t)head * p.o_head_stride;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = dt * 32 + g * 8 + half * 4;
+        Pack<T, 4> o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.v[e] = (T)(o_acc[rb][dt][g * 4 + e] * inv);
+        st_pack<T, 4>(op + d, o);
+      }
+  }
 }
 
-template <typename T, int D>
+template <typename T, int D, int RBW>
 int launch_pipe(const AttnArgs& a, dim3 grid, hipStream_t st) {
   constexpr int LDS_BYTES = 2 * 2 * kBN * 2 * D;
-  static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_varlen_pipe_kernel<T, D>),
+  static hipError_t attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_varlen_pipe_kernel<T, D, RBW>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (attr_err != hipSuccess) {
     fg_set_error("flash_attn_varlen_fwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(attr_err));
     return FG_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((attn_varlen_pipe_kernel<T, D>), grid, dim3(256), LDS_BYTES, st, a);
+  hipLaunchKernelGGL((attn_varlen_pipe_kernel<T, D, RBW>), grid, dim3(256), LDS_BYTES, st, a);
   return fg_check_launch("flash_attn_varlen_fwd");
 }

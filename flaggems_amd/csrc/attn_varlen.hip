@@ -64,12 +64,8 @@ struct AttnArgs {
   int nw, nst;        // waves per workgroup and LDS stages of the asynchronous kernel
   int page_tab_entries;  // block-table entries the asynchronous kernel keeps in LDS (0: read them from global memory)
   int use_fast;       // take the lean kernel (head dim 64/128, power-of-two pages, no ALiBi, no soft-cap)
-  int use_pair;       // take the head-pair kernel (lean kernel's conditions, head dim 128, even GQA ratio)
-  int* redo_flags;    // head-pair kernel: one flag per workgroup, set when the block has to be redone by the lean kernel
-  int redo_rows;      // lean kernel as the second pass: query rows per flagged block (0: ordinary launch)
-  int redo_grid_x;    // ... and the first grid dimension of the flagging launch
   int skip_single;    // mixed batch: sequences with one query token are left to the single-token kernel
-  int use_pipe;       // lean kernel's cases on its software-pipelined variant
+  int xcd_remap;      // lean kernel: workgroup order regrouped per XCD
 };
 
 // MFMA row slot s (0..31) of a K sub-tile -> key offset inside the 32-key sub-tile.
@@ -754,17 +750,13 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
   return launch_async_lp<T, D, RB, NW, NST, false>(a, grid, st);
 }
 
-#include "attn_fast.h"
 #include "attn_pipe.h"
-#include "attn_pair.h"
 #include "attn_decode.h"
 
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
-  if (a.use_pair) return launch_pair<T, 128>(a, grid, st);
-  if (a.use_fast && a.use_pipe) return D == 64 ? launch_pipe<T, 64>(a, grid, st) : launch_pipe<T, 128>(a, grid, st);
-  if (a.use_fast) return D == 64 ? launch_fast<T, 64>(a, grid, st) : launch_fast<T, 128>(a, grid, st);
+  if (a.use_fast) return D == 64 ? launch_pipe<T, 64, 1>(a, grid, st) : launch_pipe<T, 128, 1>(a, grid, st);
   if (a.use_async) {
     if (a.nw == 8) {
       switch (D) {
@@ -851,23 +843,6 @@ bool mixed_batch(const FgFlashParams& p) {
   if (fg_options().attn_mixed >= 0) return fg_options().attn_mixed != 0;
   return true;
 }
-// Head-pair kernel: applicable?  If so, its block shape and the size of its flag array.
-bool pair_plan(const FgFlashParams& p, int* hpb, int* rows, size_t* flag_bytes) {
-  if (p.Hk <= 0 || p.Hq % p.Hk != 0) return false;
-  const int ratio = p.Hq / p.Hk;
-  int page_shift = -1;
-  for (int sft = 4; sft < 31; ++sft)
-    if ((1 << sft) == p.page_size) page_shift = sft;
-  if (p.D != 128 || ratio % 2 != 0 || page_shift < 0 || p.max_seqlen_k > 128 * 64 || p.max_seqlen_q < 2 ||
-      p.alibi_slopes != nullptr || p.softcap > 0.f)
-    return false;
-  // Measured on MI355X the lean kernel is still ahead (see the header of attn_pair.h): opt-in for now.
-  if (fg_options().attn_kernel[0] != 'p') return false;
-  *hpb = ratio % 4 == 0 ? 4 : 2;
-  *rows = (8 / *hpb) * 32;
-  *flag_bytes = (size_t)fg_cdiv(p.max_seqlen_q, *rows) * (size_t)p.batch * (size_t)(p.Hq / *hpb) * sizeof(int);
-  return true;
-}
 }  // namespace
 
 extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int device) {
@@ -881,9 +856,6 @@ extern "C" size_t fg_flash_attn_workspace_bytes(const FgFlashParams* pp, int dev
   (void)device;
   DecodeArgs d;
   if (decode_setup(p, &d, mixed_batch(p))) return decode_workspace_bytes(p, d.splits);
-  int hpb = 0, rows = 0;
-  size_t flag_bytes = 0;
-  if (pair_plan(p, &hpb, &rows, &flag_bytes)) return flag_bytes;
   return 0;
 }
 
@@ -934,23 +906,17 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   // Kernel variant.  Head dims 32/48/64/80/96/112/128/192/256 take the asynchronous-tile kernel with 4 waves and
   // two LDS stages (measured fastest; the 8-wave variants stay selectable for head dims 64, 96 and 128);
   // everything else the register-staged kernel.
-  // FG_ATTN_KERNEL = "fast" | "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
+  // FG_ATTN_KERNEL = "fast" | "fn" | "sync" | "w4s2" | "w8s2" | "w8s3" overrides (debugging and measurement aid).
   a.use_async = (p.D == 32 || p.D == 48 || p.D == 64 || p.D == 80 || p.D == 96 || p.D == 112 || p.D == 128 || p.D == 192 ||
                  p.D == 256) ? 1 : 0;
   a.nw = 4;
   a.nst = 2;
-  // The lean kernel needs the 16 key rows a wave moves per tile inside one page, and keeps the page ids of
-  // at most 128 tiles in registers.
-  a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.max_seqlen_k <= 128 * 64 && p.alibi_slopes == nullptr &&
-               !(p.softcap > 0.f);
-  a.use_pair = 0;
-  a.use_pipe = 0;
-  a.redo_flags = nullptr;
-  a.redo_rows = 0;
-  a.redo_grid_x = 0;
+  // The lean kernel needs the 16 key rows a wave moves per tile inside one page.
+  a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.alibi_slopes == nullptr && !(p.softcap > 0.f);
+  a.xcd_remap = 1;
   if (const char* force = fg_options().attn_kernel; force[0] != 0) {
-    a.use_fast = a.use_fast && (force[0] == 'f' || force[0] == 'p' || force[0] == 'x');
-    a.use_pipe = force[0] == 'x';
+    a.use_fast = a.use_fast && force[0] == 'f';
+    if (force[0] == 'f' && force[1] == 'n') a.xcd_remap = 0;  // "fn...": the lean kernel in plain grid order
     if (force[0] == 's') a.use_async = 0;
     if (force[0] == 'w' && (p.D == 64 || p.D == 96 || p.D == 128)) {
       a.nw = force[1] == '8' ? 8 : 4;
@@ -977,25 +943,6 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.cap_in = p.softcap > 0.f ? p.softmax_scale / p.softcap : 0.f;
   a.cap_out_log2 = p.softcap * log2e;
   dim3 grid((unsigned)fg_cdiv(p.max_seqlen_q, a.rows_per_block), (unsigned)p.batch, (unsigned)(p.Hq / a.hpb));
-  {
-    // The head-pair kernel first, where it applies and the caller brought room for its flags; the lean kernel
-    // then runs as a second pass over the blocks it marked (normally none).
-    int hpb = 0, rows = 0;
-    size_t flag_bytes = 0;
-    if (a.use_fast && pair_plan(p, &hpb, &rows, &flag_bytes) && hpb == a.hpb && rows == 2 * a.rows_per_block &&
-        p.workspace != nullptr && p.workspace_bytes >= (int64_t)flag_bytes && fg_aligned(p.workspace, 4)) {
-      AttnArgs ap = a;
-      ap.use_pair = 1;
-      ap.rows_per_block = rows;
-      ap.redo_flags = (int*)p.workspace;
-      dim3 grid_p((unsigned)fg_cdiv(p.max_seqlen_q, rows), (unsigned)p.batch, (unsigned)(p.Hq / hpb));
-      const int rc = p.dtype == FG_F16 ? attn_dispatch<f16_t>(ap, grid_p, st) : attn_dispatch<bf16_t>(ap, grid_p, st);
-      if (rc != FG_OK) return rc;
-      a.redo_flags = (int*)p.workspace;
-      a.redo_rows = rows;
-      a.redo_grid_x = (int)grid_p.x;
-    }
-  }
   if (p.dtype == FG_F16) return attn_dispatch<f16_t>(a, grid, st);
   return attn_dispatch<bf16_t>(a, grid, st);
 }

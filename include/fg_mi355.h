@@ -248,8 +248,8 @@ typedef struct FgFlashParams {
   float softmax_scale;
   float softcap;            /* 0 = off */
   int32_t dtype;            /* FG_F16 or FG_BF16 */
-  void* workspace;          /* device scratch (split key ranges of single-token queries; block flags of the
-                               head-pair prefill kernel), may be NULL (see fg_flash_attn_workspace_bytes) */
+  void* workspace;          /* device scratch (split key ranges of single-token queries), may be NULL (see
+                               fg_flash_attn_workspace_bytes) */
   int64_t workspace_bytes;
 } FgFlashParams;
 

@@ -106,50 +106,42 @@ def test_flash_attn_mixed_batches(gpu, fg_env, dtype, Hq, Hk, D, block_size, mix
     check(gpu, [(1, 300), (40, 300), (1, 1000), (2, 77)], Hq, Hk, D, block_size, 512, dtype, window=(128, 0))
 
 
-# The head-pair kernel (two heads of a KV group per wave, software-pipelined tiles; opt-in through the
-# environment): same oracle, same tolerances.  The last case feeds scores that keep growing along the keys, so
-# that rows leave the exponent headroom above their fixed softmax reference and the blocks are handed to the
-# lean kernel by the second pass.
+# The lean kernel (head dim 64 / 128, power-of-two pages): its reference maximum moves lazily and is subtracted
+# inside the matrix pipe, so feed it scores that keep growing along the keys (the reference has to move many
+# times, by large steps), rows that see their first key late (windows), sequences longer than the 128-tile window
+# of page ids it keeps in registers, and the plain grid order next to the XCD-grouped one.
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("Hq,Hk", [(8, 2), (4, 2), (6, 3)])
-def test_flash_attn_head_pair_kernel(gpu, fg_env, dtype, Hq, Hk):
-    fg_env.setenv("FG_ATTN_KERNEL", "pair")
-    check(gpu, [(1, 1328), (5, 18), (129, 463), (70, 70)], Hq, Hk, 128, 16, 512, dtype)
-    check(gpu, [(200, 200), (64, 64), (65, 65), (300, 1000)], Hq, Hk, 128, 32, 1024, dtype)
-    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=False)
-    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=True, window=(50, 0))
-    check(gpu, [(7, 300), (130, 130), (64, 200)], Hq, Hk, 128, 16, 512, dtype, causal=False, window=(20, 30))
-    check(gpu, [(300, 200), (130, 130), (64, 5)], Hq, Hk, 128, 16, 512, dtype)
-    check(gpu, [(2000, 2000), (100, 3000)], Hq, Hk, 128, 16, 1024, dtype)
-
-
-@pytest.mark.parametrize("dtype,grow", [(torch.bfloat16, 0.02), (torch.float16, 0.004), (torch.bfloat16, 0.05)])
-def test_flash_attn_head_pair_second_pass(gpu, fg_env, dtype, grow):
-    fg_env.setenv("FG_ATTN_KERNEL", "pair")
-    dev, Hq, Hk, D, bs, nblk = gpu, 8, 2, 128, 16, 512
-    qlens, klens = [300, 64], [300, 700]
+@pytest.mark.parametrize("D,Hq,Hk", [(128, 8, 2), (64, 4, 4), (128, 3, 1)])
+def test_flash_attn_lean_kernel_reference_moves(gpu, dtype, D, Hq, Hk):
     torch.manual_seed(5)
-    q = torch.ones(sum(qlens), Hq, D, dtype=dtype, device=dev)
-    kc = torch.zeros(nblk, bs, Hk, D, dtype=dtype, device=dev)
-    vc = torch.randn(nblk, bs, Hk, D, dtype=dtype, device=dev)
-    pages = (max(klens) + bs - 1) // bs
-    bt = torch.randperm(nblk)[:2 * pages].reshape(2, pages).to(torch.int32).to(dev)
-    for b in range(2):
-        for j in range(pages):
-            pos = (j * bs + torch.arange(bs, device=dev)).float()
-            kc[bt[b, j].long()] = (pos * grow).to(dtype)[:, None, None].expand(bs, Hk, D)
-    cu = torch.tensor([0] + qlens, dtype=torch.int32, device=dev).cumsum(0, dtype=torch.int32)
-    sk = torch.tensor(klens, dtype=torch.int32, device=dev)
+    lens = [(200, 900), (64, 64), (33, 700)]
+    q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, lens, Hq, Hk, D, 16, 512, dtype)
+    # keys whose projection on a fixed direction grows with the slot index: scores rise along every sequence
+    ramp = torch.linspace(0, 6, kc.shape[0] * kc.shape[1], device=gpu).view(kc.shape[0], kc.shape[1], 1, 1)
+    kc = (kc.float() * 0.3 + ramp * torch.sign(torch.randn(1, 1, 1, D, device=gpu))).to(dtype)
+    q = (q.float().abs() * 0.5).to(dtype)
     scale = D ** -0.5
     out, lse = flag_gems.ops.flash_attn_varlen_func(q, kc, vc, max(qlens), cu, max(klens), seqused_k=sk, softmax_scale=scale,
                                                     causal=True, block_table=bt, return_softmax_lse=True)
     ref, rlse = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, compute_dtype=torch.float32, return_lse=True)
     torch.testing.assert_close(out.float().cpu(), ref, atol=ATOL, rtol=RTOL)
-    torch.testing.assert_close(lse.cpu(), rlse, atol=1e-2, rtol=1e-3)
+    torch.testing.assert_close(lse.cpu(), rlse, atol=2e-2, rtol=2e-3)
 
 
-# Single-token queries: the streaming kernel with split key ranges (head dim 64/128, pages >= 16) and the
-# cases it must hand back to the general kernels (small pages, left window, ALiBi, other head dims).
+@pytest.mark.parametrize("order", [None, "fn"])
+def test_flash_attn_lean_kernel_long_sequences_and_grid_orders(gpu, fg_env, order):
+    if order is None:
+        fg_env.delenv("FG_ATTN_KERNEL")
+    else:
+        fg_env.setenv("FG_ATTN_KERNEL", order)
+    # 8192 keys is 128 tiles: beyond it the page-id window is re-read; page 16 and page 128
+    check(gpu, [(40, 9000), (600, 17000), (3, 8193), (130, 130)], 4, 2, 128, 16, 2048, torch.bfloat16)
+    check(gpu, [(257, 12345), (64, 64)], 8, 8, 64, 128, 128, torch.float16)
+    check(gpu, [(300, 9000)], 4, 1, 128, 16, 1024, torch.bfloat16, causal=False)
+    check(gpu, [(500, 10000), (700, 700)], 4, 2, 128, 32, 512, torch.bfloat16, window=(300, 0))
+    check(gpu, [(1, 1328), (5, 18), (129, 463), (70, 70)], 8, 2, 128, 16, 512, torch.bfloat16)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hk,D,block_size", [(32, 8, 128, 16), (8, 8, 64, 32), (16, 2, 64, 16), (32, 32, 128, 64),
                                                  (4, 1, 128, 256), (8, 2, 128, 8), (8, 2, 96, 16)])
@@ -401,5 +393,8 @@ def test_decoder_layer_pipeline(gpu):
     gur = r(yr @ wgu.float().cpu().t())
     actr = r(O.silu_and_mul(gur[:, :F], gur[:, F:]))
     outr = r(actr @ wd.float().cpu().t()) + rr
-    torch.testing.assert_close(out.float().cpu(), outr, atol=5e-2, rtol=5e-2)
+    # (the last GEMM's bf16 result, up to ~8 with an ulp of 0.06, meets a residual of opposite sign: one ulp of it
+    # can be the whole difference at an output near zero)
+    torch.testing.assert_close(out.float().cpu(), outr, atol=0.1, rtol=5e-2)
+    assert (out.float().cpu() - outr).abs().mean().item() < 0.01
     torch.testing.assert_close(kc.float().cpu(), kcr.float(), atol=2e-2, rtol=2e-2)
