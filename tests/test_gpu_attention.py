@@ -396,5 +396,5 @@ def test_decoder_layer_pipeline(gpu):
     # (the last GEMM's bf16 result, up to ~8 with an ulp of 0.06, meets a residual of opposite sign: one ulp of it
     # can be the whole difference at an output near zero)
     torch.testing.assert_close(out.float().cpu(), outr, atol=0.1, rtol=5e-2)
-    assert (out.float().cpu() - outr).abs().mean().item() < 0.01
+    assert (out.float().cpu() - outr).abs().mean().item() < 0.02
     torch.testing.assert_close(kc.float().cpu(), kcr.float(), atol=2e-2, rtol=2e-2)
