@@ -197,6 +197,10 @@ __global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kern
   const uint32_t lane_c0 = (uint32_t)((lane_pos ^ swz<CPR>(wave * IPW * KPI + lane_key)) * 16);
   const uint32_t lane_row_k = (uint32_t)(lane_key * (int)p.k_row_stride * 2);
   const uint32_t lane_row_v = (uint32_t)(lane_key * (int)p.v_row_stride * 2);
+  // byte strides (the host admits the kernel only when they fit 31 bits)
+  const uint32_t k_page_b = (uint32_t)p.k_page_stride * 2u, v_page_b = (uint32_t)p.v_page_stride * 2u;
+  const uint32_t k_row_b = (uint32_t)p.k_row_stride * 2u, v_row_b = (uint32_t)p.v_row_stride * 2u;
+  const uint32_t wave_key0 = (uint32_t)(wave * (IPW * KPI));
   const int last_page = k_len > 0 ? (k_len - 1) >> page_shift : 0;
   // page ids of this wave's rows in tiles pg_base + l (pg_cache0) and pg_base + 64 + l (pg_cache1), lane l
   int pg_cache0, pg_cache1, pg_base;
@@ -208,6 +212,9 @@ __global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kern
     pg1 = pg1 < last_page ? pg1 : last_page;
     pg_cache0 = btab[pg0];
     pg_cache1 = btab[pg1];
+    // the ids are consumed here, so that the wait for them stays on this (rare) path: left pending, the compiler
+    // would wait for every outstanding tile copy wherever the two paths meet again
+    asm volatile("v_mov_b32 %0, %0\n\tv_mov_b32 %1, %1" : "+v"(pg_cache0), "+v"(pg_cache1));
   };
   load_page_window(0);
   // one operand tile (K: is_v = 0, V: is_v = 1) of key tile n_min + t into `slot` of its ring
@@ -216,38 +223,41 @@ __global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kern
     const int nb = n_min + t;
     char* dst = lds + (IS_V ? 2 * OPB : 0) + slot * OPB + wave * (IPW * 1024);
     const char* base = IS_V ? vbase : kbase;
-    const int64_t page_stride = IS_V ? p.v_page_stride : p.k_page_stride;
-    const int64_t row_stride = IS_V ? p.v_row_stride : p.k_row_stride;
+    const uint32_t page_b = IS_V ? v_page_b : k_page_b;
+    const uint32_t row_b = IS_V ? v_row_b : k_row_b;
     if (nb * kBN + kBN <= k_len) {
-      // full tile: every key exists; one scalar row base per instruction, one 32-bit lane offset
-      // tiles are requested in the order V(1), K(2), V(2), K(3), ...: a window that starts one tile below the
-      // request that overran it still holds the V tile that follows
+      // Full tile: every key exists.  One scalar row base per tile, 32-bit scalar arithmetic but for the product
+      // with the page id; instruction j lands 1024 bytes further in LDS through its immediate offset, which the
+      // hardware adds to the global address as well, so the scalar step between instructions is the distance of
+      // their rows less those 1024 bytes (never negative: KPI rows are at least 1024 bytes apart).
+      // Tiles are requested in the order V(1), K(2), V(2), K(3), ...: a window that starts one tile below the
+      // request that overran it still holds the V tile that follows.
       if (t - pg_base >= 128) load_page_window(t - 1);
-      const int tl = t - pg_base;
-      const int64_t page = __builtin_amdgcn_readlane(tl < 64 ? pg_cache0 : pg_cache1, tl & 63);
-      const int key = nb * kBN + wave * (IPW * KPI);
-      const int slot_in_page = key & page_mask;
-      const char* rp = base + (page * page_stride + (int64_t)slot_in_page * row_stride) * 2;
-#pragma unroll
-      for (int j = 0; j < IPW; ++j) {
-        // kept opaque so that the address stays "scalar base + 32-bit lane offset" (the compiler would otherwise
-        // precompute a 64-bit lane offset per instruction and operand and hold sixteen register pairs for them)
+      const uint32_t tl = (uint32_t)(t - pg_base);
+      const uint32_t page = (uint32_t)__builtin_amdgcn_readlane(tl < 64 ? pg_cache0 : pg_cache1, (int)(tl & 63));
+      const uint32_t slot_in_page = ((uint32_t)(nb * kBN) + wave_key0) & (uint32_t)page_mask;
+      const char* rp = base + ((uint64_t)page * page_b + (uint64_t)(slot_in_page * row_b));
+      const uint32_t step_b = (uint32_t)KPI * row_b - 1024u;
+      a_static_for<0, IPW>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        // the lane offset is kept opaque so that the address stays "scalar base + 32-bit lane offset" (the
+        // compiler would otherwise precompute a 64-bit lane offset per instruction and operand)
         uint32_t c0 = lane_c0;
         asm volatile("" : "+v"(c0));
         const uint32_t voff = (IS_V ? lane_row_v : lane_row_k) + (c0 ^ (uint32_t)(j * 16));
-        __builtin_amdgcn_global_load_lds(FG_GLBP(rp + (int64_t)j * KPI * row_stride * 2 + voff), FG_LDSP(dst + j * 1024), 16, 0, 0);
-      }
+        __builtin_amdgcn_global_load_lds(FG_GLBP(rp + (uint64_t)((uint32_t)j * step_b) + voff), FG_LDSP(dst), 16, j * 1024, 0);
+      });
     } else {
       // partial tile: keys past the end are clamped to the last one (their scores are masked)
 #pragma unroll
       for (int j = 0; j < IPW; ++j) {
         int key = nb * kBN + (wave * IPW + j) * KPI + lane_key;
         key = key < k_len ? key : k_len - 1;
-        const int64_t page = btab[key >> page_shift];
-        const int slot_in_page = key & page_mask;
+        const uint32_t page = (uint32_t)btab[key >> page_shift];
+        const uint32_t slot_in_page = (uint32_t)key & (uint32_t)page_mask;
         uint32_t c0 = lane_c0;
         asm volatile("" : "+v"(c0));
-        const char* rp = base + ((page * page_stride + (int64_t)slot_in_page * row_stride) * 2 + (c0 ^ (uint32_t)(j * 16)));
+        const char* rp = base + ((uint64_t)page * page_b + (uint64_t)(slot_in_page * row_b + (c0 ^ (uint32_t)(j * 16))));
         __builtin_amdgcn_global_load_lds(FG_GLBP(rp), FG_LDSP(dst + j * 1024), 16, 0, 0);
       }
     }
@@ -426,13 +436,26 @@ __global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kern
     tmax_a[rb] = tm;
     tmax_b[rb] = -INFINITY;
   };
-  auto needs_mask = [&](int h, int rb) {
-    const int key0 = key_base + h * kHB;
+  // half tile h of row block rb needs the mask pass from mask_from[rb] on (diagonal, right window edge, partial
+  // last tile) and below mask_below[rb] (left window edge)
+  int mask_from[RBW], mask_below[RBW];
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb) {
     const int r_first = row0 + rb * kRW;
     const int r_last = (r_first + kRW - 1 < q_len ? r_first + kRW - 1 : q_len - 1);
-    return (key0 + kHB > k_len) || (a.has_right && key0 + kHB - 1 > r_first + shift + a.right_off_w) ||
-           (a.has_left && key0 < r_last + shift - a.left_off_w);
-  };
+    // key0 + 32 > k_len  <=>  h > (k_len - key_base - 32) / 32 ;  key0 + 31 > bound  <=>  h > (bound - 31 - key_base) / 32
+    int from = (k_len - key_base - kHB) < 0 ? 0 : (k_len - key_base - kHB) / kHB + 1;
+    if (a.has_right) {
+      const int bnd = r_first + shift + a.right_off_w - (kHB - 1) - key_base;
+      const int f2 = bnd < 0 ? 0 : bnd / kHB + 1;
+      from = from < f2 ? from : f2;
+    }
+    mask_from[rb] = from;
+    // key0 < r_last + shift - left  <=>  h < ceil((r_last + shift - left - key_base) / 32)
+    const int lb = r_last + shift - a.left_off_w - key_base;
+    mask_below[rb] = a.has_left ? (lb <= 0 ? 0 : (lb + kHB - 1) / kHB) : 0;
+  }
+  auto needs_mask = [&](int h, int rb) { return h >= mask_from[rb] || h < mask_below[rb]; };
   // The scores in buffer BUF are relative to the reference m_run they were scored with.  Where a lane finds one
   // more than 2^8 above it (or the row has no reference yet and sees its first key), the row's reference moves to
   // the new maximum: the waiting scores, O and the row sum are shifted by the difference and -m is split anew.

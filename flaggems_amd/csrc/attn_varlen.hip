@@ -912,7 +912,11 @@ extern "C" int fg_flash_attn_varlen_fwd(const FgFlashParams* pp, void* stream) {
   a.nw = 4;
   a.nst = 2;
   // The lean kernel needs the 16 key rows a wave moves per tile inside one page.
-  a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.alibi_slopes == nullptr && !(p.softcap > 0.f);
+  // (and computes tile addresses with 32-bit byte strides)
+  auto fits31 = [](int64_t elems) { return elems >= 0 && elems < ((int64_t)1 << 30); };
+  a.use_fast = (p.D == 128 || p.D == 64) && a.page_shift >= 4 && p.alibi_slopes == nullptr && !(p.softcap > 0.f) &&
+               fits31(p.k_page_stride) && fits31(p.v_page_stride) && fits31(p.k_row_stride * p.page_size) &&
+               fits31(p.v_row_stride * p.page_size);
   a.xcd_remap = 1;
   if (const char* force = fg_options().attn_kernel; force[0] != 0) {
     a.use_fast = a.use_fast && force[0] == 'f';
