@@ -119,8 +119,13 @@ def main():
     # same counters read for a plain 512 MiB copy (profiles/hbm_traffic_*.txt hold the runs and their commands)
     TRAFFIC = {
         "softmax_c2": 1073780000,
-        "mm_c3a_8192": 1771500000,
-        "flash_attn_c4": 1835830000,
+        "fused_add_rms_norm_c1": 134330000,
+        "fused_add_rms_norm_c1_fp32": 268600000,
+        "mm_c3a_8192": 1768300000,
+        "mm_c3b_skinny": 122520000,
+        "addmm_c3c": 713990000,
+        "flash_attn_c4": 785740000,
+        "flash_attn_decode": 1075240000,
     }
 
     cores = torch.get_num_threads()
