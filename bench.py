@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X-native FlagGems operator path on ONE GPU.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu] [--settle-ms T]
 
 A "step" is one pass of one operator over one batch of synthetic input that is already resident in
 HBM.  The headline workload (the JSON line's metric/value) is the softmax configuration of
@@ -11,8 +11,10 @@ entries at -inf.  Its 1 GiB of algorithmic traffic (read + write of one tensor) 
 the three GEMMs, varlen GQA prefill attention, the decoder layer) are measured in the same run and
 reported under "configs", each with its own roofline entry.
 
-Timing: W untimed warm-up steps, then exactly K steps bracketed by torch.cuda.synchronize() on both
-sides (one GPU, so the barrier is the synchronize).  ms_per_step / value come from the wall clock
+Timing: an untimed run-in of T ms of the workload's own steps (the part throttles for ~40 ms of work after
+any pause, see timed() below; --settle-ms 0 switches it off and shows that transient instead of the
+sustained rate), W untimed warm-up steps, then exactly K steps bracketed by torch.cuda.synchronize() on
+both sides (one GPU, so the barrier is the synchronize).  ms_per_step / value come from the wall clock
 around the K steps; roofline.achieved comes from HIP events recorded on the stream the kernels are
 launched on (torch's current stream) around the same K steps.
 
@@ -52,6 +54,8 @@ def parse_args():
     ap.add_argument("--workload", default="softmax_c2")
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--settle-ms", type=float, default=200.0,
+                    help="untimed run-in of each workload before its warm-up steps, in ms of its own steps (0: none)")
     return ap.parse_args()
 
 
@@ -80,7 +84,23 @@ def main():
 
     # ------------------------------------------------------------------------------------------
     def timed(run, steps, warmup):
-        """(wall ms per step, event ms per step) for `steps` calls of run(i)."""
+        """(wall ms per step, event ms per step) for `steps` calls of run(i).
+
+        Run-in: after any pause of the GPU (10 ms is enough: the set-up of a workload, the CPU baseline before
+        it) the part's power management lets two launches through at full rate, throttles the next ones by
+        20-25 % and recovers over the following ~40 ms of continuous work (a bf16 GEMM of 8192^3, TFLOP/s per
+        launch: 1300 1310 1120 990 1000 1080 1110 1140 ... 1335 from the 40th launch on; the vendor library's
+        GEMM traces the same curve).  A few warm-up steps of a millisecond each end inside that trough, so each
+        workload first repeats its own step for --settle-ms of wall time, untimed; the warm-up steps and the
+        timed steps follow without a pause."""
+        if args.settle_ms > 0:
+            t_end = time.perf_counter() + args.settle_ms * 1e-3
+            i = 0
+            while time.perf_counter() < t_end:
+                for _ in range(4):
+                    run(i)
+                    i += 1
+                torch.cuda.synchronize()
         for i in range(warmup):
             run(i)
         torch.cuda.synchronize()
@@ -587,6 +607,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",

@@ -141,7 +141,8 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
 // Main loop over the K steps [kb0, kb0 + nk) of tile (tm, tn); `finish` receives the accumulators.
 // NS = number of LDS stages: K step kb lives in stage kb % NS and is requested NS - 1 steps ahead.
 template <typename T, bool B_KC, int BM, int BN, int NS, typename F>
-__device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish) {
+__device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish,
+                                                  int krot = 0) {
   static_assert(sizeof(T) == 2, "16-bit element types");
   typedef typename Mfma<T>::Frag Frag;
   constexpr int TM = BM / 64, TN = BN / 64;        // MFMA sub-tiles per wave
@@ -196,14 +197,20 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   char* const dma_a = lds + wave_s * (NA * 1024);
   char* const dma_b = lds + A_OPB + wave_s * (NB * 1024);
-  auto issue = [&](int kb, auto jc) {
+  // K step kb of the loop reads K step wrap(kb) of the operands: a launch may walk K from a rotated start (krot), which
+  // only permutes the order of the sum
+  auto wrap = [&](int kb) {
+    const int k = kb + krot;
+    return k >= nk ? k - nk : k;
+  };
+  auto issue = [&](int kb, int kk, auto jc) {
     constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
     char* l = (IS_A ? dma_a : dma_b) + stage_off(kb) + (jj >> 2) * 4096;
     const char* gp;
-    if constexpr (IS_A) gp = a_src[jj] + (int64_t)kb * kDmaRowB;
-    else gp = b_src[jj] + (int64_t)kb * b_step;
+    if constexpr (IS_A) gp = a_src[jj] + (int64_t)kk * kDmaRowB;
+    else gp = b_src[jj] + (int64_t)kk * b_step;
     __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
   };
 
@@ -271,10 +278,10 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // ---- prologue: K steps 0 .. NS-2, and the head of step NS-1 (the part sub-step 3 of the step before would issue)
   static_for<0, NS - 1>([&](auto sc) {
     constexpr int s = decltype(sc)::value;
-    if (s < nk) static_for<0, NDMA>([&](auto jc) { issue(s, jc); });
+    if (s < nk) static_for<0, NDMA>([&](auto jc) { issue(s, wrap(s), jc); });
   });
   if (nk >= NS) {
-    static_for<0, HALF>([&](auto jc) { issue(NS - 1, jc); });
+    static_for<0, HALF>([&](auto jc) { issue(NS - 1, wrap(NS - 1), jc); });
     FGK_WAIT_VM(NDMA * (NS - 2) + HALF);  // K step 0 has landed
   } else {
     FGK_WAIT_VM(0);
@@ -292,6 +299,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
     constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
     constexpr int LATER = decltype(later_c)::value;
+    const int kk_head = wrap(kb + NS), kk_tail = wrap(kb + NS - 1);
     static_for<0, 4>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
       constexpr int cur = s & 1, nxt = cur ^ 1;
@@ -303,8 +311,8 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
           if constexpr (s < 3) read_one(kb, IntC<s + 1>{}, xc, nxt);
           else read_one(kb + 1, IntC<0>{}, xc, nxt);
         }
-        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + NS, IntC<x>{});
-        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + NS - 1, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
+        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + NS, kk_head, IntC<x>{});
+        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + NS - 1, kk_tail, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       if constexpr (s == 2) {
@@ -338,8 +346,13 @@ __global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ?
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
-  dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, 0, (int)(g.K / kDmaBK),
-                                     [&](f32x16 (&acc)[BM / 64][BN / 64]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); });
+  const int nk = (int)(g.K / kDmaBK);
+  // K-rotated start per XCD (workgroups go to the XCDs round-robin by id): the eight XCDs then read eight different
+  // column ranges of the operands at any one time, which spreads the requests over the memory channels when the
+  // leading dimensions are large powers of two; the tiles of one XCD stay in step and keep sharing panels in its L2
+  const int krot = g.k_stagger ? (int)((blockIdx.x & 7u) * (unsigned)nk / 8u) : 0;
+  dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, 0, nk,
+                                     [&](f32x16 (&acc)[BM / 64][BN / 64]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); }, krot);
 }
 
 // Stream-K over 128x128 tiles with the main loop above: the (tile, K step) units, tile-major, are dealt

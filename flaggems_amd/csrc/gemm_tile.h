@@ -53,6 +53,7 @@ struct GemmArgs {
   float alpha, beta;
   int tiles_m, tiles_n;
   int tile_base;        // first tile id of a data-parallel launch (tiles below it belong to stream-K)
+  int k_stagger;        // direct-to-LDS data-parallel kernels: every XCD starts its K loop at a different eighth of K
   // stream-K (unused by the data-parallel launch)
   float* partials;      // [workers][2][BM*BN] fp32
   unsigned* tickets;    // [kMaxWorkers], zero between launches
