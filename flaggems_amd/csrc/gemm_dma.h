@@ -2,7 +2,7 @@
 //
 // The kernel for aligned 16-bit problems.  A BM x BN output tile per workgroup (256x256, 256x128 or
 // 128x128, chosen on the host by how well the tile count fills the machine), 4 waves in a 2x2 grid,
-// each wave a (BM/2) x (BN/2) sub-tile held as MFMA 32x32 accumulators (256 accumulator registers per
+// each wave a (BM/2) x (BN/2) sub-tile held as MFMA 16x16 accumulators (256 accumulator registers per
 // lane for the largest tile).  The description below uses the 256x256 numbers.
 //
 // Data movement.  Each K step covers 64 elements = one full 128-byte cache line per tile row.  The
@@ -14,26 +14,29 @@
 //
 //   A (K contiguous), and B when it is K contiguous (B = W^T, "NT"):
 //     stage layout [row][128 B]; chunk c of row r sits at position c ^ ((r >> 1) & 7).  A fragment
-//     (8 consecutive k of one row per lane) is one ds_read_b128; the 16 rows a quarter-wave reads
-//     fall into 16 different 16-byte bank groups.
+//     (16 rows x 32 k: 8 consecutive k of one row per lane) is one ds_read_b128; the 16 rows a
+//     quarter-wave reads fall into 16 different 16-byte bank groups.
 //   B when it is N contiguous (row-major [K,N], "NN"):
 //     stage layout [k][512 B] (the 256 columns of the tile); chunk c of row k sits at position
 //     c ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)).  The fragment is produced by two
 //     ds_read_b64_tr_b16, which transpose 4 k-rows x 4 column groups among 16 lanes while reading.
 //
-// Schedule.  The K step is cut into four sub-steps of one MFMA K (16): sub-step s issues its 16
-// MFMAs on fragment set s&1 while the reads for sub-step s+1 fill the other set, one LDS read per
-// MFMA.  Sub-step 3 already reads the first fragments of the next stage, so the MFMA pipe does not
-// drain at a stage boundary.  One barrier per K step, after sub-step 2: by then this wave has issued
+// Schedule.  The matrix instruction is v_mfma_f32_16x16x32: a wave's 128 x 128 tile is 8 x 8 sub-tiles and
+// a K step two k halves of 64 MFMAs.  The K step is cut into four quarters of 32 MFMAs, (k half, half of
+// the A sub-tiles): a quarter issues its MFMAs while the fragments of the next quarter are read (4 A
+// fragments, and the 8 B fragments of the next k half behind every second quarter), at most one LDS read
+// or DMA per MFMA.  Quarter 3 already reads the first fragments of the next stage, so the MFMA pipe does
+// not drain at a stage boundary.  One barrier per K step, after quarter 2: by then this wave has issued
 // and completed every read of the current stage (the stage may be refilled) and every DMA it issued
 // for the next stage has landed (vmcnt(0)).  The refill for stage kb+2 is issued right behind that
-// barrier, spread over sub-step 3 and sub-step 0 of the next step (one DMA per MFMA), which leaves
-// it two to three sub-steps to land.  The compiler's own scheduling is pinned with sched_barrier
+// barrier, spread over quarter 3 and quarter 0 of the next step, which leaves it two to three quarters
+// to land.  The compiler's own scheduling is pinned with sched_barrier
 // after every MFMA group; it keeps no counters for the DMA writes, hence the explicit waits.
 //
 // The MFMA operands are swapped (B fragment first), so a lane's accumulator registers hold 4
-// consecutive output columns of one output row; after packing to 16 bits, two v_permlane32_swap
-// give every lane 8 consecutive columns and the tile is written with 16-byte stores.
+// consecutive output columns of one output row; after packing to 16 bits, v_permlane16_swap between
+// two neighbouring sub-tiles gives every lane 8 consecutive columns and the tile is written with
+// 16-byte stores.
 //
 // Preconditions (checked on the host): 16-bit type; A K-contiguous; B K- or N-contiguous; K a
 // multiple of 64; N a multiple of 8; operand base pointers and row strides multiples of 16 bytes;
@@ -72,21 +75,58 @@ template <int OFF> __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t a
 }
 // Waits for every outstanding LDS read; tied to the registers the inline-asm reads wrote so that
 // nothing consuming them can be placed ahead of the wait.
-__device__ __forceinline__ void lds_wait_tied(u32x4 (&r)[4]) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+template <int N> __device__ __forceinline__ void lds_wait_tied(u32x4 (&r)[N]) {
+  static_assert(N == 2 || N == 3 || N == 4 || N == 8, "fragments per set");
+  if constexpr (N == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]));
+  if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]));
+  if constexpr (N >= 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+  if constexpr (N == 8) asm volatile("" : "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
 }
-// X.upper-half-lanes <-> Y.lower-half-lanes, for two register pairs at once
-__device__ __forceinline__ void swap_halves2(unsigned& x0, unsigned& y0, unsigned& x1, unsigned& y1) {
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+// rows of 16 lanes: X.row1 <-> Y.row0 and X.row3 <-> Y.row2, for two register pairs at once
+__device__ __forceinline__ void swap_rows16x2(unsigned& x0, unsigned& y0, unsigned& x1, unsigned& y1) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
                : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
+}
+
+// The matrix instruction of these kernels: 16x16 outputs over 32 k.  Under the part's power limit it sustains
+// ~14 % more than the 32x32x16 shape on the same data (2.0 against 1.78 PFLOP/s in a loop of nothing else): it
+// touches its accumulators half as often per flop.
+// The instruction is written as asm with the accumulator tied to itself in the AGPR file: a wave's 64 accumulator
+// tiles fill that file exactly, and left to the register allocator some of them travel between the two files
+// inside the loop (a v_accvgpr_read waits for the matrix pipe to drain: ~100 cycles each).  The compiler does not
+// see a matrix instruction here, so the code that reads accumulators afterwards waits for the pipe itself
+// (mfma_drain).
+template <typename T> struct MfmaK32;
+template <> struct MfmaK32<bf16_t> {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ void mma(Frag a, Frag b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+template <> struct MfmaK32<f16_t> {
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ void mma(Frag a, Frag b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+// Waits out the matrix pipe, then passes every accumulator through an empty asm: volatile asm statements keep
+// their order, so no read of an accumulator can be scheduled ahead of the wait.
+template <int TM, int TN> __device__ __forceinline__ void mfma_drain(f32x4 (&acc)[TM][TN]) {
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
 }
 
 // Epilogue of one tile (the host guarantees: C rows 16-byte aligned with unit column stride, N a multiple
 // of 8, bias -- if any -- with unit column stride and 8-byte aligned rows).  acc is in the layout the
-// main loop leaves: operands swapped, so a lane owns 4 consecutive output columns per register group.
+// main loop leaves: operands swapped, so lane (r = lane % 16, g = lane / 16) of sub-tile (i, j) owns output
+// row 16 i + r and the 4 consecutive columns 16 j + 4 g ...
 template <typename T, int BM, int BN>
-__device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int tn, f32x16 (&acc)[BM / 64][BN / 64]) {
-  constexpr int TM = BM / 64, TN = BN / 64, WTM = BM / 2, WTN = BN / 2;
+__device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int tn, f32x4 (&acc)[BM / 32][BN / 32]) {
+  constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 16, TN = WTN / 16;
+  static_assert(TN % 2 == 0, "sub-tiles are stored in pairs");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int row0 = tm * BM, col0 = tn * BN;
@@ -95,45 +135,40 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
   const T* bias = (const T*)g.bias;
   const float alpha = g.alpha, beta = g.beta;
   const bool scale = alpha != 1.0f;
-  const int lr = lane & 31, lh = lane >> 5;
+  const int lr = lane & 15, lg = lane >> 4;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int64_t r = row0 + wm * WTM + i * 32 + lr;
+    const int64_t r = row0 + wm * WTM + i * 16 + lr;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int cbase = col0 + wn * WTN + j * 32;
-      // element e of this lane: row r, column cbase + (e/4)*8 + lh*4 + e%4
-      if (bias != nullptr) {
+    for (int jp = 0; jp < TN / 2; ++jp) {
+      unsigned pk[2][2];
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          const int c = cbase + gq * 8 + lh * 4;
+      for (int jj = 0; jj < 2; ++jj) {
+        const int j = 2 * jp + jj;
+        const int c = col0 + wn * WTN + j * 16 + lg * 4;
+        if (bias != nullptr) {
           typedef T T4 __attribute__((ext_vector_type(4)));
           T4 t = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
           if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
 #pragma unroll
-          for (int t4 = 0; t4 < 4; ++t4)
-            acc[i][j][gq * 4 + t4] = acc[i][j][gq * 4 + t4] * alpha + (float)t[t4] * beta;
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = acc[i][j][e] * alpha + (float)t[e] * beta;
+        } else if (scale) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][e] *= alpha;
         }
-      } else if (scale) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] *= alpha;
+        for (int d = 0; d < 2; ++d) {
+          typedef T T2 __attribute__((ext_vector_type(2)));
+          const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
+          pk[jj][d] = __builtin_bit_cast(unsigned, t);
+        }
       }
-      unsigned pk[8];
-#pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        typedef T T2 __attribute__((ext_vector_type(2)));
-        const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
-        pk[d] = __builtin_bit_cast(unsigned, t);
-      }
-#pragma unroll
-      for (int gp = 0; gp < 2; ++gp) {
-        // register groups 2gp (X) and 2gp+1 (Y): after X.upper <-> Y.lower the lower half-wave owns
-        // the 8 columns of group 2gp, the upper half-wave those of group 2gp+1
-        unsigned x0 = pk[4 * gp], x1 = pk[4 * gp + 1], y0 = pk[4 * gp + 2], y1 = pk[4 * gp + 3];
-        swap_halves2(x0, y0, x1, y1);
-        const int c = cbase + (2 * gp + lh) * 8;
-        if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
-      }
+      // sub-tiles 2jp (X) and 2jp+1 (Y): after X.odd rows <-> Y.even rows of 16 lanes, an even lane group g owns
+      // columns 4g .. 4g+7 of sub-tile 2jp and an odd one columns 4(g-1) .. 4(g-1)+7 of sub-tile 2jp+1
+      unsigned x0 = pk[0][0], x1 = pk[0][1], y0 = pk[1][0], y1 = pk[1][1];
+      swap_rows16x2(x0, y0, x1, y1);
+      const int c = col0 + wn * WTN + (2 * jp + (lg & 1)) * 16 + (lg & 2) * 4;
+      if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
     }
   }
 }
@@ -144,18 +179,19 @@ template <typename T, bool B_KC, int BM, int BN, int NS, typename F>
 __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish,
                                                   int krot = 0) {
   static_assert(sizeof(T) == 2, "16-bit element types");
-  typedef typename Mfma<T>::Frag Frag;
-  constexpr int TM = BM / 64, TN = BN / 64;        // MFMA sub-tiles per wave
+  typedef typename MfmaK32<T>::Frag Frag;
   constexpr int WTM = BM / 2, WTN = BN / 2;        // wave tile
+  constexpr int TM = WTM / 16, TN = WTN / 16;      // 16x16 sub-tiles per wave
+  constexpr int HM = TM / 2;                       // A sub-tiles of one quarter step
   constexpr int A_OPB = BM * kDmaRowB;             // A tile, one stage
   constexpr int B_OPB = BN * kDmaRowB;             // B tile, one stage (64 k-rows of BN*2 bytes when N-contiguous)
   constexpr int STAGEB = A_OPB + B_OPB;
   constexpr int NA = BM / 32, NB = BN / 32;        // DMA instructions per wave, operand and stage
   constexpr int NDMA = NA + NB, HALF = NDMA / 2;
-  constexpr int NMF = TM * TN, NRD = TM + TN;      // MFMAs and fragment reads per sub-step
+  constexpr int NMF = HM * TN;                     // MFMAs per quarter step
   constexpr int RBB = BN * 2;                      // N-contiguous B: bytes per k-row of the tile
   constexpr int CPRB = RBB / 16, RPI = 1024 / RBB; // ... chunks per k-row, k-rows per DMA instruction
-  static_assert(HALF <= NMF && NRD <= NMF, "one LDS read or DMA per MFMA");
+  static_assert(TM % 2 == 0 && TN <= 8 && TN >= 2, "wave tile");
   static_assert(NS >= 2 && NS <= 4 && NDMA * (NS - 1) + HALF <= 63, "outstanding DMAs must fit the vmcnt counter");
   auto stage_off = [](int kb) { return (NS == 2 ? (kb & 1) : NS == 4 ? (kb & 3) : kb % NS) * STAGEB; };
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -164,36 +200,41 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   const int M = (int)g.M, N = (int)g.N;
   const int64_t b_step = B_KC ? (int64_t)kDmaRowB : g.sbk * (int64_t)(kDmaBK * 2);  // bytes per K step
 
-  // ---- DMA source addresses.  Wave w issues NA (NB) instructions per stage for A (B); instruction j
-  // lands at operand base + (w*NA + j) * 1024, split into a part that goes through M0 ((j/4)*4096)
-  // and an instruction immediate ((j%4)*1024).  The hardware adds the immediate to the global address
-  // as well, so it is subtracted here.
-  const char* a_src[NA];
-  const char* b_src[NB];
+  // ---- DMA source addresses: a scalar base per operand and K step plus a 32-bit byte offset per lane and
+  // instruction, so that the loop spends no vector instruction on addresses.  Wave w issues NA (NB) instructions
+  // per stage for A (B); instruction j lands at operand base + (w*NA + j) * 1024, split into a part that goes
+  // through M0 ((j/4)*4096) and an instruction immediate ((j%4)*1024).  The hardware adds the immediate to the
+  // global address as well, so it is taken out of the lane offset; the scalar bases sit 3072 bytes low to keep
+  // every lane offset non-negative.  (The host admits only operands whose tile-local offsets fit 32 bits.)
+  uint32_t a_off[NA], b_off[NB];
 #pragma unroll
   for (int j = 0; j < NA; ++j) {
     const int r = (wave * NA + j) * 8 + (lane >> 3);
     const int c = (lane & 7) ^ ((r >> 1) & 7);
     int ra = row0 + r;
-    ra = ra < M ? ra : M - 1;
-    a_src[j] = (const char*)g.A + ((int64_t)ra * g.sam + c * 8) * 2 - (j & 3) * 1024 + (int64_t)kb0 * kDmaRowB;
+    ra = (ra < M ? ra : M - 1) - row0;
+    a_off[j] = (uint32_t)(((int64_t)ra * g.sam + c * 8) * 2) + 3072u - (uint32_t)((j & 3) * 1024);
   }
+  const char* a_base = (const char*)g.A + ((int64_t)row0 * g.sam) * 2 + (int64_t)kb0 * kDmaRowB - 3072;
+  const char* b_base;
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     if constexpr (B_KC) {
       const int r = (wave * NB + j) * 8 + (lane >> 3);
       const int c = (lane & 7) ^ ((r >> 1) & 7);
       int rb = col0 + r;
-      rb = rb < N ? rb : N - 1;
-      b_src[j] = (const char*)g.B + ((int64_t)rb * g.sbn + c * 8) * 2 - (j & 3) * 1024 + kb0 * b_step;
+      rb = (rb < N ? rb : N - 1) - col0;
+      b_off[j] = (uint32_t)(((int64_t)rb * g.sbn + c * 8) * 2) + 3072u - (uint32_t)((j & 3) * 1024);
     } else {
       const int k = (wave * NB + j) * RPI + lane / CPRB;
       const int c = (lane % CPRB) ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1));
       int cb = col0 + c * 8;
-      cb = cb + 8 <= N ? cb : N - 8;
-      b_src[j] = (const char*)g.B + ((int64_t)k * g.sbk + cb) * 2 - (j & 3) * 1024 + kb0 * b_step;
+      cb = (cb + 8 <= N ? cb : N - 8) - col0;
+      b_off[j] = (uint32_t)(((int64_t)k * g.sbk + cb) * 2) + 3072u - (uint32_t)((j & 3) * 1024);
     }
   }
+  if constexpr (B_KC) b_base = (const char*)g.B + ((int64_t)col0 * g.sbn) * 2 + kb0 * b_step - 3072;
+  else b_base = (const char*)g.B + (int64_t)col0 * 2 + kb0 * b_step - 3072;
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   char* const dma_a = lds + wave_s * (NA * 1024);
   char* const dma_b = lds + A_OPB + wave_s * (NB * 1024);
@@ -203,24 +244,38 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     const int k = kb + krot;
     return k >= nk ? k - nk : k;
   };
-  auto issue = [&](int kb, int kk, auto jc) {
+  // operand bases of K step kk, forced into scalar registers
+  auto uniform_ptr = [](const char* q) {
+    const uint64_t v = (uint64_t)(uintptr_t)q;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+  };
+  struct KBase { const char* a; const char* b; };
+  auto bases_of = [&](int kb) {
+    const int kk = wrap(kb);
+    return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step)};
+  };
+  auto issue = [&](int kb, const KBase& kbase, auto jc) {
     constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
     char* l = (IS_A ? dma_a : dma_b) + stage_off(kb) + (jj >> 2) * 4096;
-    const char* gp;
-    if constexpr (IS_A) gp = a_src[jj] + (int64_t)kk * kDmaRowB;
-    else gp = b_src[jj] + (int64_t)kk * b_step;
+    // (the lane offset is kept opaque: the compiler would otherwise go back to 64-bit lane addresses, precomputed per
+    // instruction and advanced by a 64-bit vector add per K step)
+    uint32_t off = IS_A ? a_off[jj] : b_off[jj];
+    asm volatile("" : "+v"(off));
+    const char* gp = (IS_A ? kbase.a : kbase.b) + (uint64_t)off;
     __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
   };
 
-  // ---- fragment addresses
-  const int fr = lane & 31, fh = lane >> 5;
-  const int q = (fr >> 1) & 7;  // sub-tile rows start at multiples of 32, so (row >> 1) & 7 depends on fr only
+  // ---- fragment addresses.  A fragment is 16 rows x 32 k: lane (r = lane % 16, g = lane / 16) holds the 8 k
+  // 32 ks + 8 g ... of row r, i.e. chunk 4 ks + g of the row's 128 bytes.
+  const int fr = lane & 15, fg = lane >> 4;
+  const int q = fr >> 1;  // sub-tile rows start at multiples of 16, so (row >> 1) & 7 depends on fr only
   const int a_lane = (wm * WTM + fr) * kDmaRowB;
-  int pos[4];
+  int pos[2];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) pos[s] = ((2 * s + fh) ^ q) * 16;
+  for (int ks = 0; ks < 2; ++ks) pos[ks] = ((4 * ks + fg) ^ q) * 16;
   int b_lane = 0;      // K-contiguous B: like A
   uint32_t b_tr[TN];   // N-contiguous B: per sub-tile j, the lane's address within a stage
 #pragma unroll
@@ -228,99 +283,115 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   if constexpr (B_KC) {
     b_lane = A_OPB + (wn * WTN + fr) * kDmaRowB;
   } else {
-    // lane -> k-row 8*hh + m (+ 16*sub-step, +4 for the second read), columns 16*b4 + 4*(lane&3) .. +3 of sub-tile j
-    const int m = (lane & 15) >> 2, hh = lane >> 5, b4 = (lane >> 4) & 1, b1 = (lane & 3) >> 1;
-    const int krow = 8 * hh + m;
-    const int sw = (m << 2) | (hh << 1);
+    // the transposing read hands lane t of every 16-lane row the 4 k of column t that the row's lanes addressed as
+    // 4 k-rows x 4 column quads: lane -> k-row 8 g + m (+ 32 ks, + 4 for the second read), columns 4 (lane & 3) ...
+    // of sub-tile j
+    const int m = (lane & 15) >> 2, b1 = (lane & 3) >> 1;
+    const int krow = 8 * fg + m;
+    const int sw = (m << 2) | ((fg & 1) << 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int chunk = (wn * (WTN / 8) + j * 4 + ((b4 << 1) | b1)) ^ sw;
+      const int chunk = (wn * (WTN / 8) + j * 2 + b1) ^ sw;
       b_tr[j] = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + A_OPB + krow * RBB + chunk * 16 +
                 (lane & 1) * 8;
     }
   }
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  Frag fa[2][TM];
-  u32x4 fb[2][4];
-  // read x of fragment set `set` for sub-step S of `stage`: x < TM -> A sub-tile x, else B sub-tile x-TM
-  auto read_one = [&](int stage, auto sc, auto xc, int set) {
-    constexpr int S = decltype(sc)::value;
-    constexpr int x = decltype(xc)::value;
+  // A fragments of sub-tiles 0 .. HM-1 (set 0) and HM .. TM-1 (set 1); B fragments of the k half 0 and 1
+  Frag fa[2][HM];
+  u32x4 fb[2][TN];
+  auto read_a = [&](int stage, auto ksc, auto hc, auto xc) {
+    constexpr int ks = decltype(ksc)::value, h = decltype(hc)::value, x = decltype(xc)::value;
+    fa[h][x] = *reinterpret_cast<const Frag*>(lds + stage_off(stage) + a_lane + (h * HM + x) * 16 * kDmaRowB + pos[ks]);
+  };
+  auto read_b = [&](int stage, auto ksc, auto xc) {
+    constexpr int ks = decltype(ksc)::value, x = decltype(xc)::value;
     const int sb = stage_off(stage);
-    if constexpr (x < TM) {
-      fa[set][x] = *reinterpret_cast<const Frag*>(lds + sb + a_lane + x * 32 * kDmaRowB + pos[S]);
-    } else if constexpr (B_KC) {
-      fb[set][x - TM] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + (x - TM) * 32 * kDmaRowB + pos[S]);
+    if constexpr (B_KC) {
+      fb[ks][x] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + x * 16 * kDmaRowB + pos[ks]);
     } else {
-      const u32x2 lo = lds_read_tr16_b64<(16 * S) * RBB>(b_tr[x - TM] + sb);
-      const u32x2 hi = lds_read_tr16_b64<(16 * S + 4) * RBB>(b_tr[x - TM] + sb);
-      fb[set][x - TM] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      const u32x2 lo = lds_read_tr16_b64<(32 * ks) * RBB>(b_tr[x] + sb);
+      const u32x2 hi = lds_read_tr16_b64<(32 * ks + 4) * RBB>(b_tr[x] + sb);
+      fb[ks][x] = u32x4{lo[0], lo[1], hi[0], hi[1]};
     }
   };
-  auto wait_reads = [&](int set) {
+  auto wait_reads = [&](auto ksc) {
     if constexpr (B_KC) FGK_WAIT_LGKM0();
-    else lds_wait_tied(fb[set]);
+    else lds_wait_tied(fb[decltype(ksc)::value]);
   };
-  if constexpr (!B_KC && TN < 4) {
-    // the tied wait names four registers per set; give the unused ones a value
-#pragma unroll
-    for (int j = TN; j < 4; ++j) fb[0][j] = fb[1][j] = u32x4{0u, 0u, 0u, 0u};
-  }
 
-  // ---- prologue: K steps 0 .. NS-2, and the head of step NS-1 (the part sub-step 3 of the step before would issue)
+  // ---- prologue: K steps 0 .. NS-2, and the head of step NS-1 (the part the last quarter of the step before
+  // would issue)
   static_for<0, NS - 1>([&](auto sc) {
     constexpr int s = decltype(sc)::value;
-    if (s < nk) static_for<0, NDMA>([&](auto jc) { issue(s, wrap(s), jc); });
+    if (s < nk) {
+      const KBase kbase = bases_of(s);
+      static_for<0, NDMA>([&](auto jc) { issue(s, kbase, jc); });
+    }
   });
   if (nk >= NS) {
-    static_for<0, HALF>([&](auto jc) { issue(NS - 1, wrap(NS - 1), jc); });
+    const KBase kbase = bases_of(NS - 1);
+    static_for<0, HALF>([&](auto jc) { issue(NS - 1, kbase, jc); });
     FGK_WAIT_VM(NDMA * (NS - 2) + HALF);  // K step 0 has landed
   } else {
     FGK_WAIT_VM(0);
   }
   __builtin_amdgcn_s_barrier();
-  static_for<0, NRD>([&](auto xc) { read_one(0, IntC<0>{}, xc, 0); });
-  wait_reads(0);
+  static_for<0, HM>([&](auto xc) { read_a(0, IntC<0>{}, IntC<0>{}, xc); });
+  static_for<0, TN>([&](auto xc) { read_b(0, IntC<0>{}, xc); });
+  wait_reads(IntC<0>{});
   __builtin_amdgcn_sched_barrier(0);
 
-  // One K step.  REFILL_TAIL: sub-step 0 issues the second half of the DMAs of K step kb+NS-1;
-  // REFILL_HEAD: sub-step 3 issues the first half of the DMAs of K step kb+NS (into the stage this step
-  // has just finished reading).  LATER = DMAs that may still be in flight once K step kb+1 has landed:
-  // those of the K steps behind it, which retire in order after it.
+  // One K step = four quarter steps of HM x TN MFMAs: quarter (ks, h) multiplies the A sub-tiles of half h by all
+  // B sub-tiles over the k half ks, while the fragments of the next quarter are read: the other A half, and behind
+  // an h = 1 quarter also the B fragments of the next k half (quarter 3 reads them from the next stage).  The
+  // memory operations of a quarter, reads first, are spread over its MFMAs.
+  // REFILL_TAIL: quarter 0 issues the second half of the DMAs of K step kb+NS-1; REFILL_HEAD: quarter 3 issues the
+  // first half of the DMAs of K step kb+NS (into the stage this step has just finished reading).  LATER = DMAs
+  // that may still be in flight once K step kb+1 has landed: those of the K steps behind it, which retire in
+  // order after it.
   auto k_step = [&](int kb, auto tail_c, auto head_c, auto later_c) {
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
     constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
     constexpr int LATER = decltype(later_c)::value;
-    const int kk_head = wrap(kb + NS), kk_tail = wrap(kb + NS - 1);
-    static_for<0, 4>([&](auto sc) {
-      constexpr int s = decltype(sc)::value;
-      constexpr int cur = s & 1, nxt = cur ^ 1;
+    KBase kk_head = {nullptr, nullptr}, kk_tail = {nullptr, nullptr};
+    if constexpr (REFILL_HEAD) kk_head = bases_of(kb + NS);
+    if constexpr (REFILL_TAIL) kk_tail = bases_of(kb + NS - 1);
+    static_for<0, 4>([&](auto qc) {
+      constexpr int qt = decltype(qc)::value;
+      constexpr int ks = qt >> 1, h = qt & 1;
+      constexpr int nks = ((qt + 1) & 3) >> 1, nh = (qt + 1) & 1;   // the quarter the reads are for
+      constexpr int NRA = HM, NRB = nh == 0 ? TN : 0, NRD = NRA + NRB;
+      constexpr int ND = (qt == 0 && REFILL_TAIL) ? NDMA - HALF : (qt == 3 && REFILL_HEAD) ? HALF : 0;
+      constexpr int NOPS = NRD + ND, OPM = (NOPS + NMF - 1) / NMF;
+      const int rstage = qt == 3 ? kb + 1 : kb;
       static_for<0, NMF>([&](auto xc) {
         constexpr int x = decltype(xc)::value;
-        constexpr int i = x / TN, j = x % TN;
-        acc[i][j] = Mfma<T>::mma(__builtin_bit_cast(Frag, fb[cur][j]), fa[cur][i], acc[i][j]);
-        if constexpr (x < NRD) {
-          if constexpr (s < 3) read_one(kb, IntC<s + 1>{}, xc, nxt);
-          else read_one(kb + 1, IntC<0>{}, xc, nxt);
-        }
-        if constexpr (s == 3 && REFILL_HEAD && x < HALF) issue(kb + NS, kk_head, IntC<x>{});
-        if constexpr (s == 0 && REFILL_TAIL && x < NDMA - HALF) issue(kb + NS - 1, kk_tail, IntC<(x < NDMA - HALF ? HALF + x : 0)>{});
+        constexpr int il = x / TN, j = x % TN;
+        MfmaK32<T>::mma(__builtin_bit_cast(Frag, fb[ks][j]), fa[h][il], acc[h * HM + il][j]);
+        static_for<0, OPM>([&](auto oc) {
+          constexpr int o = x * OPM + decltype(oc)::value;
+          if constexpr (o < NRA) read_a(rstage, IntC<nks>{}, IntC<nh>{}, IntC<(o < NRA ? o : 0)>{});
+          else if constexpr (o < NRD) read_b(rstage, IntC<nks>{}, IntC<(o < NRD ? o - NRA : 0)>{});
+          else if constexpr (o < NOPS) {
+            if constexpr (qt == 0) issue(kb + NS - 1, kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{});
+            else issue(kb + NS, kk_head, IntC<(o < NOPS ? o - NRD : 0)>{});
+          }
+        });
         __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr (s == 2) {
+      if constexpr (qt == 2) {
         FGK_WAIT_VM(LATER);
-        wait_reads(nxt);
+        wait_reads(IntC<nks>{});
         __builtin_amdgcn_s_barrier();
       } else {
-        wait_reads(nxt);
+        wait_reads(IntC<nks>{});
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -337,6 +408,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     }
   });
   k_step(kb, IntC<0>{}, IntC<0>{}, IntC<0>{});
+  mfma_drain(acc);
 
   finish(acc);
 }
@@ -348,20 +420,18 @@ __global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ?
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
   const int nk = (int)(g.K / kDmaBK);
   // K-rotated start per XCD (workgroups go to the XCDs round-robin by id): the eight XCDs then read eight different
-  // column ranges of the operands at any one time, which spreads the requests over the memory channels when the
-  // leading dimensions are large powers of two; the tiles of one XCD stay in step and keep sharing panels in its L2
+  // column ranges of the operands at any one time; the tiles of one XCD stay in step and keep sharing panels in its L2
   const int krot = g.k_stagger ? (int)((blockIdx.x & 7u) * (unsigned)nk / 8u) : 0;
-  dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, 0, nk,
-                                     [&](f32x16 (&acc)[BM / 64][BN / 64]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); }, krot);
+  dma_tile_mainloop<T, B_KC, BM, BN, NS>(
+      g, lds, tm, tn, 0, nk, [&](f32x4 (&acc)[BM / 32][BN / 32]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); }, krot);
 }
-
 // Stream-K over 128x128 tiles with the main loop above: the (tile, K step) units, tile-major, are dealt
 // in equal contiguous ranges to the workgroups; a tile split between workgroups is finished by whichever
 // of them arrives last (ticket per tile, fp32 partial tiles in the workspace, added in workgroup order so
 // the result does not depend on who finishes).  Same scheme as gemm_streamk_kernel in gemm_tile.h.
 template <typename T, bool B_KC, int NS>
 __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
-  constexpr int BM = 128, BN = 128, TM = 2, TN = 2;
+  constexpr int BM = 128, BN = 128, TM = 4, TN = 4;  // 16x16 sub-tiles per wave
   extern __shared__ __attribute__((aligned(16))) char lds[];
   __shared__ unsigned ticket_s;
   const int w = blockIdx.x, tid = threadIdx.x;
@@ -377,7 +447,7 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
     int tm, tn;
     tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
     __syncthreads();  // the LDS stages of the previous segment are no longer read
-    dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, it0, it1 - it0, [&](f32x16 (&acc)[TM][TN]) {
+    dma_tile_mainloop<T, B_KC, BM, BN, NS>(g, lds, tm, tn, it0, it1 - it0, [&](f32x4 (&acc)[TM][TN]) {
       bool finish = (it0 == 0 && it1 == g.iters_per_tile);
       if (!finish) {
         // slot 0 of a workgroup: the tile it starts in; slot 1: a tile it enters from the left
@@ -387,8 +457,8 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
-              __hip_atomic_store(slot + ((i * TN + j) * 16 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED,
+            for (int e = 0; e < 4; ++e)
+              __hip_atomic_store(slot + ((i * TN + j) * 4 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
         // device-coherent stores: every one of them has completed before the ticket publishes them
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -406,7 +476,7 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-              for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+              for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
           auto slot_of = [&](int w2) {
             return g.partials + ((int64_t)w2 * 2 + (sk_begin(g.sk_per, g.sk_rem, w2) < tile_begin ? 1 : 0)) * (BM * BN) + tid;
           };
@@ -416,17 +486,17 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
           for (; w2 < w_last; w2 += 2) {
             const float* s0 = slot_of(w2);
             const float* s1 = slot_of(w2 + 1);
-            float t0[TM * TN * 16], t1[TM * TN * 16];
+            float t0[TM * TN * 4], t1[TM * TN * 4];
 #pragma unroll
-            for (int x = 0; x < TM * TN * 16; ++x) t0[x] = __hip_atomic_load(s0 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int x = 0; x < TM * TN * 4; ++x) t0[x] = __hip_atomic_load(s0 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-            for (int x = 0; x < TM * TN * 16; ++x) t1[x] = __hip_atomic_load(s1 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int x = 0; x < TM * TN * 4; ++x) t1[x] = __hip_atomic_load(s1 + x * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
               for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = (acc[i][j][e] + t0[(i * TN + j) * 16 + e]) + t1[(i * TN + j) * 16 + e];
+                for (int e = 0; e < 4; ++e) acc[i][j][e] = (acc[i][j][e] + t0[(i * TN + j) * 4 + e]) + t1[(i * TN + j) * 4 + e];
           }
           if (w2 == w_last) {
             const float* s0 = slot_of(w2);
@@ -435,8 +505,8 @@ __global__ __launch_bounds__(256, 2) void gemm_dma_streamk_kernel(GemmArgs g) {
 #pragma unroll
               for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e)
-                  acc[i][j][e] += __hip_atomic_load(s0 + ((i * TN + j) * 16 + e) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int e = 0; e < 4; ++e)
+                  acc[i][j][e] += __hip_atomic_load(s0 + ((i * TN + j) * 4 + e) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
           if (tid == 0) __hip_atomic_store(g.tickets + w_first, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }

@@ -13,8 +13,12 @@ bool dma_supported(const GemmArgs& g, int elem_bytes) {
   if (g.sak != 1 || g.sam % 8 != 0 || !fg_aligned(g.A, 16) || !fg_aligned(g.B, 16)) return false;
   if (g.scn != 1 || g.scm % 8 != 0 || !fg_aligned(g.C, 16)) return false;
   if (g.bias != nullptr && (g.sin != 1 || g.sim % 4 != 0 || !fg_aligned(g.bias, 8))) return false;
-  if (g.sbk == 1) return g.sbn % 8 == 0;  // K-contiguous B
-  if (g.sbn == 1) return g.sbk % 8 == 0;  // N-contiguous B
+  // the kernels address a tile's rows through 32-bit byte offsets from a scalar base: 256 rows (64 for the k-rows
+  // of an N-contiguous B) of the leading dimension, plus a row, must stay below 4 GiB
+  const int64_t lim = ((int64_t)1 << 32) - 8192;
+  if (g.sam * 2 * 256 + g.K * 2 >= lim) return false;
+  if (g.sbk == 1) return g.sbn % 8 == 0 && g.sbn * 2 * 256 + g.K * 2 < lim;  // K-contiguous B
+  if (g.sbn == 1) return g.sbk % 8 == 0 && g.sbk * 2 * 64 + g.N * 2 < lim;   // N-contiguous B
   return false;
 }
 
