@@ -517,13 +517,13 @@ def main():
                     workload="reference: torch copy of a [131072,2048] bf16 tensor (512 MiB read + 512 MiB written)", cpu=None)
 
     def wl_mfma_ceiling(random_operands):
-        # calibration, not an operator: the rate the matrix cores sustain on nothing but MFMA 32x32x16
-        # bf16, with operand fragments of zeros or of N(0,1) values.  The chip is power-limited, so the
+        # calibration, not an operator: the rate the matrix cores sustain on nothing but MFMA 16x16x32
+        # bf16 (the GEMM kernels' instruction), with operand fragments of zeros or of N(0,1) values.  The chip is power-limited, so the
         # second figure -- not the 2.5 PFLOP/s of the data sheet -- is what a real bf16 GEMM can approach.
         import ctypes
         from flaggems_amd import _C
         src = (torch.randn(8 * 256 * 8, device=dev) if random_operands else torch.zeros(8 * 256 * 8, device=dev)).to(bf16)
-        blocks, iters = 1024, 4096
+        blocks, iters = 1024, 2048
         out = torch.empty(blocks * 256, device=dev)
         flops = ctypes.c_double(0.0)
 

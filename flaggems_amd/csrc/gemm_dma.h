@@ -255,17 +255,23 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     const int kk = wrap(kb);
     return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step)};
   };
-  auto issue = [&](int kb, const KBase& kbase, auto jc) {
+  // `first_c`: the instruction opens a run of consecutive issue() calls (M0 holds nothing known)
+  auto issue = [&](int kb, const KBase& kbase, auto jc, auto first_c) {
     constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
     char* l = (IS_A ? dma_a : dma_b) + stage_off(kb) + (jj >> 2) * 4096;
-    // (the lane offset is kept opaque: the compiler would otherwise go back to 64-bit lane addresses, precomputed per
-    // instruction and advanced by a 64-bit vector add per K step)
-    uint32_t off = IS_A ? a_off[jj] : b_off[jj];
-    asm volatile("" : "+v"(off));
-    const char* gp = (IS_A ? kbase.a : kbase.b) + (uint64_t)off;
-    __builtin_amdgcn_global_load_lds(FGK_GLBP(gp), FGK_LDSP(l), 16, (jj & 3) * 1024, 0);
+    // Written as asm: scalar base + 32-bit lane offset + immediate, LDS address in M0 (set here, with the wait
+    // state the hardware wants between a scalar write of M0 and an LDS-direct load; nothing else in these kernels
+    // uses M0).  Through the builtin the compiler either goes back to 64-bit lane addresses (a quarter-rate
+    // vector add per instruction) or needs a register copy and a wait state per instruction, and every
+    // instruction issued here is a slot the wave's next MFMA waits for.
+    if constexpr (decltype(first_c)::value != 0 || (jj & 3) == 0) {
+      const uint32_t m0v = (uint32_t)(uintptr_t)FGK_LDSP(l);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory");
+    }
+    const uint32_t off = IS_A ? a_off[jj] : b_off[jj];
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(off), "s"(IS_A ? kbase.a : kbase.b), "n"((jj & 3) * 1024) : "memory");
   };
 
   // ---- fragment addresses.  A fragment is 16 rows x 32 k: lane (r = lane % 16, g = lane / 16) holds the 8 k
@@ -332,12 +338,12 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     constexpr int s = decltype(sc)::value;
     if (s < nk) {
       const KBase kbase = bases_of(s);
-      static_for<0, NDMA>([&](auto jc) { issue(s, kbase, jc); });
+      static_for<0, NDMA>([&](auto jc) { issue(s, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
     }
   });
   if (nk >= NS) {
     const KBase kbase = bases_of(NS - 1);
-    static_for<0, HALF>([&](auto jc) { issue(NS - 1, kbase, jc); });
+    static_for<0, HALF>([&](auto jc) { issue(NS - 1, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
     FGK_WAIT_VM(NDMA * (NS - 2) + HALF);  // K step 0 has landed
   } else {
     FGK_WAIT_VM(0);
@@ -380,8 +386,8 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
           if constexpr (o < NRA) read_a(rstage, IntC<nks>{}, IntC<nh>{}, IntC<(o < NRA ? o : 0)>{});
           else if constexpr (o < NRD) read_b(rstage, IntC<nks>{}, IntC<(o < NRD ? o - NRA : 0)>{});
           else if constexpr (o < NOPS) {
-            if constexpr (qt == 0) issue(kb + NS - 1, kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{});
-            else issue(kb + NS, kk_head, IntC<(o < NOPS ? o - NRD : 0)>{});
+            if constexpr (qt == 0) issue(kb + NS - 1, kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{}, IntC<(o == NRD)>{});
+            else issue(kb + NS, kk_head, IntC<(o < NOPS ? o - NRD : 0)>{}, IntC<(o == NRD)>{});
           }
         });
         __builtin_amdgcn_sched_barrier(0);

@@ -50,7 +50,7 @@ void fg_reload_options(void);
 int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
 
 /* Calibration of the matrix-core roofline (no counterpart in the reference; used by bench.py):
- * every wave of `blocks` 256-thread workgroups issues 16 * iters MFMA 32x32x16 bf16 on operand
+ * every wave of `blocks` 256-thread workgroups issues 64 * iters MFMA 16x16x32 bf16 on operand
  * fragments read once from `operands` (8 * 256 * 16 bytes).  `out` receives blocks * 256 floats;
  * *flops the floating-point operations of the launch.  The sustained rate depends on the operand
  * bits (power): random operands give the ceiling a real bf16 GEMM can approach on this part. */
