@@ -17,6 +17,8 @@ int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace,
 
 // implemented in gemm_dma.hip
 bool dma_supported(const GemmArgs& g, int elem_bytes);
+bool dma_supported_ragged(const GemmArgs& g, int elem_bytes);
+const void* dma_zeros();
 double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep);
 double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, int* workers);
 int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st);
@@ -104,6 +106,8 @@ int pick_mode(const void* base, int64_t rows, int64_t K, int64_t s_row, int64_t 
   return LOAD_GEN;
 }
 
+constexpr int kDmaBKHost = 64;  // K step of the direct-to-LDS kernels
+
 void set_tiles(GemmArgs& g, int BM, int BN, int BK) {
   g.tiles_m = (int)fg_cdiv(g.M, BM);
   g.tiles_n = (int)fg_cdiv(g.N, BN);
@@ -128,6 +132,17 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
     }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
+    // K a multiple of 8 but not of 64: the direct-to-LDS kernel on one of two tiles, the last K step padded with zeros
+    if (amode != LOAD_GEN && dma_supported_ragged(g, (int)sizeof(T)) && !fg_options().gemm_no_dma) {
+      g.zeros = dma_zeros();
+      if (g.zeros != nullptr) {
+        const bool big = big_tiles * 10 >= (int64_t)num_cu * 9;
+        set_tiles(g, big ? 256 : 128, big ? 256 : 128, BK);
+        g.k_ragged = (int)(g.K % kDmaBKHost);
+        g.k_stagger = 0;
+        return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, big ? 256 : 128, big ? 256 : 128, true, st);
+      }
+    }
     if (amode != LOAD_GEN && amode != LOAD_KU && amode != LOAD_MNU && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
       set_tiles(g, 256, 256, BK);
       return launch_dp_modes<T, 256, 256>(g, amode, bmode, st);

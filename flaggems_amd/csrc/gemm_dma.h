@@ -39,7 +39,8 @@
 // 16-byte stores.
 //
 // Preconditions (checked on the host): 16-bit type; A K-contiguous; B K- or N-contiguous; K a
-// multiple of 64; N a multiple of 8; operand base pointers and row strides multiples of 16 bytes;
+// multiple of 64 (a multiple of 8 above 64 for the data-parallel 256x256 and 128x128 kernels, which then copy the
+// missing chunks of the last K step from a buffer of zeros); N a multiple of 8; operand base pointers and row strides multiples of 16 bytes;
 // C with unit column stride and 16-byte aligned rows; a bias with unit column stride and 8-byte
 // aligned rows.  M and N are otherwise arbitrary: tile rows past the edge are clamped to the last
 // valid row (or 8-column chunk) on load and never stored.  Everything else runs on the
@@ -175,7 +176,9 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
 
 // Main loop over the K steps [kb0, kb0 + nk) of tile (tm, tn); `finish` receives the accumulators.
 // NS = number of LDS stages: K step kb lives in stage kb % NS and is requested NS - 1 steps ahead.
-template <typename T, bool B_KC, int BM, int BN, int NS, typename F>
+// RAGGED: K is a multiple of 8 but not of 64; nk counts the partial last K step, whose 16-byte chunks past K are
+// copied from a buffer of zeros instead (both operands, so whatever follows the rows in memory never enters a sum).
+template <typename T, bool B_KC, int BM, int BN, int NS, bool RAGGED = false, typename F>
 __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish,
                                                   int krot = 0) {
   static_assert(sizeof(T) == 2, "16-bit element types");
@@ -250,10 +253,10 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
   };
-  struct KBase { const char* a; const char* b; };
+  struct KBase { const char* a; const char* b; bool last; };
   auto bases_of = [&](int kb) {
     const int kk = wrap(kb);
-    return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step)};
+    return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step), RAGGED && kk == nk - 1};
   };
   // `first_c`: the instruction opens a run of consecutive issue() calls (M0 holds nothing known)
   auto issue = [&](int kb, const KBase& kbase, auto jc, auto first_c) {
@@ -271,6 +274,21 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory");
     }
     const uint32_t off = IS_A ? a_off[jj] : b_off[jj];
+    if constexpr (RAGGED) {
+      if (kbase.last) {
+        // the partial K step: per-lane 64-bit addresses, lanes whose chunk lies past K read zeros
+        bool valid;
+        if constexpr (IS_A || B_KC) {
+          const int r = (wave * (IS_A ? NA : NB) + jj) * 8 + (lane >> 3);
+          valid = (((lane & 7) ^ ((r >> 1) & 7)) * 8) < g.k_ragged;
+        } else {
+          valid = (wave * NB + jj) * RPI + lane / CPRB < g.k_ragged;
+        }
+        const char* gp = valid ? (IS_A ? kbase.a : kbase.b) + (uint64_t)off : (const char*)g.zeros;
+        asm volatile("global_load_lds_dwordx4 %0, off offset:%1" : : "v"(gp), "n"((jj & 3) * 1024) : "memory");
+        return;
+      }
+    }
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(off), "s"(IS_A ? kbase.a : kbase.b), "n"((jj & 3) * 1024) : "memory");
   };
 
@@ -366,7 +384,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
     constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
     constexpr int LATER = decltype(later_c)::value;
-    KBase kk_head = {nullptr, nullptr}, kk_tail = {nullptr, nullptr};
+    KBase kk_head = {nullptr, nullptr, false}, kk_tail = {nullptr, nullptr, false};
     if constexpr (REFILL_HEAD) kk_head = bases_of(kb + NS);
     if constexpr (REFILL_TAIL) kk_tail = bases_of(kb + NS - 1);
     static_for<0, 4>([&](auto qc) {
@@ -419,16 +437,16 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   finish(acc);
 }
 
-template <typename T, bool B_KC, int BM, int BN, int NS = 2>
+template <typename T, bool B_KC, int BM, int BN, int NS = 2, bool RAGGED = false>
 __global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
-  const int nk = (int)(g.K / kDmaBK);
+  const int nk = (int)((g.K + kDmaBK - 1) / kDmaBK);
   // K-rotated start per XCD (workgroups go to the XCDs round-robin by id): the eight XCDs then read eight different
   // column ranges of the operands at any one time; the tiles of one XCD stay in step and keep sharing panels in its L2
   const int krot = g.k_stagger ? (int)((blockIdx.x & 7u) * (unsigned)nk / 8u) : 0;
-  dma_tile_mainloop<T, B_KC, BM, BN, NS>(
+  dma_tile_mainloop<T, B_KC, BM, BN, NS, RAGGED>(
       g, lds, tm, tn, 0, nk, [&](f32x4 (&acc)[BM / 32][BN / 32]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); }, krot);
 }
 // Stream-K over 128x128 tiles with the main loop above: the (tile, K step) units, tile-major, are dealt

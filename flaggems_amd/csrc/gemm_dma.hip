@@ -7,9 +7,11 @@
 namespace fgk {
 
 // The kernel's preconditions.  `elem_bytes` is the size of the A/B/C element type.
-bool dma_supported(const GemmArgs& g, int elem_bytes) {
+// `ragged`: K a multiple of 8 above 64 but not of 64 (the data-parallel 256x256 and 128x128 kernels only)
+static bool dma_supported_k(const GemmArgs& g, int elem_bytes, bool ragged) {
   if (elem_bytes != 2) return false;
-  if (g.K < kDmaBK || g.K % kDmaBK != 0 || g.M < 1 || g.N < 8 || g.N % 8 != 0) return false;
+  if (ragged ? (g.K <= kDmaBK || g.K % 8 != 0 || g.K % kDmaBK == 0) : (g.K < kDmaBK || g.K % kDmaBK != 0)) return false;
+  if (g.M < 1 || g.N < 8 || g.N % 8 != 0) return false;
   if (g.sak != 1 || g.sam % 8 != 0 || !fg_aligned(g.A, 16) || !fg_aligned(g.B, 16)) return false;
   if (g.scn != 1 || g.scm % 8 != 0 || !fg_aligned(g.C, 16)) return false;
   if (g.bias != nullptr && (g.sin != 1 || g.sim % 4 != 0 || !fg_aligned(g.bias, 8))) return false;
@@ -21,14 +23,32 @@ bool dma_supported(const GemmArgs& g, int elem_bytes) {
   if (g.sbn == 1) return g.sbk % 8 == 0 && g.sbk * 2 * 64 + g.N * 2 < lim;   // N-contiguous B
   return false;
 }
+bool dma_supported(const GemmArgs& g, int elem_bytes) { return dma_supported_k(g, elem_bytes, false); }
+bool dma_supported_ragged(const GemmArgs& g, int elem_bytes) { return dma_supported_k(g, elem_bytes, true); }
 
-template <typename T, bool B_KC, int BM, int BN, int NS>
+// 4 KB of zeros per device: the source of the chunks past K in the last K step of a ragged problem
+static __device__ __align__(256) unsigned char dma_zero_chunks[4096];
+const void* dma_zeros() {
+  static std::mutex mu;
+  static const void* per_device[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (per_device[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(dma_zero_chunks)) != hipSuccess) return nullptr;
+    per_device[dev] = p;
+  }
+  return per_device[dev];
+}
+
+template <typename T, bool B_KC, int BM, int BN, int NS, bool RAGGED = false>
 static int launch_dma_t(const GemmArgs& g, hipStream_t st) {
   constexpr int LDS = dma_lds_bytes(BM, BN, NS);
   static_assert(LDS <= 160 * 1024, "LDS of one CU");
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
-  auto kern = gemm_dma_kernel<T, B_KC, BM, BN, NS>;
+  auto kern = gemm_dma_kernel<T, B_KC, BM, BN, NS, RAGGED>;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
   });
@@ -41,9 +61,9 @@ static int launch_dma_t(const GemmArgs& g, hipStream_t st) {
   return fg_check_launch("gemm");
 }
 
-template <typename T, int BM, int BN, int NS>
+template <typename T, int BM, int BN, int NS, bool RAGGED = false>
 static int launch_dma_b(const GemmArgs& g, hipStream_t st) {
-  return g.sbk == 1 ? launch_dma_t<T, true, BM, BN, NS>(g, st) : launch_dma_t<T, false, BM, BN, NS>(g, st);
+  return g.sbk == 1 ? launch_dma_t<T, true, BM, BN, NS, RAGGED>(g, st) : launch_dma_t<T, false, BM, BN, NS, RAGGED>(g, st);
 }
 
 // Duration model of a data-parallel launch, in microseconds.  A CU holds one workgroup, so the tiles run in rounds
@@ -118,6 +138,11 @@ double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, in
 int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st) {
 #define FG_DMA(T)                                                                                         \
   do {                                                                                                    \
+    if (g.k_ragged != 0) {                                                                                \
+      if (bm == 256 && bn == 256) return launch_dma_b<T, 256, 256, 2, true>(g, st);                       \
+      if (bm == 128 && bn == 128) return launch_dma_b<T, 128, 128, 4, true>(g, st);                       \
+      break;                                                                                              \
+    }                                                                                                     \
     if (bm == 256 && bn == 256) return launch_dma_b<T, 256, 256, 2>(g, st);                               \
     if (bm == 192 && bn == 256) return launch_dma_b<T, 192, 256, 2>(g, st);                               \
     if (bm == 256 && bn == 128) return deep ? launch_dma_b<T, 256, 128, 3>(g, st) : launch_dma_b<T, 256, 128, 2>(g, st); \

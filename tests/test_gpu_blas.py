@@ -264,8 +264,8 @@ def test_stream_k_needs_workspace(gpu):
 
 
 # Shapes with enough 256x256 tiles to take the direct-to-LDS kernel (first three), and neighbours that
-# miss one of its preconditions (K not a multiple of 64, N not a multiple of 8) and must take the
-# register-staged kernel instead; ragged M and N edges in both.
+# miss one of its preconditions (K = 72 takes its zero-padded last K step, N not a multiple of 8 the
+# register-staged kernel instead); ragged M and N edges in both.
 LARGE_TILE_SHAPES = [(3857, 4104, 64), (4100, 4104, 256), (4096, 4096, 192), (4096, 4096, 72), (3900, 4100, 128)]
 
 
@@ -294,6 +294,40 @@ def test_mm_addmm_large_tiles(gpu, M, N, K, dtype, b_col_major):
         torch.mm(a, b, out=out)
     gems_assert_close(out[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
     gems_assert_close(out[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
+
+
+# K a multiple of 8 but not of 64: the direct-to-LDS kernels copy the chunks of the last K step that lie past K from a
+# buffer of zeros.  Two to 44 K steps, 8 to 56 valid k in the last one, both tiles (the large shapes fill the machine
+# with 256x256 tiles), ragged M and N edges.  The operands are views into larger tensors whose memory behind every row
+# (and behind the last row) holds NaN: a chunk read from there instead of the zeros poisons its row or column.
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(300, 520, 72), (1100, 2824, 136), (2040, 1032, 1000), (513, 4104, 2744), (4100, 4104, 200),
+                                   (3900, 4096, 120)])
+@pytest.mark.parametrize("b_col_major", [False, True])
+def test_mm_addmm_k_not_a_multiple_of_64(gpu, M, N, K, dtype, b_col_major):
+    torch.manual_seed(M + K)
+    pad = 64 - K % 64
+    a_full = torch.full((M + 1, K + pad), float("nan"), dtype=dtype, device=gpu)
+    a = a_full[:M, :K]
+    a.copy_(torch.randn(M, K, device=gpu))
+    if b_col_major:
+        b_full = torch.full((N + 1, K + pad), float("nan"), dtype=dtype, device=gpu)
+        b_full[:N, :K] = torch.randn(N, K, device=gpu).to(dtype)
+        b = b_full[:N, :K].t()
+    else:
+        b_full = torch.full((K + pad, N), float("nan"), dtype=dtype, device=gpu)
+        b_full[:K] = torch.randn(K, N, device=gpu).to(dtype)
+        b = b_full[:K]
+    rows = torch.tensor([0, 1, 15, 16, 127, 128, 255, 256, M // 2, M - 129, M - 2, M - 1], device=gpu)
+    cols = torch.tensor([0, 7, 8, 15, 16, 255, 256, N // 2, N - 257, N - 9, N - 8, N - 1], device=gpu)
+    c = flag_gems.mm(a, b)
+    assert torch.isfinite(c).all()
+    gems_assert_close(c[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
+    gems_assert_close(c[:, cols], O.mm(a, b[:, cols]), dtype, reduce_dim=K)
+    bias = torch.randn(N, dtype=dtype, device=gpu)
+    d = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
+    gems_assert_close(d[rows], O.addmm(bias, a[rows], b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
+    assert torch.equal(flag_gems.mm(a, b), c)
 
 
 # The direct-to-LDS kernel exists for five tile sizes; the library picks by how the tile count fills the
