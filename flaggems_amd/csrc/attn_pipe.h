@@ -238,14 +238,19 @@ __global__ __launch_bounds__(256, (RBW == 1 ? 2 : 1)) void attn_varlen_pipe_kern
       const uint32_t slot_in_page = ((uint32_t)(nb * kBN) + wave_key0) & (uint32_t)page_mask;
       const char* rp = base + ((uint64_t)page * page_b + (uint64_t)(slot_in_page * row_b));
       const uint32_t step_b = (uint32_t)KPI * row_b - 1024u;
+      // The copies are written as asm: scalar row base, 32-bit lane offset, immediate; M0 (the LDS address of the
+      // wave's part of the slot) is set once per operand tile, with the wait state the hardware wants between a
+      // scalar write of M0 and an LDS-direct load.  Through the builtin every copy costs a register move and a wait
+      // state more, and on this part vector instructions are paid for in matrix-pipe time.
+      {
+        const uint32_t m0v = (uint32_t)(uintptr_t)FG_LDSP(dst);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory", "m0");
+      }
       a_static_for<0, IPW>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
-        // the lane offset is kept opaque so that the address stays "scalar base + 32-bit lane offset" (the
-        // compiler would otherwise precompute a 64-bit lane offset per instruction and operand)
-        uint32_t c0 = lane_c0;
-        asm volatile("" : "+v"(c0));
-        const uint32_t voff = (IS_V ? lane_row_v : lane_row_k) + (c0 ^ (uint32_t)(j * 16));
-        __builtin_amdgcn_global_load_lds(FG_GLBP(rp + (uint64_t)((uint32_t)j * step_b) + voff), FG_LDSP(dst), 16, j * 1024, 0);
+        const uint32_t voff = (IS_V ? lane_row_v : lane_row_k) + (lane_c0 ^ (uint32_t)(j * 16));
+        const char* rj = rp + (uint64_t)((uint32_t)j * step_b);
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(rj), "n"(j * 1024) : "memory");
       });
     } else {
       // partial tile: keys past the end are clamped to the last one (their scores are masked)

@@ -137,6 +137,17 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
   const float alpha = g.alpha, beta = g.beta;
   const bool scale = alpha != 1.0f;
   const int lr = lane & 15, lg = lane >> 4;
+  // a bias row broadcast over M (the addmm of a linear layer) is the same for every output row: fetched once per
+  // lane and sub-tile column instead of once per output element group
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  const bool bcast = bias != nullptr && g.sim == 0;
+  T4 brow[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int c = col0 + wn * WTN + j * 16 + lg * 4;
+    brow[j] = T4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    if (bcast && c < N) brow[j] = *reinterpret_cast<const T4*>(bias + c);
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int64_t r = row0 + wm * WTM + i * 16 + lr;
@@ -148,9 +159,8 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
         const int j = 2 * jp + jj;
         const int c = col0 + wn * WTN + j * 16 + lg * 4;
         if (bias != nullptr) {
-          typedef T T4 __attribute__((ext_vector_type(4)));
-          T4 t = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-          if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+          T4 t = brow[j];
+          if (!bcast && r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
 #pragma unroll
           for (int e = 0; e < 4; ++e) acc[i][j][e] = acc[i][j][e] * alpha + (float)t[e] * beta;
         } else if (scale) {
