@@ -31,8 +31,6 @@ void load_options() {
   FgOptions o = {};
   o.gemm_no_dma = getenv("FG_GEMM_NO_DMA") != nullptr;
   o.gemm_sk_even = getenv("FG_GEMM_SK_EVEN") != nullptr;
-  o.gemm_k_stagger = -1;
-  if (const char* e = getenv("FG_GEMM_KSTAGGER")) o.gemm_k_stagger = e[0] != '0' ? 1 : 0;
   if (const char* e = getenv("FG_GEMM_TILE")) {
     int a = 0, b = 0;
     char c = 0;

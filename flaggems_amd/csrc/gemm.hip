@@ -125,9 +125,6 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
       bool deep = false;
       dma_pick_tile(g.M, g.N, g.K, num_cu, &bm, &bn, &deep);
       set_tiles(g, bm, bn, BK);
-      const int ks = fg_options().gemm_k_stagger;
-      g.k_stagger = ks >= 0 ? ks : 0;
-      if (g.iters_per_tile < 8) g.k_stagger = 0;
       return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, deep, st);
     }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
@@ -139,7 +136,6 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
         const bool big = big_tiles * 10 >= (int64_t)num_cu * 9;
         set_tiles(g, big ? 256 : 128, big ? 256 : 128, BK);
         g.k_ragged = (int)(g.K % kDmaBKHost);
-        g.k_stagger = 0;
         return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, big ? 256 : 128, big ? 256 : 128, true, st);
       }
     }

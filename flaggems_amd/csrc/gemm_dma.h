@@ -189,8 +189,7 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
 // RAGGED: K is a multiple of 8 but not of 64; nk counts the partial last K step, whose 16-byte chunks past K are
 // copied from a buffer of zeros instead (both operands, so whatever follows the rows in memory never enters a sum).
 template <typename T, bool B_KC, int BM, int BN, int NS, bool RAGGED = false, typename F>
-__device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish,
-                                                  int krot = 0) {
+__device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, int tm, int tn, int kb0, int nk, F&& finish) {
   static_assert(sizeof(T) == 2, "16-bit element types");
   typedef typename MfmaK32<T>::Frag Frag;
   constexpr int WTM = BM / 2, WTN = BN / 2;        // wave tile
@@ -251,12 +250,6 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   char* const dma_a = lds + wave_s * (NA * 1024);
   char* const dma_b = lds + A_OPB + wave_s * (NB * 1024);
-  // K step kb of the loop reads K step wrap(kb) of the operands: a launch may walk K from a rotated start (krot), which
-  // only permutes the order of the sum
-  auto wrap = [&](int kb) {
-    const int k = kb + krot;
-    return k >= nk ? k - nk : k;
-  };
   // operand bases of K step kk, forced into scalar registers
   auto uniform_ptr = [](const char* q) {
     const uint64_t v = (uint64_t)(uintptr_t)q;
@@ -264,16 +257,15 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
   };
   struct KBase { const char* a; const char* b; bool last; };
-  auto bases_of = [&](int kb) {
-    const int kk = wrap(kb);
+  auto bases_of = [&](int kk) {
     return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step), RAGGED && kk == nk - 1};
   };
   // `first_c`: the instruction opens a run of consecutive issue() calls (M0 holds nothing known)
-  auto issue = [&](int kb, const KBase& kbase, auto jc, auto first_c) {
+  auto issue = [&](int stage_bytes, const KBase& kbase, auto jc, auto first_c) {
     constexpr int j = decltype(jc)::value;  // 0..NDMA-1: the A instructions, then the B instructions
     constexpr bool IS_A = j < NA;
     constexpr int jj = IS_A ? j : j - NA;
-    char* l = (IS_A ? dma_a : dma_b) + stage_off(kb) + (jj >> 2) * 4096;
+    char* l = (IS_A ? dma_a : dma_b) + stage_bytes + (jj >> 2) * 4096;
     // Written as asm: scalar base + 32-bit lane offset + immediate, LDS address in M0 (set here, with the wait
     // state the hardware wants between a scalar write of M0 and an LDS-direct load; nothing else in these kernels
     // uses M0).  Through the builtin the compiler either goes back to 64-bit lane addresses (a quarter-rate
@@ -340,18 +332,44 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // A fragments of sub-tiles 0 .. HM-1 (set 0) and HM .. TM-1 (set 1); B fragments of the k half 0 and 1
   Frag fa[2][HM];
   u32x4 fb[2][TN];
-  auto read_a = [&](int stage, auto ksc, auto hc, auto xc) {
-    constexpr int ks = decltype(ksc)::value, h = decltype(hc)::value, x = decltype(xc)::value;
-    fa[h][x] = *reinterpret_cast<const Frag*>(lds + stage_off(stage) + a_lane + (h * HM + x) * 16 * kDmaRowB + pos[ks]);
+  // Per-stage lane addresses, kept in registers: a stage sits up to 3 x 64 KB into LDS, more than the offset field of
+  // an LDS instruction holds, and the compiler would otherwise add the stage offset once per read.
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  uint32_t a_st[NS][2], b_st[NS][2], b_tr_st[NS][B_KC ? 1 : TN];
+#pragma unroll
+  for (int st = 0; st < NS; ++st) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      a_st[st][ks] = lds0 + st * STAGEB + a_lane + pos[ks];
+      b_st[st][ks] = lds0 + st * STAGEB + b_lane + pos[ks];
+      asm volatile("" : "+v"(a_st[st][ks]), "+v"(b_st[st][ks]));
+    }
+#pragma unroll
+    for (int x = 0; x < (B_KC ? 1 : TN); ++x) {
+      b_tr_st[st][x] = b_tr[B_KC ? 0 : x] + st * STAGEB;
+      asm volatile("" : "+v"(b_tr_st[st][x]));
+    }
+  }
+  typedef __attribute__((address_space(3))) const char* LdsPtr;
+  // `stc`: the stage as a constant (IntC<0 .. NS-1>) or IntC<-1> with its byte offset in stage_bytes
+  auto read_a = [&](auto stc, int stage_bytes, auto ksc, auto hc, auto xc) {
+    constexpr int ST = decltype(stc)::value, ks = decltype(ksc)::value, h = decltype(hc)::value, x = decltype(xc)::value;
+    if constexpr (ST >= 0)
+      fa[h][x] = *reinterpret_cast<__attribute__((address_space(3))) const Frag*>((LdsPtr)(uintptr_t)a_st[ST][ks] + (h * HM + x) * 16 * kDmaRowB);
+    else
+      fa[h][x] = *reinterpret_cast<const Frag*>(lds + stage_bytes + a_lane + (h * HM + x) * 16 * kDmaRowB + pos[ks]);
   };
-  auto read_b = [&](int stage, auto ksc, auto xc) {
-    constexpr int ks = decltype(ksc)::value, x = decltype(xc)::value;
-    const int sb = stage_off(stage);
+  auto read_b = [&](auto stc, int stage_bytes, auto ksc, auto xc) {
+    constexpr int ST = decltype(stc)::value, ks = decltype(ksc)::value, x = decltype(xc)::value;
     if constexpr (B_KC) {
-      fb[ks][x] = *reinterpret_cast<const u32x4*>(lds + sb + b_lane + x * 16 * kDmaRowB + pos[ks]);
+      if constexpr (ST >= 0)
+        fb[ks][x] = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>((LdsPtr)(uintptr_t)b_st[ST][ks] + x * 16 * kDmaRowB);
+      else
+        fb[ks][x] = *reinterpret_cast<const u32x4*>(lds + stage_bytes + b_lane + x * 16 * kDmaRowB + pos[ks]);
     } else {
-      const u32x2 lo = lds_read_tr16_b64<(32 * ks) * RBB>(b_tr[x] + sb);
-      const u32x2 hi = lds_read_tr16_b64<(32 * ks + 4) * RBB>(b_tr[x] + sb);
+      const uint32_t addr = ST >= 0 ? b_tr_st[ST >= 0 ? ST : 0][B_KC ? 0 : x] : b_tr[x] + stage_bytes;
+      const u32x2 lo = lds_read_tr16_b64<(32 * ks) * RBB>(addr);
+      const u32x2 hi = lds_read_tr16_b64<(32 * ks + 4) * RBB>(addr);
       fb[ks][x] = u32x4{lo[0], lo[1], hi[0], hi[1]};
     }
   };
@@ -366,19 +384,19 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     constexpr int s = decltype(sc)::value;
     if (s < nk) {
       const KBase kbase = bases_of(s);
-      static_for<0, NDMA>([&](auto jc) { issue(s, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
+      static_for<0, NDMA>([&](auto jc) { issue(s * STAGEB, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
     }
   });
   if (nk >= NS) {
     const KBase kbase = bases_of(NS - 1);
-    static_for<0, HALF>([&](auto jc) { issue(NS - 1, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
+    static_for<0, HALF>([&](auto jc) { issue((NS - 1) * STAGEB, kbase, jc, IntC<(decltype(jc)::value == 0)>{}); });
     FGK_WAIT_VM(NDMA * (NS - 2) + HALF);  // K step 0 has landed
   } else {
     FGK_WAIT_VM(0);
   }
   __builtin_amdgcn_s_barrier();
-  static_for<0, HM>([&](auto xc) { read_a(0, IntC<0>{}, IntC<0>{}, xc); });
-  static_for<0, TN>([&](auto xc) { read_b(0, IntC<0>{}, xc); });
+  static_for<0, HM>([&](auto xc) { read_a(IntC<0>{}, 0, IntC<0>{}, IntC<0>{}, xc); });
+  static_for<0, TN>([&](auto xc) { read_b(IntC<0>{}, 0, IntC<0>{}, xc); });
   wait_reads(IntC<0>{});
   __builtin_amdgcn_sched_barrier(0);
 
@@ -390,7 +408,15 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // first half of the DMAs of K step kb+NS (into the stage this step has just finished reading).  LATER = DMAs
   // that may still be in flight once K step kb+1 has landed: those of the K steps behind it, which retire in
   // order after it.
-  auto k_step = [&](int kb, auto tail_c, auto head_c, auto later_c) {
+  // ST: the stage of K step kb when the caller knows it at compile time (the unrolled part of the loop), else -1.
+  auto k_step = [&](int kb, auto st_c, auto tail_c, auto head_c, auto later_c) {
+    constexpr int ST = decltype(st_c)::value;
+    // LDS byte offset of the stage of K step kb + d
+    auto stage_of = [&](auto dc) {
+      constexpr int d = decltype(dc)::value;
+      if constexpr (ST >= 0) return ((ST + d) % NS) * STAGEB;
+      else return stage_off(kb + d);
+    };
     constexpr bool REFILL_TAIL = decltype(tail_c)::value != 0;
     constexpr bool REFILL_HEAD = decltype(head_c)::value != 0;
     constexpr int LATER = decltype(later_c)::value;
@@ -404,18 +430,19 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
       constexpr int NRA = HM, NRB = nh == 0 ? TN : 0, NRD = NRA + NRB;
       constexpr int ND = (qt == 0 && REFILL_TAIL) ? NDMA - HALF : (qt == 3 && REFILL_HEAD) ? HALF : 0;
       constexpr int NOPS = NRD + ND, OPM = (NOPS + NMF - 1) / NMF;
-      const int rstage = qt == 3 ? kb + 1 : kb;
+      const int rstage = stage_of(IntC<(qt == 3 ? 1 : 0)>{});
+      constexpr int RST = ST >= 0 ? (ST + (qt == 3 ? 1 : 0)) % NS : -1;
       static_for<0, NMF>([&](auto xc) {
         constexpr int x = decltype(xc)::value;
         constexpr int il = x / TN, j = x % TN;
         MfmaK32<T>::mma(__builtin_bit_cast(Frag, fb[ks][j]), fa[h][il], acc[h * HM + il][j]);
         static_for<0, OPM>([&](auto oc) {
           constexpr int o = x * OPM + decltype(oc)::value;
-          if constexpr (o < NRA) read_a(rstage, IntC<nks>{}, IntC<nh>{}, IntC<(o < NRA ? o : 0)>{});
-          else if constexpr (o < NRD) read_b(rstage, IntC<nks>{}, IntC<(o < NRD ? o - NRA : 0)>{});
+          if constexpr (o < NRA) read_a(IntC<RST>{}, rstage, IntC<nks>{}, IntC<nh>{}, IntC<(o < NRA ? o : 0)>{});
+          else if constexpr (o < NRD) read_b(IntC<RST>{}, rstage, IntC<nks>{}, IntC<(o < NRD ? o - NRA : 0)>{});
           else if constexpr (o < NOPS) {
-            if constexpr (qt == 0) issue(kb + NS - 1, kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{}, IntC<(o == NRD)>{});
-            else issue(kb + NS, kk_head, IntC<(o < NOPS ? o - NRD : 0)>{}, IntC<(o == NRD)>{});
+            if constexpr (qt == 0) issue(stage_of(IntC<NS - 1>{}), kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{}, IntC<(o == NRD)>{});
+            else issue(stage_of(IntC<NS>{}), kk_head, IntC<(o < NOPS ? o - NRD : 0)>{}, IntC<(o == NRD)>{});
           }
         });
         __builtin_amdgcn_sched_barrier(0);
@@ -430,18 +457,21 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
       __builtin_amdgcn_sched_barrier(0);
     });
   };
+  // the steady state, NS steps per trip so that the stage of every step is a constant of the code
   int kb = 0;
-  for (; kb < nk - NS; ++kb) k_step(kb, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{});
+  for (; kb + NS <= nk - NS; kb += NS)
+    static_for<0, NS>([&](auto sc) { k_step(kb + decltype(sc)::value, sc, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{}); });
+  for (; kb < nk - NS; ++kb) k_step(kb, IntC<-1>{}, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{});
   // the last NS steps (fewer when nk < NS), by the number r of K steps behind them: nothing new to request
   // except the second half of the last step, and ever fewer DMAs left in flight
   static_for<0, NS - 1>([&](auto ic) {
     constexpr int r = NS - 1 - decltype(ic)::value;
     if (kb == nk - 1 - r) {
-      k_step(kb, IntC<(r >= NS - 1 ? 1 : 0)>{}, IntC<0>{}, IntC<NDMA * cmin(NS - 2, r - 1)>{});
+      k_step(kb, IntC<-1>{}, IntC<(r >= NS - 1 ? 1 : 0)>{}, IntC<0>{}, IntC<NDMA * cmin(NS - 2, r - 1)>{});
       ++kb;
     }
   });
-  k_step(kb, IntC<0>{}, IntC<0>{}, IntC<0>{});
+  k_step(kb, IntC<-1>{}, IntC<0>{}, IntC<0>{}, IntC<0>{});
   mfma_drain(acc);
 
   finish(acc);
@@ -453,11 +483,8 @@ __global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ?
   int tm, tn;
   tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
   const int nk = (int)((g.K + kDmaBK - 1) / kDmaBK);
-  // K-rotated start per XCD (workgroups go to the XCDs round-robin by id): the eight XCDs then read eight different
-  // column ranges of the operands at any one time; the tiles of one XCD stay in step and keep sharing panels in its L2
-  const int krot = g.k_stagger ? (int)((blockIdx.x & 7u) * (unsigned)nk / 8u) : 0;
   dma_tile_mainloop<T, B_KC, BM, BN, NS, RAGGED>(
-      g, lds, tm, tn, 0, nk, [&](f32x4 (&acc)[BM / 32][BN / 32]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); }, krot);
+      g, lds, tm, tn, 0, nk, [&](f32x4 (&acc)[BM / 32][BN / 32]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); });
 }
 // Stream-K over 128x128 tiles with the main loop above: the (tile, K step) units, tile-major, are dealt
 // in equal contiguous ranges to the workgroups; a tile split between workgroups is finished by whichever

@@ -53,7 +53,6 @@ struct GemmArgs {
   float alpha, beta;
   int tiles_m, tiles_n;
   int tile_base;        // first tile id of a data-parallel launch (tiles below it belong to stream-K)
-  int k_stagger;        // direct-to-LDS data-parallel kernels: every XCD starts its K loop at a different eighth of K
   int k_ragged;         // direct-to-LDS kernels, K not a multiple of 64: valid k of the last K step (a multiple of 8), else 0
   const void* zeros;    // ... and 4 KB of zeros in device memory, the source of that step's chunks past K
   // stream-K (unused by the data-parallel launch)

@@ -361,28 +361,6 @@ def test_mm_addmm_tile_sizes(gpu, fg_env, M, N, K, dtype, tile, b_col_major):
     assert torch.equal(flag_gems.mm(a, b), c)
 
 
-@pytest.mark.parametrize("tile", ["256x256", "128x256", "128x128", None])
-@pytest.mark.parametrize("M,N,K", [(1100, 2824, 512), (1024, 4096, 576), (2040, 4104, 1088), (512, 1024, 4096)])
-@pytest.mark.parametrize("b_col_major", [False, True])
-def test_mm_k_rotated_start(gpu, fg_env, M, N, K, tile, b_col_major):
-    """FG_GEMM_KSTAGGER=1: every XCD starts its K loop at a different eighth of K (8, 9, 17 and 64 K steps here).  Only
-    the order of the sum changes, so the result stays within the reference's tolerance and is the same on every run."""
-    fg_env.setenv("FG_GEMM_KSTAGGER", "1")
-    if tile is not None:
-        fg_env.setenv("FG_GEMM_TILE", tile)
-    dtype = torch.bfloat16
-    torch.manual_seed(K + M)
-    a = torch.randn(M, K, dtype=dtype, device=gpu)
-    b = _operand(K, N, dtype, gpu, b_col_major)
-    rows = torch.tensor([0, 1, 127, 128, 255, 256, M // 2, M - 129, M - 1], device=gpu)
-    c = flag_gems.mm(a, b)
-    gems_assert_close(c[rows], O.mm(a[rows], b), dtype, reduce_dim=K)
-    bias = torch.randn(N, dtype=dtype, device=gpu)
-    d = flag_gems.addmm(bias, a, b, alpha=0.5, beta=2.0)
-    gems_assert_close(d[rows], O.addmm(bias, a[rows], b, alpha=0.5, beta=2.0), dtype, reduce_dim=K)
-    assert torch.equal(flag_gems.mm(a, b), c)
-
-
 def test_mm_full_size_properties(gpu):
     """8192^3 bf16 (the benchmark shape): sampled rows against the oracle, plus linearity in A."""
     torch.manual_seed(3)
