@@ -273,7 +273,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     // instruction issued here is a slot the wave's next MFMA waits for.
     if constexpr (decltype(first_c)::value != 0 || (jj & 3) == 0) {
       const uint32_t m0v = (uint32_t)(uintptr_t)FGK_LDSP(l);
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory", "m0");
     }
     const uint32_t off = IS_A ? a_off[jj] : b_off[jj];
     if constexpr (RAGGED) {
