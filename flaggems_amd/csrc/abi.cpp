@@ -33,9 +33,8 @@ void load_options() {
   o.gemm_sk_even = getenv("FG_GEMM_SK_EVEN") != nullptr;
   if (const char* e = getenv("FG_GEMM_TILE")) {
     int a = 0, b = 0;
-    char c = 0;
-    if (sscanf(e, "%dx%d%c", &a, &b, &c) >= 2 && a > 0 && b > 0) {
-      o.gemm_tile_bm = a; o.gemm_tile_bn = b; o.gemm_tile_deep = c != 's';
+    if (sscanf(e, "%dx%d", &a, &b) == 2 && a > 0 && b > 0) {
+      o.gemm_tile_bm = a; o.gemm_tile_bn = b;
     }
   }
   o.skinny_no_lds = getenv("FG_SKINNY_NO_LDS") != nullptr;

@@ -25,8 +25,7 @@ int fg_check_launch(const char* what);
 struct FgOptions {
   bool gemm_no_dma;       // FG_GEMM_NO_DMA: keep 16-bit GEMMs off the direct-to-LDS kernels
   bool gemm_sk_even;      // FG_GEMM_SK_EVEN: stream-K always in equal shares
-  int gemm_tile_bm, gemm_tile_bn;  // FG_GEMM_TILE=256x128[s]: forced direct-to-LDS tile (bm == 0: not forced)
-  bool gemm_tile_deep;    // ... false with the "s" suffix (two LDS stages)
+  int gemm_tile_bm, gemm_tile_bn;  // FG_GEMM_TILE=256x128: forced direct-to-LDS tile (bm == 0: not forced)
   bool skinny_no_lds;     // FG_SKINNY_NO_LDS
   bool skinny_rows64;     // FG_SKINNY_ROWS64
   int skinny_tile;        // FG_SKINNY_TILE=16|32 (0: not set)

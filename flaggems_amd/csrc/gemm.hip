@@ -19,9 +19,9 @@ int streamk_launch(GemmArgs g, int dtype, int amode, int bmode, void* workspace,
 bool dma_supported(const GemmArgs& g, int elem_bytes);
 bool dma_supported_ragged(const GemmArgs& g, int elem_bytes);
 const void* dma_zeros();
-double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep);
+double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn);
 double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, int* workers);
-int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st);
+int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st);
 int dma_streamk_launch(GemmArgs g, int dtype, void* workspace, size_t workspace_bytes, int num_cu, hipStream_t st);
 
 int num_cus(int device) {
@@ -122,10 +122,9 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
     // the machine best (even a lone 128x128 workgroup per CU runs twice as fast as the register-staged kernel).
     if (amode != LOAD_GEN && dma_supported(g, (int)sizeof(T)) && !fg_options().gemm_no_dma) {
       int bm = 256, bn = 256;
-      bool deep = false;
-      dma_pick_tile(g.M, g.N, g.K, num_cu, &bm, &bn, &deep);
+      dma_pick_tile(g.M, g.N, g.K, num_cu, &bm, &bn);
       set_tiles(g, bm, bn, BK);
-      return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, deep, st);
+      return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, bm, bn, st);
     }
     // The 256x256 tile halves LDS and L2 traffic per flop; it pays once it can fill the machine.
     const int64_t big_tiles = fg_cdiv(g.M, 256) * fg_cdiv(g.N, 256);
@@ -136,7 +135,7 @@ int run_dp(GemmArgs g, int amode, int bmode, int num_cu, hipStream_t st) {
         const bool big = big_tiles * 10 >= (int64_t)num_cu * 9;
         set_tiles(g, big ? 256 : 128, big ? 256 : 128, BK);
         g.k_ragged = (int)(g.K % kDmaBKHost);
-        return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, big ? 256 : 128, big ? 256 : 128, true, st);
+        return dma_launch(g, std::is_same<T, bf16_t>::value ? FG_BF16 : FG_F16, big ? 256 : 128, big ? 256 : 128, st);
       }
     }
     if (amode != LOAD_GEN && amode != LOAD_KU && amode != LOAD_MNU && g.M >= 256 && g.N >= 256 && big_tiles * 10 >= (int64_t)num_cu * 9) {
@@ -263,9 +262,8 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
           const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && !fg_options().gemm_no_dma;
           if (dma) {
             int bm, bn, workers;
-            bool deep;
             use_streamk = tiles <= cu && tiles * iters >= 4 * (int64_t)cu &&
-                          dma_streamk_plan(tiles, iters, cu, &workers) < dma_pick_tile(M, N, K, cu, &bm, &bn, &deep);
+                          dma_streamk_plan(tiles, iters, cu, &workers) < dma_pick_tile(M, N, K, cu, &bm, &bn);
           } else {
             // (the stream-K kernels have no element-aligned vector modes: such operands stay data-parallel)
             use_streamk = !vec_unaligned && tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;

@@ -72,13 +72,13 @@ static int launch_dma_b(const GemmArgs& g, hipStream_t st) {
 // still runs at the lone rate).  A ragged round behind full ones starts while their stragglers finish: it adds
 // 0.55 to 1.0 of a lone round on top of that.  Constants measured on MI355X, bf16, K = 4096, weights not resident in
 // the caches, 16 to 512 tiles of each size.
-struct DmaTileCost { int bm, bn; bool deep; double lone, loaded; };
+struct DmaTileCost { int bm, bn; double lone, loaded; };
 static const DmaTileCost kDmaTiles[] = {
-    {256, 256, false, 1.31, 1.75},
-    {192, 256, false, 1.20, 1.375},
-    {256, 128, true, 0.77, 0.97},
-    {128, 256, true, 0.84, 1.00},
-    {128, 128, true, 0.58, 0.59},
+    {256, 256, 1.31, 1.75},
+    {192, 256, 1.20, 1.375},
+    {256, 128, 0.77, 0.97},
+    {128, 256, 0.84, 1.00},
+    {128, 128, 0.58, 0.59},
 };
 static double dma_dp_cost(const DmaTileCost& t, int64_t M, int64_t N, int64_t K, int num_cu) {
   const int64_t tiles = fg_cdiv(M, t.bm) * fg_cdiv(N, t.bn);
@@ -95,17 +95,17 @@ static bool dma_tile_exists(int bm, int bn) {
 }
 
 // Tile choice: the candidate the model above finishes first.  Returns its estimated duration.
-double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn, bool* deep) {
+double dma_pick_tile(int64_t M, int64_t N, int64_t K, int num_cu, int* bm, int* bn) {
   const FgOptions& opt = fg_options();  // measurement aid: one of the tiles above forced
   if (opt.gemm_tile_bm > 0 && dma_tile_exists(opt.gemm_tile_bm, opt.gemm_tile_bn)) {
-    *bm = opt.gemm_tile_bm; *bn = opt.gemm_tile_bn; *deep = opt.gemm_tile_deep;
+    *bm = opt.gemm_tile_bm; *bn = opt.gemm_tile_bn;
     return 0.0;
   }
   double best = 0.0;
   bool have = false;
   for (const DmaTileCost& t : kDmaTiles) {
     const double c = dma_dp_cost(t, M, N, K, num_cu);
-    if (!have || c < best) { best = c; *bm = t.bm; *bn = t.bn; *deep = t.deep; have = true; }
+    if (!have || c < best) { best = c; *bm = t.bm; *bn = t.bn; have = true; }
   }
   return best;
 }
@@ -133,9 +133,9 @@ double dma_streamk_plan(int64_t sk_tiles, int64_t iters_per_tile, int num_cu, in
   return best;
 }
 
-// g.tiles_m / g.tiles_n must describe bm x bn tiles.  `deep`: as many LDS stages as one workgroup per CU can
-// hold (3 for 256x128 and 128x256, 4 for 128x128) instead of two.
-int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStream_t st) {
+// g.tiles_m / g.tiles_n must describe bm x bn tiles.  Every tile runs with as many LDS stages as one workgroup per CU
+// can hold: two for 256x256 and 192x256, three for 256x128 and 128x256, four for 128x128.
+int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, hipStream_t st) {
 #define FG_DMA(T)                                                                                         \
   do {                                                                                                    \
     if (g.k_ragged != 0) {                                                                                \
@@ -145,9 +145,9 @@ int dma_launch(const GemmArgs& g, int dtype, int bm, int bn, bool deep, hipStrea
     }                                                                                                     \
     if (bm == 256 && bn == 256) return launch_dma_b<T, 256, 256, 2>(g, st);                               \
     if (bm == 192 && bn == 256) return launch_dma_b<T, 192, 256, 2>(g, st);                               \
-    if (bm == 256 && bn == 128) return deep ? launch_dma_b<T, 256, 128, 3>(g, st) : launch_dma_b<T, 256, 128, 2>(g, st); \
-    if (bm == 128 && bn == 256) return deep ? launch_dma_b<T, 128, 256, 3>(g, st) : launch_dma_b<T, 128, 256, 2>(g, st); \
-    if (bm == 128 && bn == 128) return deep ? launch_dma_b<T, 128, 128, 4>(g, st) : launch_dma_b<T, 128, 128, 2>(g, st); \
+    if (bm == 256 && bn == 128) return launch_dma_b<T, 256, 128, 3>(g, st);                               \
+    if (bm == 128 && bn == 256) return launch_dma_b<T, 128, 256, 3>(g, st);                               \
+    if (bm == 128 && bn == 128) return launch_dma_b<T, 128, 128, 4>(g, st);                               \
   } while (0)
   if (dtype == FG_BF16) FG_DMA(bf16_t);
   else FG_DMA(f16_t);

@@ -333,10 +333,9 @@ def test_mm_addmm_k_not_a_multiple_of_64(gpu, M, N, K, dtype, b_col_major):
 # The direct-to-LDS kernel exists for five tile sizes; the library picks by how the tile count fills the
 # machine.  Each is forced in turn on ragged shapes (edge tiles in M and N; one to four K steps, which is fewer
 # than or as many as the LDS ring has stages, and seventeen) and, with no forcing, on shapes whose automatic
-# choice is the 128x128 and the 256x128 tile.  The two smaller tiles run with a ring of four / three stages;
-# an "s" appended forces their two-stage variants.
+# choice is the 128x128 and the 256x128 tile.  The smaller tiles run with a ring of three or four stages.
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("tile", ["256x256", "192x256", "256x128", "128x256", "128x128", "256x128s", "128x256s", "128x128s", None])
+@pytest.mark.parametrize("tile", ["256x256", "192x256", "256x128", "128x256", "128x128", None])
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 128), (1100, 4104, 64), (2040, 4104, 256), (1537, 2824, 192), (1100, 2824, 1088)])
 @pytest.mark.parametrize("b_col_major", [False, True])
 def test_mm_addmm_tile_sizes(gpu, fg_env, M, N, K, dtype, tile, b_col_major):
