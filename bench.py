@@ -139,12 +139,12 @@ def main():
     # same counters read for a plain 512 MiB copy (profiles/hbm_traffic_*.txt hold the runs and their commands)
     TRAFFIC = {
         "softmax_c2": 1073780000,
-        "fused_add_rms_norm_c1": 134350000,
+        "fused_add_rms_norm_c1": 134340000,
         "fused_add_rms_norm_c1_fp32": 268600000,
-        "mm_c3a_8192": 1746080000,
+        "mm_c3a_8192": 1772630000,
         "mm_c3b_skinny": 122520000,
-        "addmm_c3c": 711700000,
-        "flash_attn_c4": 785850000,
+        "addmm_c3c": 745590000,
+        "flash_attn_c4": 786030000,
         "flash_attn_decode": 1075240000,
     }
 

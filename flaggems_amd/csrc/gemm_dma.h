@@ -158,19 +158,22 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
       for (int jj = 0; jj < 2; ++jj) {
         const int j = 2 * jp + jj;
         const int c = col0 + wn * WTN + j * 16 + lg * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
         if (bias != nullptr) {
           T4 t = brow[j];
           if (!bcast && r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] = acc[i][j][e] * alpha + (float)t[e] * beta;
+          for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
         } else if (scale) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] *= alpha;
+          for (int e = 0; e < 4; ++e) v[e] *= alpha;
         }
 #pragma unroll
         for (int d = 0; d < 2; ++d) {
           typedef T T2 __attribute__((ext_vector_type(2)));
-          const T2 t = {(T)acc[i][j][2 * d], (T)acc[i][j][2 * d + 1]};
+          const T2 t = {(T)v[2 * d], (T)v[2 * d + 1]};
           pk[jj][d] = __builtin_bit_cast(unsigned, t);
         }
       }
@@ -180,6 +183,8 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
       swap_rows16x2(x0, y0, x1, y1);
       const int c = col0 + wn * WTN + (2 * jp + (lg & 1)) * 16 + (lg & 2) * 4;
       if (r < M && c < N) *reinterpret_cast<u32x4*>(C + r * g.scm + c) = u32x4{x0, x1, y0, y1};
+      // (keeps the scheduler from fetching every accumulator up front: 256 registers at once spill)
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -461,7 +466,12 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   int kb = 0;
   for (; kb + NS <= nk - NS; kb += NS)
     static_for<0, NS>([&](auto sc) { k_step(kb + decltype(sc)::value, sc, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{}); });
-  for (; kb < nk - NS; ++kb) k_step(kb, IntC<-1>{}, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{});
+  static_for<0, NS - 1>([&](auto) {  // up to NS - 1 steady-state steps are left
+    if (kb < nk - NS) {
+      k_step(kb, IntC<-1>{}, IntC<1>{}, IntC<1>{}, IntC<NDMA * (NS - 2)>{});
+      ++kb;
+    }
+  });
   // the last NS steps (fewer when nk < NS), by the number r of K steps behind them: nothing new to request
   // except the second half of the last step, and ever fewer DMAs left in flight
   static_for<0, NS - 1>([&](auto ic) {
