@@ -491,7 +491,7 @@ template <typename T, bool B_KC, int BM, int BN, int NS = 2, bool RAGGED = false
 __global__ __launch_bounds__(256, (2 * dma_lds_bytes(BM, BN, NS) <= 160 * 1024 ? 2 : 1)) void gemm_dma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   int tm, tn;
-  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn);
+  tile_coords(blockIdx.x + g.tile_base, g.tiles_m, g.tiles_n, tm, tn, B_KC ? 2 : 4);
   const int nk = (int)((g.K + kDmaBK - 1) / kDmaBK);
   dma_tile_mainloop<T, B_KC, BM, BN, NS, RAGGED>(
       g, lds, tm, tn, 0, nk, [&](f32x4 (&acc)[BM / 32][BN / 32]) { dma_tile_epilogue<T, BM, BN>(g, tm, tn, acc); });

@@ -326,12 +326,48 @@ template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_GEN> {
 };
 
 // ---------------------------------------------------------------------------------------------
-// tile id -> (tile_m, tile_n).  Workgroups are dispatched round-robin over the 8 XCDs, each with
-// its own L2: ids congruent mod 8 are first made consecutive, then walked in column-major groups
-// of GROUP_M tile rows, so the tiles one XCD works on at any time share A and B panels.
+// tile id -> (tile_m, tile_n), a bijection on [0, tiles_m * tiles_n).  Workgroups are dispatched
+// round-robin over the 8 XCDs (XCD = id mod 8), each with its own L2 and 32 CUs, and in id order
+// within an XCD.
+//
+// Regular grids (tiles_m a multiple of 8, tiles_n of 4): the grid is cut into sub-blocks of 8 x 4
+// tiles, one per XCD and round, so the 32 tiles an XCD works on at any time share 8 A panels and
+// 4 B panels in its L2.  The 8 sub-blocks of a round are neighbours, 2 x 4 of them = 16 x 16 tiles,
+// and rounds walk strips of 16 tile rows back and forth: a round needs as few distinct rows of A
+// and columns of B as 256 tiles can (the memory-side cache holds them while the 8 XCDs fetch
+// them one after the other), and consecutive rounds share their A rows, or their B columns at the
+// turn of a strip.  A last partial round deals its sub-blocks to the XCDs in equal contiguous parts.
+//
+// Other grids: ids congruent mod 8 are made consecutive, then walked in column-major groups of
+// 8 tile rows.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int XCDS = 8, GROUP_M = 8;
+__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int& tm, int& tn, int strip_rows = 2) {
+  constexpr int XCDS = 8, SUB_M = 8, SUB_N = 4, PER = SUB_M * SUB_N;
+  if (tiles_m % SUB_M == 0 && tiles_n % SUB_N == 0) {
+    const int sm_count = tiles_m / SUB_M, sn_count = tiles_n / SUB_N, nsub = sm_count * sn_count;
+    const int x = id % XCDS, turn = id / XCDS;
+    const int full = nsub / XCDS;  // rounds in which every XCD has a sub-block of its own
+    int q, s;
+    if (turn < full * PER) {
+      q = (turn / PER) * XCDS + x;
+      s = turn % PER;
+    } else {
+      const int rem = nsub - full * XCDS;  // 1..7 sub-blocks, PER * rem / 8 turns per XCD
+      const int u = x * (PER / XCDS * rem) + (turn - full * PER);
+      q = full * XCDS + u / PER;
+      s = u % PER;
+    }
+    const int strip = q / (strip_rows * sn_count);
+    const int left = sm_count - strip_rows * strip;
+    const int rows = left < strip_rows ? left : strip_rows;
+    const int r = q - strip * strip_rows * sn_count;
+    int sn = r / rows;
+    if (strip & 1) sn = sn_count - 1 - sn;
+    tm = (strip * strip_rows + r % rows) * SUB_M + s % SUB_M;
+    tn = sn * SUB_N + s / SUB_M;
+    return;
+  }
+  constexpr int GROUP_M = 8;
   const int total = tiles_m * tiles_n;
   const int per_xcd = total / XCDS;
   int t = id;

@@ -360,6 +360,27 @@ def test_mm_addmm_tile_sizes(gpu, fg_env, M, N, K, dtype, tile, b_col_major):
     assert torch.equal(flag_gems.mm(a, b), c)
 
 
+@pytest.mark.parametrize("tile", ["256x256", "128x128", None])
+@pytest.mark.parametrize("M,N,K", [(8192, 8192, 64), (4096, 3072, 128), (6144, 5120, 64), (2048, 9216, 64), (4096, 11008, 64),
+                                   (10240, 1024, 64), (256, 12288, 192)])
+def test_mm_every_tile_is_written_once(gpu, fg_env, M, N, K, tile):
+    """The workgroup id -> output tile map is a bijection on every kind of tile grid it treats differently (multiples of
+    the 8 x 4 sub-blocks with whole and partial rounds, an odd number of sub-block rows, a single row of them, grids that
+    are not multiples): an output pre-filled with NaN holds the whole product afterwards, checked against the oracle."""
+    if tile is None:
+        fg_env.delenv("FG_GEMM_TILE", raising=False)
+    else:
+        fg_env.setenv("FG_GEMM_TILE", tile)
+    torch.manual_seed(N + K)
+    dtype = torch.bfloat16
+    a = torch.randn(M, K, dtype=dtype, device=gpu)
+    b = _operand(K, N, dtype, gpu, True)
+    c = torch.full((M, N), float("nan"), dtype=dtype, device=gpu)
+    flag_gems.mm_out(a, b, out=c)
+    assert not torch.isnan(c).any()
+    gems_assert_close(c, O.mm(a, b), dtype, reduce_dim=K)
+
+
 def test_mm_full_size_properties(gpu):
     """8192^3 bf16 (the benchmark shape): sampled rows against the oracle, plus linearity in A."""
     torch.manual_seed(3)
