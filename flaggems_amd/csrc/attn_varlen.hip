@@ -43,11 +43,18 @@ template <> struct AttnMfma<bf16_t> {
   static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // 16x16 outputs over 32 k: A = 16 rows x 8 k per lane group of 16, B likewise by column, C column-major by lane
+  static __device__ __forceinline__ f32x4 mma16(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
 };
 template <> struct AttnMfma<f16_t> {
   typedef f16x8 Frag;
   static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mma16(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -756,7 +763,7 @@ int launch_async(const AttnArgs& a, dim3 grid, hipStream_t st) {
 template <typename T>
 int attn_dispatch(const AttnArgs& a, dim3 grid, hipStream_t st) {
   const int D = a.p.D;
-  if (a.use_fast) return D == 64 ? launch_pipe<T, 64, 1>(a, grid, st) : launch_pipe<T, 128, 1>(a, grid, st);
+  if (a.use_fast) return D == 64 ? launch_pipe<T, 64>(a, grid, st) : launch_pipe<T, 128>(a, grid, st);
   if (a.use_async) {
     if (a.nw == 8) {
       switch (D) {
