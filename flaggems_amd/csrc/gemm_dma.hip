@@ -66,26 +66,38 @@ static int launch_dma_b(const GemmArgs& g, hipStream_t st) {
   return g.sbk == 1 ? launch_dma_t<T, true, BM, BN, NS, RAGGED>(g, st) : launch_dma_t<T, false, BM, BN, NS, RAGGED>(g, st);
 }
 
-// Duration model of a data-parallel launch, in microseconds.  A CU holds one workgroup, so the tiles run in rounds
-// of num_cu.  A K step of a round that is the whole launch costs `lone` when few CUs are busy and `loaded` when all
-// are (the matrix cores then share the power budget); in between the cost follows the cube of the fill (half a round
-// still runs at the lone rate).  A ragged round behind full ones starts while their stragglers finish: it adds
-// 0.55 to 1.0 of a lone round on top of that.  Constants measured on MI355X, bf16, K = 4096, weights not resident in
-// the caches, 16 to 512 tiles of each size.
-struct DmaTileCost { int bm, bn; double lone, loaded; };
+// Duration model of a data-parallel launch, in microseconds.  A CU holds `per_cu` workgroups of a tile size, so the
+// tiles run in rounds of per_cu * num_cu.  A K step of a round that is the whole launch costs `lone` when few CUs are
+// busy and `loaded` when all are (the matrix cores then share the power budget); in between the cost follows the cube
+// of the fill (half a round still runs at the lone rate).  A ragged round behind full ones starts while their
+// stragglers finish: it adds 0.70 to 0.95 of a lone round on top of that.  Constants measured on MI355X on sustained
+// clocks, bf16, K = 4096, weights not resident in the caches, 32 to 1024 tiles of each size (us per K step and
+// round: 256x256 1.38 at 32-192 tiles, 1.57 at 256, 1.51-1.57 per round at 512-1024; 128x128 0.57 up to 256 tiles,
+// 0.91 at 320, 0.94 at 384, 1.05 at 512, 1.00 per 512 tiles beyond).
+struct DmaTileCost { int bm, bn, per_cu; double lone, loaded; };
 static const DmaTileCost kDmaTiles[] = {
-    {256, 256, 1.31, 1.75},
-    {192, 256, 1.20, 1.375},
-    {256, 128, 0.77, 0.97},
-    {128, 256, 0.84, 1.00},
-    {128, 128, 0.58, 0.59},
+    {256, 256, 1, 1.38, 1.55},
+    {192, 256, 1, 1.25, 1.26},
+    {256, 128, 1, 0.78, 0.88},
+    {128, 256, 1, 0.835, 0.89},
+    {128, 128, 2, 0.57, 1.02},
 };
 static double dma_dp_cost(const DmaTileCost& t, int64_t M, int64_t N, int64_t K, int num_cu) {
   const int64_t tiles = fg_cdiv(M, t.bm) * fg_cdiv(N, t.bn);
-  const int64_t full = tiles / num_cu, last = tiles % num_cu;
-  const double f = (double)last / num_cu;
+  const int64_t cap = (int64_t)num_cu * t.per_cu;
+  const int64_t full = tiles / cap, last = tiles % cap;
+  const double f = (double)last / (double)cap;
   double steps = (double)full * t.loaded;
-  if (last > 0) steps += (full > 0 ? t.lone * (0.55 + 0.45 * f) : t.lone) + (t.loaded - t.lone) * f * f * f;
+  if (last > 0) {
+    const double behind = full > 0 ? 0.70 + 0.25 * f : 1.0;
+    if (t.per_cu == 1) {
+      steps += t.lone * behind + (t.loaded - t.lone) * f * f * f;
+    } else {
+      // two workgroups on a CU run at little more than half speed each: the cost steps up where the second ones arrive
+      const double part = last <= num_cu ? t.lone : 0.90 + 0.15 * (double)(last - num_cu) / (double)num_cu;
+      steps += part * behind;
+    }
+  }
   return steps * (double)(K / kDmaBK);
 }
 static bool dma_tile_exists(int bm, int bn) {
