@@ -141,10 +141,10 @@ def main():
         "softmax_c2": 1073780000,
         "fused_add_rms_norm_c1": 134340000,
         "fused_add_rms_norm_c1_fp32": 268600000,
-        "mm_c3a_8192": 1772630000,
-        "mm_c3b_skinny": 122520000,
+        "mm_c3a_8192": 1771210000,
+        "mm_c3b_skinny": 122530000,
         "addmm_c3c": 745590000,
-        "flash_attn_c4": 786030000,
+        "flash_attn_c4": 770080000,
         "flash_attn_decode": 1075240000,
     }
 
