@@ -843,11 +843,13 @@ bool decode_setup(const FgFlashParams& p, DecodeArgs* d, bool mixed = false) {
 }
 // A batch of at least four sequences with max_seqlen_q > 1 is treated as mixed: the single-token kernel takes the
 // sequences with one query token (it streams K/V 2-3 times faster than the prefill kernels do for one row, and
-// splits long sequences), the prefill kernel skips them.  Both read the lengths on the device; a batch without
-// such sequences pays two launches of workgroups that leave at once.
+// splits long sequences), the prefill kernel skips them.  Both read the lengths on the device; a ragged batch without
+// such sequences pays two launches of workgroups that leave at once (a uniform batch is recognised on the host).
 bool mixed_batch(const FgFlashParams& p) {
   if (p.max_seqlen_q <= 1 || p.batch < 4) return false;
   if (fg_options().attn_mixed >= 0) return fg_options().attn_mixed != 0;
+  // every sequence as long as the longest: none has a single query token
+  if ((int64_t)p.total_q >= (int64_t)p.batch * p.max_seqlen_q) return false;
   return true;
 }
 }  // namespace
