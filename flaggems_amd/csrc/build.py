@@ -10,6 +10,8 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
 PKG = os.path.dirname(HERE)
 OUT = os.path.join(PKG, "libfg_mi355.so")
 OBJ_DIR = os.path.join(HERE, "build")
@@ -30,6 +32,10 @@ SOURCES = [
     "attn_varlen.hip",
     "probe.hip",
 ]
+
+# Sources whose kernels issue memory instructions from inline asm: the compiler does not keep the scalar-register
+# wait states for those, so their device assembly is kept (-save-temps) and scanned by isa_check.py.
+ASM_CHECKED = {"gemm_dma.hip", "attn_varlen.hip"}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -59,12 +65,36 @@ def _compile(src, force):
     if not force and not _newer([path] + headers, obj):
         return obj, ""
     lang = ["-x", "hip"] if src.endswith(".hip") else []
-    cmd = [HIPCC] + FLAGS + lang + ["-c", path, "-o", obj]
+    keep = ["-save-temps=obj"] if src in ASM_CHECKED else []
+    cmd = [HIPCC] + FLAGS + keep + lang + ["-c", path, "-o", obj]
     p = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(l for l in (p.stdout + p.stderr).splitlines() if "packed-fp32-ops" not in l)
     if p.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    if keep:
+        _check_wait_states(src, obj)
     return obj, log
+
+
+def _check_wait_states(src, obj):
+    """Scan the device assembly the object was assembled from; drop the other intermediate files."""
+    import isa_check
+
+    stem = os.path.join(OBJ_DIR, os.path.splitext(src)[0])
+    asm = stem + "-hip-amdgcn-amd-amdhsa-gfx950.s"
+    if not os.path.exists(asm):
+        os.remove(obj)
+        raise RuntimeError("no device assembly for %s at %s: the wait-state check cannot run" % (src, asm))
+    hits = isa_check.check_file(asm)
+    for f in os.listdir(OBJ_DIR):
+        full = os.path.join(OBJ_DIR, f)
+        if full != asm and full != obj and (f.startswith(os.path.basename(stem) + "-") or f.startswith(src + "-")):
+            os.remove(full)
+    if hits:
+        os.remove(obj)  # a later build without --force must not link it
+        lines = ["  %s: %s  <- %s" % (k[:70], line, why) for k, _, line, why in hits[:10]]
+        raise RuntimeError("%s: %d memory instruction(s) read a scalar register too early after it was written "
+                           "(see isa_check.py):\n%s" % (src, len(hits), "\n".join(lines)))
 
 
 def build(force=False, jobs=None, verbose=True):

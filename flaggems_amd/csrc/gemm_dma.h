@@ -261,6 +261,15 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
   };
+  // A scalar register written by a vector instruction (v_readfirstlane) may be read by a memory instruction only
+  // five wait states later.  The compiler keeps that distance for the loads it emits itself, but it cannot see
+  // that the asm of issue() is such a load.  So the tile's two bases are made scalar once, here, with the wait
+  // states behind them; what bases_of() derives from them is scalar arithmetic on scalar registers, which has no
+  // such rule.  (The tile's row and column come from integer divisions, which run on the vector unit: without
+  // this, how far a v_readfirstlane lands ahead of the first copy is up to the instruction scheduler.)
+  a_base = uniform_ptr(a_base);
+  b_base = uniform_ptr(b_base);
+  asm volatile("s_nop 4" : "+s"(a_base), "+s"(b_base));
   struct KBase { const char* a; const char* b; bool last; };
   auto bases_of = [&](int kk) {
     return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step), RAGGED && kk == nk - 1};

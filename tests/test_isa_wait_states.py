@@ -1,0 +1,71 @@
+"""The wait-state scan that the library's build runs over the device assembly of its asm-issued copies
+(flaggems_amd/csrc/isa_check.py): known-answer cases on hand-written assembly, so that a scan that stops seeing
+the hazard (a regex that no longer matches, an off-by-one in the count) fails here and not on a GPU."""
+import importlib.util
+import os
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_spec = importlib.util.spec_from_file_location("fg_isa_check", os.path.join(ROOT, "flaggems_amd", "csrc", "isa_check.py"))
+isa_check = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(isa_check)
+
+
+def kernel(body, name="k0"):
+    return "%s:                ; @%s\n; %%bb.0:\n%s\n\ts_endpgm\n.Lfunc_end0:\n" % (name, name, body)
+
+
+COPY = "\tglobal_load_lds_dwordx4 v47, s[6:7] offset:1024"
+
+
+@pytest.mark.parametrize("between,expect", [(0, 1), (1, 1), (4, 1), (5, 0), (9, 0)])
+def test_readfirstlane_then_copy_needs_five_wait_states(between, expect):
+    body = "\tv_readfirstlane_b32 s6, v36\n" + "\tv_add_u32_e32 v1, v2, v3\n" * between + COPY
+    assert len(isa_check.scan(kernel(body))) == expect
+
+
+def test_both_halves_of_the_base_are_seen():
+    body = "\tv_readfirstlane_b32 s6, v36\n\tv_readfirstlane_b32 s7, v37\n" + COPY
+    hits = isa_check.scan(kernel(body))
+    assert len(hits) == 2 and all("global_load_lds" in h[2] for h in hits)
+
+
+@pytest.mark.parametrize("nop,expect", [(3, 1), (4, 0)])
+def test_s_nop_counts_as_its_argument_plus_one(nop, expect):
+    body = "\tv_readlane_b32 s7, v3, 5\n\ts_nop %d\n%s" % (nop, COPY)
+    assert len(isa_check.scan(kernel(body))) == expect
+
+
+def test_scalar_arithmetic_on_the_base_is_no_hazard():
+    body = "\ts_add_u32 s6, s6, 0x80\n\ts_addc_u32 s7, s7, 0\n" + COPY
+    assert isa_check.scan(kernel(body)) == []
+
+
+def test_other_registers_do_not_count():
+    body = "\tv_readfirstlane_b32 s8, v36\n" + COPY + "\n\tglobal_load_dwordx4 v[0:3], v8, s[10:11]"
+    assert isa_check.scan(kernel(body)) == []
+
+
+def test_compare_into_scalar_pair_then_store_with_that_base():
+    body = "\tv_cmp_lt_u32_e64 s[6:7], v1, v2\n\tglobal_store_dword v0, v1, s[6:7]"
+    assert len(isa_check.scan(kernel(body))) == 1
+
+
+def test_m0_needs_one_wait_state_before_an_lds_direct_load():
+    assert len(isa_check.scan(kernel("\ts_mov_b32 m0, s9\n" + COPY))) == 1
+    assert isa_check.scan(kernel("\ts_mov_b32 m0, s9\n\ts_nop 0\n" + COPY)) == []
+    # an ordinary load does not read M0
+    assert isa_check.scan(kernel("\ts_mov_b32 m0, s9\n\tglobal_load_dwordx4 v[0:3], v8, s[6:7]")) == []
+
+
+def test_every_function_and_every_exit_is_scanned():
+    early = "\ts_cbranch_scc1 .LBB0_2\n\ts_endpgm\n.LBB0_2:\n\tv_readfirstlane_b32 s6, v36\n" + COPY
+    text = kernel("\ts_nop 0", "k0") + kernel(early, "k1")
+    hits = isa_check.scan(text)
+    assert [h[0] for h in hits] == ["k1"]
+
+
+def test_state_does_not_leak_between_functions():
+    text = kernel("\tv_readfirstlane_b32 s6, v36", "k0") + kernel(COPY, "k1")
+    assert isa_check.scan(text) == []
