@@ -52,6 +52,10 @@ namespace fgk {
 
 constexpr int kDmaRowB = 128;   // bytes of K per stage per A row
 constexpr int kDmaBK = 64;
+// Quarter steps of a K step that issue copies: 2 (quarter 3 and quarter 0, half of the copies each) for every tile,
+// or 3 (quarters 3, 0 and 1) for the 256x256 tile with two stages.  3 was measured 2-6 % faster on large products
+// and is switched off: it has run on a few large shapes only, not under the parity tests.
+constexpr int kDmaCopyRuns = 2;
 constexpr int dma_lds_bytes(int bm, int bn, int stages = 2) { return stages * (bm + bn) * kDmaRowB; }  // stages of (A tile + B tile)
 constexpr int cmin(int a, int b) { return a < b ? a : b; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
@@ -204,7 +208,17 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   constexpr int B_OPB = BN * kDmaRowB;             // B tile, one stage (64 k-rows of BN*2 bytes when N-contiguous)
   constexpr int STAGEB = A_OPB + B_OPB;
   constexpr int NA = BM / 32, NB = BN / 32;        // DMA instructions per wave, operand and stage
-  constexpr int NDMA = NA + NB, HALF = NDMA / 2;
+  constexpr int NDMA = NA + NB;
+  // The copies of one K step, by the quarter step that issues them: C3 in quarter 3 of the step NS steps earlier
+  // (whose stage has just been read for the last time), C0 and C1 in quarters 0 and 1 of the step after that one.
+  // The barrier of a K step puts the four waves back in step, so they reach these quarters together, and a copy
+  // holds the CU's address path for 16 cycles: the more quarters share the copies, the less the waves queue.
+  constexpr bool THREE_RUNS = kDmaCopyRuns == 3 && BM == 256 && BN == 256 && NS == 2 && !RAGGED;
+  constexpr int C3 = THREE_RUNS ? (B_KC ? 6 : 8) : NDMA / 2;
+  constexpr int C0 = THREE_RUNS ? 5 : NDMA - C3;
+  constexpr int C1 = NDMA - C3 - C0;
+  constexpr int HALF = C3;
+  static_assert(C0 > 0 && C1 >= 0, "copy split");
   constexpr int NMF = HM * TN;                     // MFMAs per quarter step
   constexpr int RBB = BN * 2;                      // N-contiguous B: bytes per k-row of the tile
   constexpr int CPRB = RBB / 16, RPI = 1024 / RBB; // ... chunks per k-row, k-rows per DMA instruction
@@ -418,8 +432,8 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // B sub-tiles over the k half ks, while the fragments of the next quarter are read: the other A half, and behind
   // an h = 1 quarter also the B fragments of the next k half (quarter 3 reads them from the next stage).  The
   // memory operations of a quarter, reads first, are spread over its MFMAs.
-  // REFILL_TAIL: quarter 0 issues the second half of the DMAs of K step kb+NS-1; REFILL_HEAD: quarter 3 issues the
-  // first half of the DMAs of K step kb+NS (into the stage this step has just finished reading).  LATER = DMAs
+  // REFILL_TAIL: quarters 0 and 1 issue the last C0 + C1 DMAs of K step kb+NS-1; REFILL_HEAD: quarter 3 issues the
+  // first C3 DMAs of K step kb+NS (into the stage this step has just finished reading).  LATER = DMAs
   // that may still be in flight once K step kb+1 has landed: those of the K steps behind it, which retire in
   // order after it.
   // ST: the stage of K step kb when the caller knows it at compile time (the unrolled part of the loop), else -1.
@@ -442,7 +456,8 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
       constexpr int ks = qt >> 1, h = qt & 1;
       constexpr int nks = ((qt + 1) & 3) >> 1, nh = (qt + 1) & 1;   // the quarter the reads are for
       constexpr int NRA = HM, NRB = nh == 0 ? TN : 0, NRD = NRA + NRB;
-      constexpr int ND = (qt == 0 && REFILL_TAIL) ? NDMA - HALF : (qt == 3 && REFILL_HEAD) ? HALF : 0;
+      constexpr int ND = (qt == 0 && REFILL_TAIL) ? C0 : (qt == 1 && REFILL_TAIL) ? C1 : (qt == 3 && REFILL_HEAD) ? C3 : 0;
+      constexpr int DONE = qt == 1 ? C3 + C0 : C3;  // copies of the tail's K step issued before this quarter
       constexpr int NOPS = NRD + ND, OPM = (NOPS + NMF - 1) / NMF;
       const int rstage = stage_of(IntC<(qt == 3 ? 1 : 0)>{});
       constexpr int RST = ST >= 0 ? (ST + (qt == 3 ? 1 : 0)) % NS : -1;
@@ -455,7 +470,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
           if constexpr (o < NRA) read_a(IntC<RST>{}, rstage, IntC<nks>{}, IntC<nh>{}, IntC<(o < NRA ? o : 0)>{});
           else if constexpr (o < NRD) read_b(IntC<RST>{}, rstage, IntC<nks>{}, IntC<(o < NRD ? o - NRA : 0)>{});
           else if constexpr (o < NOPS) {
-            if constexpr (qt == 0) issue(stage_of(IntC<NS - 1>{}), kk_tail, IntC<(o < NOPS ? HALF + (o - NRD) : 0)>{}, IntC<(o == NRD)>{});
+            if constexpr (qt != 3) issue(stage_of(IntC<NS - 1>{}), kk_tail, IntC<(o < NOPS ? DONE + (o - NRD) : 0)>{}, IntC<(o == NRD)>{});
             else issue(stage_of(IntC<NS>{}), kk_head, IntC<(o < NOPS ? o - NRD : 0)>{}, IntC<(o == NRD)>{});
           }
         });
