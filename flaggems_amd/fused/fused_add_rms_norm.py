@@ -2,8 +2,6 @@
 import logging
 import math
 
-import torch
-
 from .. import _C
 
 logger = logging.getLogger("flag_gems.fused.fused_add_rms_norm")

@@ -10,7 +10,6 @@ reference holds no golden vectors for these operators (every expectation is comp
 torch), so the pinning of this module is: (a) the torch library routines themselves for mm, addmm
 and softmax, (b) closed forms and invariants checked in tests/test_oracle.py for the rest.
 """
-import math
 
 import torch
 import torch.nn.functional as F

@@ -1,6 +1,5 @@
 """GPU parity of mm / addmm (data-parallel and stream-K schedules) against the CPU oracle.
 Shapes, scalars and layouts follow tests/test_blas_ops.py:17-136 of the reference."""
-import numpy as np
 import pytest
 import torch
 

@@ -4,7 +4,6 @@ import numpy as np
 import pytest
 import torch
 
-import flag_gems
 from flag_gems.modules import GemsDeepseekYarnRoPE, GemsRMSNorm, GemsRope, GemsSiluAndMul
 from oracle import torch_ref as O
 
