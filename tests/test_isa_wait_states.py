@@ -69,3 +69,23 @@ def test_every_function_and_every_exit_is_scanned():
 def test_state_does_not_leak_between_functions():
     text = kernel("\tv_readfirstlane_b32 s6, v36", "k0") + kernel(COPY, "k1")
     assert isa_check.scan(text) == []
+
+
+MFMA = "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[10:13], v[20:23], a[0:3]"
+
+
+@pytest.mark.parametrize("between,expect", [(0, 1), (10, 1), (11, 0)])
+def test_accumulator_read_after_a_matrix_instruction(between, expect):
+    body = MFMA + "\n" + "\tv_add_u32_e32 v1, v2, v3\n" * between + "\tv_accvgpr_read_b32 v5, a2"
+    assert len(isa_check.scan(kernel(body))) == expect
+
+
+def test_two_s_nop_15_clear_the_accumulators():
+    body = MFMA + "\n\ts_nop 15\n\ts_nop 15\n\tv_accvgpr_read_b32 v5, a0\n\tv_accvgpr_write_b32 a3, v1"
+    assert isa_check.scan(kernel(body)) == []
+
+
+def test_chained_matrix_instructions_and_other_accumulators_are_fine():
+    other = "\tv_mfma_f32_16x16x32_bf16 a[4:7], v[10:13], v[20:23], a[4:7]"
+    body = MFMA + "\n" + MFMA + "\n" + other + "\n\tv_accvgpr_read_b32 v5, a9"
+    assert isa_check.scan(kernel(body)) == []
