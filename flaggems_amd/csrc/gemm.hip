@@ -191,6 +191,37 @@ extern "C" int fg_gemm_workspace_layout(int device, size_t* max_bytes, size_t* h
   return FG_OK;
 }
 
+// The automatic schedule's choice between the two direct-to-LDS launches (shared by fg_gemm and fg_gemm_plan).
+static bool dma_auto_streamk(int64_t M, int64_t N, int64_t K, int cu, int* bm, int* bn, double* dp_us, int* workers,
+                             double* sk_us) {
+  const int64_t tiles = fg_cdiv(M, 128) * fg_cdiv(N, 128);
+  const int64_t iters = fg_cdiv(K, 64);
+  *dp_us = dma_pick_tile(M, N, K, cu, bm, bn);
+  *workers = 0;
+  *sk_us = 0.0;
+  if (!(tiles <= cu && tiles * iters >= 4 * (int64_t)cu)) return false;
+  *sk_us = dma_streamk_plan(tiles, iters, cu, workers);
+  return *sk_us < *dp_us;
+}
+
+extern "C" int fg_gemm_plan(int64_t M, int64_t N, int64_t K, int num_cu, int* tile_m, int* tile_n, double* dp_us,
+                            int* streamk_workers, double* streamk_us, int* streamk_chosen) {
+  FG_REQUIRE(M > 0 && N > 0 && K > 0, FG_ERR_INVALID, "gemm_plan: sizes must be positive");
+  FG_REQUIRE(K % 64 == 0, FG_ERR_UNSUPPORTED, "gemm_plan: K = %lld is not a multiple of 64", (long long)K);
+  const int cu = num_cu > 0 ? num_cu : num_cus(-1);
+  FG_REQUIRE(cu > 0, FG_ERR_INVALID, "gemm_plan: no device and no CU count given");
+  int bm = 0, bn = 0, workers = 0;
+  double dp = 0.0, sk = 0.0;
+  const bool chosen = dma_auto_streamk(M, N, K, cu, &bm, &bn, &dp, &workers, &sk);
+  if (tile_m) *tile_m = bm;
+  if (tile_n) *tile_n = bn;
+  if (dp_us) *dp_us = dp;
+  if (streamk_workers) *streamk_workers = workers;
+  if (streamk_us) *streamk_us = sk;
+  if (streamk_chosen) *streamk_chosen = chosen ? 1 : 0;
+  return FG_OK;
+}
+
 extern "C" int fg_stream_capture_id(void* stream, unsigned long long* id) {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
   unsigned long long cid = 0;
@@ -262,8 +293,8 @@ extern "C" int fg_gemm(const void* A, const void* B, const void* bias, void* C, 
           const bool dma = amode != LOAD_GEN && dma_supported(g, eb) && !fg_options().gemm_no_dma;
           if (dma) {
             int bm, bn, workers;
-            use_streamk = tiles <= cu && tiles * iters >= 4 * (int64_t)cu &&
-                          dma_streamk_plan(tiles, iters, cu, &workers) < dma_pick_tile(M, N, K, cu, &bm, &bn);
+            double dp_us, sk_us;
+            use_streamk = dma_auto_streamk(M, N, K, cu, &bm, &bn, &dp_us, &workers, &sk_us);
           } else {
             // (the stream-K kernels have no element-aligned vector modes: such operands stay data-parallel)
             use_streamk = !vec_unaligned && tiles * 2 <= (int64_t)cu && tiles * iters >= 4 * (int64_t)cu;

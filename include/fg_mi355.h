@@ -175,6 +175,19 @@ size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, in
  * src/flag_gems/ops/mm_streamk.py:488-491. */
 int fg_gemm_workspace_layout(int device, size_t* max_bytes /*host*/, size_t* header_bytes /*host*/);
 
+/* What fg_gemm's automatic schedule selects for 16-bit operands that qualify for the direct-to-LDS kernels (16-byte
+ * aligned rows, unit stride along K or N, K a multiple of 64) on a device of `num_cu` compute units (<= 0: the
+ * current device's): the workgroup tile of the data-parallel launch with its modelled duration in microseconds, and
+ * the number of workgroups and modelled duration of the stream-K launch on 128x128 tiles (*streamk_workers = 0 when
+ * the problem does not qualify for it: more tiles than CUs or fewer than four K steps per CU).  *streamk_chosen tells
+ * which of the two the automatic schedule takes when a workspace is given.  Host arithmetic only when num_cu > 0: no
+ * device is touched.  Any output pointer may be NULL.
+ * Stands in for the tuned-configuration lookup of src/flag_gems/ops/mm.py:54-62 and the schedule test
+ * streamk_scenario, src/flag_gems/ops/mm.py:186-197. */
+int fg_gemm_plan(int64_t M, int64_t N, int64_t K, int num_cu, int* tile_m /*host*/, int* tile_n /*host*/,
+                 double* dp_us /*host*/, int* streamk_workers /*host*/, double* streamk_us /*host*/,
+                 int* streamk_chosen /*host*/);
+
 /* *id = 0 when `stream` is not capturing into a HIP graph, otherwise a non-zero number unique to the capture in
  * progress.  Host code uses it to record one clearing of the workspace header per captured graph.  No counterpart
  * in the reference (its Triton launches allocate and clear per call). */
