@@ -191,6 +191,16 @@ extern "C" int fg_gemm_workspace_layout(int device, size_t* max_bytes, size_t* h
   return FG_OK;
 }
 
+extern "C" int fg_gemm_tile_order(int tiles_m, int tiles_n, int b_k_contiguous, int* tile_m, int* tile_n) {
+  FG_REQUIRE(tiles_m > 0 && tiles_n > 0 && (int64_t)tiles_m * tiles_n < ((int64_t)1 << 31), FG_ERR_INVALID,
+             "gemm_tile_order: bad grid %d x %d", tiles_m, tiles_n);
+  FG_REQUIRE(tile_m && tile_n, FG_ERR_INVALID, "gemm_tile_order: null pointer");
+  const int total = tiles_m * tiles_n;
+  // the direct-to-LDS kernels walk strips of 2 sub-block rows for a K-contiguous B and of 4 for a row-major one
+  for (int id = 0; id < total; ++id) tile_coords(id, tiles_m, tiles_n, tile_m[id], tile_n[id], b_k_contiguous ? 2 : 4);
+  return FG_OK;
+}
+
 // The automatic schedule's choice between the two direct-to-LDS launches (shared by fg_gemm and fg_gemm_plan).
 static bool dma_auto_streamk(int64_t M, int64_t N, int64_t K, int cu, int* bm, int* bn, double* dp_us, int* workers,
                              double* sk_us) {

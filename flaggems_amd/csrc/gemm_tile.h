@@ -341,7 +341,7 @@ template <typename T, int ROWS> struct Stager<T, ROWS, LOAD_GEN> {
 // Other grids: ids congruent mod 8 are made consecutive, then walked in column-major groups of
 // 8 tile rows.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int& tm, int& tn, int strip_rows = 2) {
+__host__ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int& tm, int& tn, int strip_rows = 2) {
   constexpr int XCDS = 8, SUB_M = 8, SUB_N = 4, PER = SUB_M * SUB_N;
   if (tiles_m % SUB_M == 0 && tiles_n % SUB_N == 0) {
     const int sm_count = tiles_m / SUB_M, sn_count = tiles_n / SUB_N, nsub = sm_count * sn_count;

@@ -188,6 +188,13 @@ int fg_gemm_plan(int64_t M, int64_t N, int64_t K, int num_cu, int* tile_m /*host
                  double* dp_us /*host*/, int* streamk_workers /*host*/, double* streamk_us /*host*/,
                  int* streamk_chosen /*host*/);
 
+/* The order in which a data-parallel launch of tiles_m x tiles_n workgroup tiles walks its grid: workgroup id i
+ * computes tile (tile_m[i], tile_n[i]); both arrays hold tiles_m * tiles_n entries.  Workgroup i runs on XCD i mod 8,
+ * so the order decides which A and B panels share an L2.  b_k_contiguous selects the variant used for B = W^T
+ * (non-zero) or row-major B.  Host arithmetic only; the kernels call the same function.
+ * Stands in for the grouped ordering of mm_kernel_general, src/flag_gems/ops/mm.py:83-91 (GROUP_M grouping of the program ids). */
+int fg_gemm_tile_order(int tiles_m, int tiles_n, int b_k_contiguous, int* tile_m /*host*/, int* tile_n /*host*/);
+
 /* *id = 0 when `stream` is not capturing into a HIP graph, otherwise a non-zero number unique to the capture in
  * progress.  Host code uses it to record one clearing of the workspace header per captured graph.  No counterpart
  * in the reference (its Triton launches allocate and clear per call). */
