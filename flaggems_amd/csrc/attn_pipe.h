@@ -318,8 +318,11 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   };
   auto read_v = [&](auto i_c, auto sv_c, auto kt_c) {
     constexpr int i = decltype(i_c)::value, SV = decltype(sv_c)::value, KT = decltype(kt_c)::value;
-    vring[i % RING][0] = lds_read_tr_b64_imm<SV * OPB + (KT * 32) * RB>(v_addr[i]);
-    vring[i % RING][1] = lds_read_tr_b64_imm<SV * OPB + (KT * 32 + 16) * RB>(v_addr[i]);
+    // (callers guard with `if constexpr (i < NPV)`, but inside nested generic lambdas the compiler still instantiates
+    // this body for the discarded calls; the clamp keeps those instantiations inside the array)
+    constexpr int ia = i < NPV ? i : 0;
+    vring[i % RING][0] = lds_read_tr_b64_imm<SV * OPB + (KT * 32) * RB>(v_addr[ia]);
+    vring[i % RING][1] = lds_read_tr_b64_imm<SV * OPB + (KT * 32 + 16) * RB>(v_addr[ia]);
   };
   // score pair pi (0..7) of a half tile: elements 2 w, 2 w + 1 of tile (KT2, QT); it is word 2 KT2 + w of pf[QT]
   // Phase A of the step whose scores S(h) sit in buffer CUR.  QK: S(h+1) = K.Q^T - m -> buffer CUR^1, from half

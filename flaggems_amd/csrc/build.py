@@ -5,6 +5,7 @@ The library lands next to the package (flaggems_amd/libfg_mi355.so) so it travel
 """
 import argparse
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -57,6 +58,31 @@ def _newer(src_paths, target):
     return any(os.path.getmtime(p) > t for p in src_paths)
 
 
+_DIAG = re.compile(r"^\S+:\d+:\d+: (warning|error|note): ")
+# expected diagnostics: the host pass does not know the device feature switch; the asm copies set M0 themselves and
+# say so in their clobber lists, which the compiler remarks on for every instantiation
+_EXPECTED = ("packed-fp32-ops", "inline asm clobber list contains reserved registers: m0",
+             "Reserved registers on the clobber list may not be preserved")
+
+
+def _quiet(text):
+    """The compiler's output without the expected diagnostics (each with its include trail, source excerpt and caret
+    lines)."""
+    out, trail, skipping = [], [], False
+    for line in text.splitlines():
+        if line.startswith("In file included"):
+            trail.append(line)
+            continue
+        if _DIAG.match(line):
+            skipping = any(e in line for e in _EXPECTED)
+            if not skipping:
+                out.extend(trail)
+            trail = []
+        if not skipping and "warnings generated" not in line and not any(e in line for e in _EXPECTED):
+            out.append(line)
+    return "\n".join(out)
+
+
 def _compile(src, force):
     path = os.path.join(HERE, src)
     obj = os.path.join(OBJ_DIR, src + ".o")
@@ -68,7 +94,7 @@ def _compile(src, force):
     keep = ["-save-temps=obj"] if src in ASM_CHECKED else []
     cmd = [HIPCC] + FLAGS + keep + lang + ["-c", path, "-o", obj]
     p = subprocess.run(cmd, capture_output=True, text=True)
-    log = "\n".join(l for l in (p.stdout + p.stderr).splitlines() if "packed-fp32-ops" not in l)
+    log = _quiet(p.stdout + p.stderr)
     if p.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
     if keep:

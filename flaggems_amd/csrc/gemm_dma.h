@@ -303,7 +303,7 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
       const uint32_t m0v = (uint32_t)(uintptr_t)FGK_LDSP(l);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(m0v) : "memory", "m0");
     }
-    const uint32_t off = IS_A ? a_off[jj] : b_off[jj];
+    const uint32_t off = IS_A ? a_off[IS_A ? jj : 0] : b_off[IS_A ? 0 : jj];
     if constexpr (RAGGED) {
       if (kbase.last) {
         // the partial K step: per-lane 64-bit addresses, lanes whose chunk lies past K read zeros
