@@ -52,10 +52,16 @@ namespace fgk {
 
 constexpr int kDmaRowB = 128;   // bytes of K per stage per A row
 constexpr int kDmaBK = 64;
-// Quarter steps of a K step that issue copies: 2 (quarter 3 and quarter 0, half of the copies each) for every tile,
-// or 3 (quarters 3, 0 and 1) for the 256x256 tile with two stages.  3 was measured 2-6 % faster on large products
-// and is switched off: it has run on a few large shapes only, not under the parity tests.
+// Quarter steps of a K step that issue copies: 2 (quarter 3 and quarter 0, half of the copies each), or 3 (quarters
+// 3, 0 and 1).  3 on the 256x256 tile was measured 2-6 % faster on large products; it is switched off because it has
+// run on a few large shapes only, not under the parity tests.  kDmaCopyRunsEveryTile extends 3 from the 256x256 tile
+// with two stages to every tile (never measured).
 constexpr int kDmaCopyRuns = 2;
+constexpr bool kDmaCopyRunsEveryTile = false;
+// with three quarters: the copies of a step issued in quarter 3 and in quarter 0 (the rest go to quarter 1), by the
+// number of copies per wave and step
+constexpr int dma_split_q3(int ndma, bool b_kc) { return ndma == 16 ? (b_kc ? 6 : 8) : ndma == 14 ? 5 : ndma == 12 ? 4 : 3; }
+constexpr int dma_split_q0(int ndma) { return ndma == 16 ? 5 : ndma == 14 ? 5 : ndma == 12 ? 4 : 3; }
 constexpr int dma_lds_bytes(int bm, int bn, int stages = 2) { return stages * (bm + bn) * kDmaRowB; }  // stages of (A tile + B tile)
 constexpr int cmin(int a, int b) { return a < b ? a : b; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
@@ -213,9 +219,9 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // (whose stage has just been read for the last time), C0 and C1 in quarters 0 and 1 of the step after that one.
   // The barrier of a K step puts the four waves back in step, so they reach these quarters together, and a copy
   // holds the CU's address path for 16 cycles: the more quarters share the copies, the less the waves queue.
-  constexpr bool THREE_RUNS = kDmaCopyRuns == 3 && BM == 256 && BN == 256 && NS == 2 && !RAGGED;
-  constexpr int C3 = THREE_RUNS ? (B_KC ? 6 : 8) : NDMA / 2;
-  constexpr int C0 = THREE_RUNS ? 5 : NDMA - C3;
+  constexpr bool THREE_RUNS = kDmaCopyRuns == 3 && !RAGGED && (kDmaCopyRunsEveryTile || (BM == 256 && BN == 256 && NS == 2));
+  constexpr int C3 = THREE_RUNS ? dma_split_q3(NDMA, B_KC) : NDMA / 2;
+  constexpr int C0 = THREE_RUNS ? dma_split_q0(NDMA) : NDMA - C3;
   constexpr int C1 = NDMA - C3 - C0;
   constexpr int HALF = C3;
   static_assert(C0 > 0 && C1 >= 0, "copy split");

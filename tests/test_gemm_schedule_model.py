@@ -120,21 +120,25 @@ def violations(nk, ns, ndma, c3, c0, c1, events=None):
 
 
 def header_splits():
-    """(tile, stages, copies per step) -> list of (c3, c0, c1) the header can select for it."""
+    """(stages, copies per step, [(c3, c0, c1), ...]): every split the header can select for a tile it instantiates."""
     src = open(HEADER).read()
-    m = re.search(r"constexpr int C3 = THREE_RUNS \? \(B_KC \? (\d+) : (\d+)\) : NDMA / 2;", src)
-    m0 = re.search(r"constexpr int C0 = THREE_RUNS \? (\d+) : NDMA - C3;", src)
-    assert m and m0, "the copy split of dma_tile_mainloop is no longer written the way this test reads it"
-    assert re.search(r"THREE_RUNS = kDmaCopyRuns == 3 && BM == 256 && BN == 256 && NS == 2 && !RAGGED;", src)
-    three = [(int(c3), int(m0.group(1)), 16 - int(c3) - int(m0.group(1))) for c3 in m.groups()]
+    q3 = re.search(r"constexpr int dma_split_q3\(int ndma, bool b_kc\) \{ return ndma == 16 \? \(b_kc \? (\d+) : (\d+)\) : "
+                   r"ndma == 14 \? (\d+) : ndma == 12 \? (\d+) : (\d+); \}", src)
+    q0 = re.search(r"constexpr int dma_split_q0\(int ndma\) \{ return ndma == 16 \? (\d+) : ndma == 14 \? (\d+) : "
+                   r"ndma == 12 \? (\d+) : (\d+); \}", src)
+    assert q3 and q0, "the copy split of dma_tile_mainloop is no longer written the way this test reads it"
+    assert "constexpr int C3 = THREE_RUNS ? dma_split_q3(NDMA, B_KC) : NDMA / 2;" in src
+    assert "constexpr int C0 = THREE_RUNS ? dma_split_q0(NDMA) : NDMA - C3;" in src
+    assert "constexpr int C1 = NDMA - C3 - C0;" in src
+    a, b, c14, c12, c8 = (int(x) for x in q3.groups())
+    z16, z14, z12, z8 = (int(x) for x in q0.groups())
+    three = {16: [(a, z16), (b, z16)], 14: [(c14, z14)], 12: [(c12, z12)], 8: [(c8, z8)]}
     # tiles and stage counts the launcher instantiates: copies per wave and step = (BM + BN) / 32
     tiles = [(256, 256, 2), (192, 256, 2), (256, 128, 3), (128, 256, 3), (128, 128, 4), (128, 128, 2)]
     out = []
     for bm, bn, ns in tiles:
         ndma = (bm + bn) // 32
-        splits = [(ndma // 2, ndma - ndma // 2, 0)]
-        if (bm, bn, ns) == (256, 256, 2):
-            splits += three
+        splits = [(ndma // 2, ndma - ndma // 2, 0)] + [(c3, c0, ndma - c3 - c0) for c3, c0 in three[ndma]]
         out.append((ns, ndma, splits))
     return out
 
