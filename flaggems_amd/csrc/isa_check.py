@@ -15,7 +15,10 @@ v_readfirstlane that produces a base address and the copy that reads it is whate
 leave: a copy issued too early takes the register's previous contents as its address.  build.py keeps the device
 assembly of those sources and fails the build when this scan finds such a pair.
 
-The scan is textual: it walks each kernel's instructions in program order, counts every instruction as one wait
+A fourth check (scan_lds_reads, further down) follows the LDS counter through the control-flow graph and reports uses
+of a register whose LDS read, issued from asm with a hand-counted wait, may not have returned.
+
+The scan of the three hazards above is textual: it walks each kernel's instructions in program order, counts every instruction as one wait
 state (s_nop N as N + 1) and ignores control flow, which errs on the side of reporting (a pair split by a label
 is still reported).
 """
@@ -126,9 +129,132 @@ def scan(text):
     return hits
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# LDS reads written as asm.  The compiler places s_waitcnt for the loads it selects; the destination registers of
+# a ds_read inside an asm statement are, to it, written when the statement ends, so nothing stops it from scheduling
+# a use in front of the wait the source placed by hand, and a hand-counted `s_waitcnt lgkmcnt(N)` that is one too
+# large lets an instruction read a register whose load has not returned.  Both give stale data, not a fault, and only
+# sometimes.  This pass follows the LDS counter through the control-flow graph: LDS operations return in order, so
+# after lgkmcnt(N) at most the N youngest are outstanding; any instruction that reads or writes a vector register a
+# still outstanding read is going to write is reported.  Scalar loads share the counter and return out of order:
+# while one is outstanding only lgkmcnt(0) is taken to retire anything.
+# ---------------------------------------------------------------------------------------------------------------
+_SMEM = "smem"
+_MAX_STATES = 256
+
+
+def _vgprs(tok):
+    tok = tok.strip()
+    m = re.match(r"^v\[(\d+):(\d+)\]$", tok)
+    if m:
+        return frozenset(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"^v(\d+)$", tok)
+    return frozenset({int(m.group(1))}) if m else frozenset()
+
+
+def _blocks(body):
+    """[(label or None, [(op, ops, line), ...])] in layout order."""
+    out, cur, name = [], [], None
+    for raw in body.splitlines():
+        line = raw.split(";")[0].split("//")[0].strip()
+        if not line:
+            continue
+        if line.endswith(":"):
+            out.append((name, cur))
+            name, cur = line[:-1], []
+            continue
+        if line.startswith("."):
+            continue
+        parts = line.split(None, 1)
+        ops = [a.strip() for a in parts[1].split(",")] if len(parts) > 1 else []
+        cur.append((parts[0], ops, line))
+        if parts[0].startswith(("s_branch", "s_cbranch", "s_endpgm", "s_setpc")):
+            out.append((name, cur))
+            name, cur = None, []
+    out.append((name, cur))
+    return [(n, b) for n, b in out if n is not None or b]
+
+
+def _lds_step(state, op, ops, line, report):
+    """Transfer function of one instruction on a tuple of outstanding LDS-counter operations (oldest first)."""
+    if op == "s_waitcnt":
+        text = " ".join(ops)
+        m = re.search(r"lgkmcnt\((\d+)\)", text)
+        if m is None:
+            # a bare immediate: bits 11:8 hold the LDS counter on gfx9
+            m2 = re.match(r"^(0x[0-9a-fA-F]+|\d+)$", text.strip())
+            if m2 is None:
+                return state
+            n = (int(m2.group(1), 0) >> 8) & 0xF
+        else:
+            n = int(m.group(1))
+        if n == 0:
+            return ()
+        if _SMEM in state:
+            return state
+        return state[len(state) - n:] if len(state) > n else state
+    is_read = op.startswith(("ds_read", "ds_bpermute", "ds_permute", "ds_swizzle", "ds_consume", "ds_append"))
+    # (a second read into the same registers is no hazard: LDS operations return in order)
+    srcs = ops[1:] if is_read else ops
+    used = frozenset().union(*[_vgprs(o.split()[0]) for o in srcs if o]) if srcs else frozenset()
+    for dst in state:
+        if dst is not _SMEM and dst & used:
+            report(line, "touches v%s while the LDS read into it may be outstanding" % sorted(dst & used))
+            break
+    if is_read:
+        return state + (_vgprs(ops[0]) if ops else frozenset(),)
+    if op.startswith("ds_"):
+        return state + (frozenset(),)
+    if op.startswith(("s_load", "s_buffer_load", "s_scratch_load", "s_atc_probe", "s_memtime", "s_memrealtime")):
+        return state + (_SMEM,)
+    return state
+
+
+def scan_lds_reads(text):
+    """Uses of a register before the LDS read that writes it is known to have returned: (kernel, line, reason)."""
+    hits = []
+    for km in _KERNEL.finditer(text):
+        kernel, blocks = km.group(1), _blocks(km.group(2))
+        index = {n: i for i, (n, _) in enumerate(blocks) if n is not None}
+        succ = []
+        for i, (_, ins) in enumerate(blocks):
+            last = ins[-1] if ins else None
+            nxt = [i + 1] if i + 1 < len(blocks) else []
+            if last is None:
+                succ.append(nxt)
+            elif last[0] == "s_branch":
+                succ.append([index[last[1][0]]] if last[1] and last[1][0] in index else [])
+            elif last[0].startswith("s_cbranch"):
+                succ.append(nxt + ([index[last[1][0]]] if last[1] and last[1][0] in index else []))
+            elif last[0].startswith(("s_endpgm", "s_setpc")):
+                succ.append([])
+            else:
+                succ.append(nxt)
+        seen = [set() for _ in blocks]
+        seen[0].add(())
+        work = [(0, ())]
+        found = set()
+        while work:
+            b, state = work.pop()
+            for op, ops, line in blocks[b][1]:
+                state = _lds_step(state, op, ops, line, lambda l, why: found.add((l, why)))
+                if len(state) > 15:  # the counter has four bits: the 16th operation is not issued before the oldest returns
+                    state = state[-15:]
+            for nb in succ[b]:
+                if state not in seen[nb]:
+                    if len(seen[nb]) >= _MAX_STATES:
+                        found.add((blocks[nb][0] or "?", "too many distinct LDS-counter states reach this block"))
+                        continue
+                    seen[nb].add(state)
+                    work.append((nb, state))
+        hits += [(kernel, l, why) for l, why in sorted(found)]
+    return hits
+
+
 def check_file(path):
     with open(path) as f:
-        return scan(f.read())
+        text = f.read()
+    return scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)]
 
 
 if __name__ == "__main__":

@@ -89,3 +89,54 @@ def test_chained_matrix_instructions_and_other_accumulators_are_fine():
     other = "\tv_mfma_f32_16x16x32_bf16 a[4:7], v[10:13], v[20:23], a[4:7]"
     body = MFMA + "\n" + MFMA + "\n" + other + "\n\tv_accvgpr_read_b32 v5, a9"
     assert isa_check.scan(kernel(body)) == []
+
+
+# ---- LDS reads against the LDS counter ------------------------------------------------------------------------
+READS = "\tds_read_b128 v[0:3], v40\n\tds_read_b128 v[4:7], v40 offset:1024\n\tds_read_b64_tr_b16 v[8:9], v41\n"
+USE0 = "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[20:23], a[0:3]"
+
+
+@pytest.mark.parametrize("wait,expect", [(0, 0), (2, 0), (3, 1)])
+def test_a_counted_wait_retires_the_oldest_reads_only(wait, expect):
+    body = READS + "\ts_waitcnt lgkmcnt(%d)\n" % wait + USE0
+    assert len(isa_check.scan_lds_reads(kernel(body))) == expect
+
+
+def test_use_of_a_younger_read_needs_a_smaller_count():
+    use2 = "\tv_pk_mul_f16 v30, v8, v9"
+    assert len(isa_check.scan_lds_reads(kernel(READS + "\ts_waitcnt lgkmcnt(1)\n" + use2))) == 1
+    assert isa_check.scan_lds_reads(kernel(READS + "\ts_waitcnt vmcnt(3) lgkmcnt(0)\n" + use2)) == []
+    # a wait on the vector-memory counter alone retires nothing here
+    assert len(isa_check.scan_lds_reads(kernel(READS + "\ts_waitcnt vmcnt(0)\n" + USE0))) == 1
+
+
+def test_overwriting_a_register_with_a_read_in_flight_is_reported():
+    body = "\tds_read_b128 v[0:3], v40\n\tv_mov_b32_e32 v2, 0\n\ts_waitcnt lgkmcnt(0)"
+    assert len(isa_check.scan_lds_reads(kernel(body))) == 1
+
+
+def test_the_address_register_may_be_reused_at_once():
+    body = "\tds_read_b128 v[0:3], v40\n\tv_add_u32_e32 v40, 16, v40\n\ts_waitcnt lgkmcnt(0)\n" + USE0
+    assert isa_check.scan_lds_reads(kernel(body)) == []
+
+
+def test_lds_writes_and_scalar_loads_count_too():
+    body = "\tds_read_b128 v[0:3], v40\n\tds_write_b32 v41, v42\n\ts_waitcnt lgkmcnt(1)\n" + USE0
+    assert isa_check.scan_lds_reads(kernel(body)) == []
+    # a scalar load in flight returns out of order: lgkmcnt(1) proves nothing about the read
+    body = "\tds_read_b128 v[0:3], v40\n\ts_load_dwordx2 s[4:5], s[0:1], 0x0\n\ts_waitcnt lgkmcnt(1)\n" + USE0
+    assert len(isa_check.scan_lds_reads(kernel(body))) == 1
+
+
+def test_the_counter_is_followed_around_a_loop():
+    """The read issued at the bottom of the loop body is still in flight at its top on the way round; the use at the
+    top is fine on entry (nothing outstanding) and stale on the back edge unless the body waits first."""
+    loop = ("\ts_mov_b32 s4, 8\n.LBB0_1:\n%s" + USE0 + "\n\tds_read_b128 v[0:3], v40\n\ts_sub_u32 s4, s4, 1\n"
+            "\ts_cmp_lg_u32 s4, 0\n\ts_cbranch_scc1 .LBB0_1\n\ts_waitcnt lgkmcnt(0)")
+    assert len(isa_check.scan_lds_reads(kernel(loop % ""))) == 1
+    assert isa_check.scan_lds_reads(kernel(loop % "\ts_waitcnt lgkmcnt(0)\n")) == []
+
+
+def test_both_arms_of_a_branch_are_followed():
+    body = ("\tds_read_b128 v[0:3], v40\n\ts_cbranch_scc1 .LBB0_2\n\ts_waitcnt lgkmcnt(0)\n.LBB0_2:\n" + USE0)
+    assert len(isa_check.scan_lds_reads(kernel(body))) == 1   # the taken arm skips the wait
