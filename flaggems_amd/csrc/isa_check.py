@@ -1,4 +1,5 @@
-"""Wait-state check of the device assembly of the sources that issue memory instructions from inline asm.
+"""Checks of the device assembly that the library's build runs on every HIP source: wait states around instructions
+issued from inline asm, LDS reads issued from asm against the LDS counter, and no packed fp32 arithmetic.
 
 gfx9 leaves these data hazards to software:
   * a vector instruction writes a scalar register (v_readfirstlane, v_readlane, a v_cmp with a scalar destination)
@@ -251,10 +252,24 @@ def scan_lds_reads(text):
     return hits
 
 
+# Packed fp32 arithmetic is switched off for this library (a compiler flag removes the feature, and no source writes
+# the instructions by hand); this confirms it on what was actually generated.
+_PACKED_F32 = ("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32")
+
+
+def scan_packed_f32(text):
+    hits = []
+    for km in _KERNEL.finditer(text):
+        for i, (op, _, line) in enumerate(_instructions(km.group(2))):
+            if op.startswith(_PACKED_F32):
+                hits.append((km.group(1), i, line, "packed fp32 arithmetic is not to be generated for this library"))
+    return hits
+
+
 def check_file(path):
     with open(path) as f:
         text = f.read()
-    return scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)]
+    return scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] + scan_packed_f32(text)
 
 
 if __name__ == "__main__":

@@ -140,3 +140,8 @@ def test_the_counter_is_followed_around_a_loop():
 def test_both_arms_of_a_branch_are_followed():
     body = ("\tds_read_b128 v[0:3], v40\n\ts_cbranch_scc1 .LBB0_2\n\ts_waitcnt lgkmcnt(0)\n.LBB0_2:\n" + USE0)
     assert len(isa_check.scan_lds_reads(kernel(body))) == 1   # the taken arm skips the wait
+
+
+def test_packed_fp32_arithmetic_is_reported():
+    assert len(isa_check.scan_packed_f32(kernel("\tv_pk_fma_f32 v[0:1], v[2:3], v[4:5], v[6:7]"))) == 1
+    assert isa_check.scan_packed_f32(kernel("\tv_pk_mul_f16 v0, v1, v2\n\tv_fma_f32 v0, v1, v2, v3")) == []
