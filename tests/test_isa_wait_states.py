@@ -145,3 +145,54 @@ def test_both_arms_of_a_branch_are_followed():
 def test_packed_fp32_arithmetic_is_reported():
     assert len(isa_check.scan_packed_f32(kernel("\tv_pk_fma_f32 v[0:1], v[2:3], v[4:5], v[6:7]"))) == 1
     assert isa_check.scan_packed_f32(kernel("\tv_pk_mul_f16 v0, v1, v2\n\tv_fma_f32 v0, v1, v2, v3")) == []
+
+
+def _build_module():
+    spec = importlib.util.spec_from_file_location("fg_build_for_test", os.path.join(ROOT, "flaggems_amd", "csrc", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_the_build_refuses_an_object_whose_assembly_fails_the_scan(tmp_path, monkeypatch):
+    build = _build_module()
+    monkeypatch.setattr(build, "OBJ_DIR", str(tmp_path))
+    obj = tmp_path / "x.hip.o"
+    asm = tmp_path / "x-hip-amdgcn-amd-amdhsa-gfx950.s"
+    leftover = tmp_path / "x-hip-amdgcn-amd-amdhsa-gfx950.hipi"
+    other = tmp_path / "y.hip.o"
+    for f in (obj, leftover, other):
+        f.write_text("")
+    asm.write_text(kernel("\tv_readfirstlane_b32 s6, v36\n" + COPY))
+    with pytest.raises(RuntimeError, match="fails 1 check"):
+        build._check_wait_states("x.hip", str(obj))
+    assert not obj.exists() and other.exists()        # nothing stale left to link
+    # a clean assembly: the object stays, the bulky intermediates go, the assembly is kept for inspection
+    obj.write_text("")
+    leftover.write_text("")
+    asm.write_text(kernel("\tv_readfirstlane_b32 s6, v36\n\ts_nop 4\n" + COPY))
+    build._check_wait_states("x.hip", str(obj))
+    assert obj.exists() and asm.exists() and not leftover.exists() and other.exists()
+    # no assembly at all is an error too: the check must not be skipped silently
+    asm.unlink()
+    with pytest.raises(RuntimeError, match="no device assembly"):
+        build._check_wait_states("x.hip", str(obj))
+
+
+def test_expected_compiler_remarks_are_dropped_from_the_build_log():
+    build = _build_module()
+    text = "\n".join([
+        "'-packed-fp32-ops' is not a recognized feature for this target (ignoring feature)",
+        "In file included from x.hip:5:",
+        "/a/gemm_dma.h:290:20: warning: inline asm clobber list contains reserved registers: m0 [-Winline-asm]",
+        "  290 |       asm volatile(...);",
+        "      |                    ^",
+        "/a/gemm_dma.h:290:20: note: Reserved registers on the clobber list may not be preserved across the asm statement",
+        "In file included from x.hip:6:",
+        "/a/foo.h:12:3: warning: unused variable 'x' [-Wunused-variable]",
+        "   12 |   int x;",
+        "800 warnings generated.",
+    ])
+    kept = build._quiet(text).splitlines()
+    assert kept == ["In file included from x.hip:6:", "/a/foo.h:12:3: warning: unused variable 'x' [-Wunused-variable]",
+                    "   12 |   int x;"]
