@@ -60,6 +60,11 @@ int launch_dp(const GemmArgs& g, hipStream_t st) {
   return fg_check_launch("gemm");
 }
 
+// (split in two so that the element-wise stager, the last resort of the small tile, is never instantiated for the
+// large one: it would not be launched there, and it compiles to a kernel that spills a thousand registers)
+template <typename T, int BM, int BN>
+int launch_dp_small_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st);
+
 template <typename T, int BM, int BN>
 int launch_dp_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
   if constexpr (BM == 256) {
@@ -68,7 +73,14 @@ int launch_dp_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
     if (amode == LOAD_K && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_K, LOAD_MN>(g, st);
     if (amode == LOAD_MN && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_MN, LOAD_K>(g, st);
     return launch_dp<T, BM, BN, LOAD_MN, LOAD_MN>(g, st);
-  } else if constexpr (sizeof(T) == 2) {
+  } else {
+    return launch_dp_small_modes<T, BM, BN>(g, amode, bmode, st);
+  }
+}
+
+template <typename T, int BM, int BN>
+int launch_dp_small_modes(const GemmArgs& g, int amode, int bmode, hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
     if (amode == LOAD_K && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_K, LOAD_K>(g, st);
     if (amode == LOAD_K && bmode == LOAD_MN) return launch_dp<T, BM, BN, LOAD_K, LOAD_MN>(g, st);
     if (amode == LOAD_MN && bmode == LOAD_K) return launch_dp<T, BM, BN, LOAD_MN, LOAD_K>(g, st);

@@ -216,21 +216,7 @@ def scan_lds_reads(text):
     hits = []
     for km in _KERNEL.finditer(text):
         kernel, blocks = km.group(1), _blocks(km.group(2))
-        index = {n: i for i, (n, _) in enumerate(blocks) if n is not None}
-        succ = []
-        for i, (_, ins) in enumerate(blocks):
-            last = ins[-1] if ins else None
-            nxt = [i + 1] if i + 1 < len(blocks) else []
-            if last is None:
-                succ.append(nxt)
-            elif last[0] == "s_branch":
-                succ.append([index[last[1][0]]] if last[1] and last[1][0] in index else [])
-            elif last[0].startswith("s_cbranch"):
-                succ.append(nxt + ([index[last[1][0]]] if last[1] and last[1][0] in index else []))
-            elif last[0].startswith(("s_endpgm", "s_setpc")):
-                succ.append([])
-            else:
-                succ.append(nxt)
+        succ = _successors(blocks)
         seen = [set() for _ in blocks]
         seen[0].add(())
         work = [(0, ())]
@@ -266,10 +252,99 @@ def scan_packed_f32(text):
     return hits
 
 
+def _successors(blocks):
+    index = {n: i for i, (n, _) in enumerate(blocks) if n is not None}
+    succ = []
+    for i, (_, ins) in enumerate(blocks):
+        last = ins[-1] if ins else None
+        nxt = [i + 1] if i + 1 < len(blocks) else []
+        target = [index[last[1][0]]] if last and last[1] and last[1][0] in index else []
+        if last is None:
+            succ.append(nxt)
+        elif last[0] == "s_branch":
+            succ.append(target)
+        elif last[0].startswith("s_cbranch"):
+            succ.append(nxt + target)
+        elif last[0].startswith(("s_endpgm", "s_setpc")):
+            succ.append([])
+        else:
+            succ.append(nxt)
+    return succ
+
+
+def _blocks_in_loops(succ):
+    """Indices of the basic blocks that lie on a cycle of the control-flow graph (Tarjan, iterative)."""
+    n = len(succ)
+    order, low, on_stack, comp = [None] * n, [0] * n, [False] * n, [None] * n
+    stack, counter, ncomp = [], 0, 0
+    for root in range(n):
+        if order[root] is not None:
+            continue
+        work = [(root, 0)]
+        while work:
+            v, k0 = work[-1]
+            if k0 == 0:
+                order[v] = low[v] = counter
+                counter += 1
+                stack.append(v)
+                on_stack[v] = True
+            descended = False
+            for k in range(k0, len(succ[v])):
+                w = succ[v][k]
+                if order[w] is None:
+                    work[-1] = (v, k + 1)
+                    work.append((w, 0))
+                    descended = True
+                    break
+                if on_stack[w]:
+                    low[v] = min(low[v], order[w])
+            if descended:
+                continue
+            if low[v] == order[v]:
+                while True:
+                    w = stack.pop()
+                    on_stack[w] = False
+                    comp[w] = ncomp
+                    if w == v:
+                        break
+                ncomp += 1
+            work.pop()
+            if work:
+                low[work[-1][0]] = min(low[work[-1][0]], low[v])
+    size = {}
+    for v in range(n):
+        size[comp[v]] = size.get(comp[v], 0) + 1
+    return [v for v in range(n) if size[comp[v]] > 1 or v in succ[v]]
+
+
+# Kernels whose loops are known to touch scratch memory, with the reason each is tolerated.
+SCRATCH_IN_LOOP_ALLOWED = {
+    # rms_norm backward for rows of 8193..16384 elements: 1024 threads x 2 packs leave 128 registers a thread
+    "rms_bwd_rows_kernel": "three values of a 1024-thread variant live in scratch",
+    # stream-K on the element-by-element stager: the last resort for operands contiguous along neither axis
+    "gemm_streamk_kernel": "the element-wise stager of the last-resort stream-K kernel spills",
+}
+
+
+def scan_scratch_in_loops(text, allowed=SCRATCH_IN_LOOP_ALLOWED):
+    """Register spills (or private arrays) that are accessed inside a loop: (kernel, count, first instruction)."""
+    hits = []
+    for km in _KERNEL.finditer(text):
+        if any(a in km.group(1) for a in allowed):
+            continue
+        blocks = _blocks(km.group(2))
+        ops = [line for v in _blocks_in_loops(_successors(blocks)) for op, _, line in blocks[v][1] if op.startswith("scratch_")]
+        if ops:
+            hits.append((km.group(1), len(ops), ops[0]))
+    return hits
+
+
 def check_file(path):
     with open(path) as f:
         text = f.read()
-    return scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] + scan_packed_f32(text)
+    return (scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] + scan_packed_f32(text) +
+            [(k, 0, first, "%d scratch accesses inside a loop: registers spill there" % n)
+             for k, n, first in scan_scratch_in_loops(text)])
 
 
 if __name__ == "__main__":

@@ -196,3 +196,19 @@ def test_expected_compiler_remarks_are_dropped_from_the_build_log():
     kept = build._quiet(text).splitlines()
     assert kept == ["In file included from x.hip:6:", "/a/foo.h:12:3: warning: unused variable 'x' [-Wunused-variable]",
                     "   12 |   int x;"]
+
+
+def test_scratch_accesses_are_reported_inside_loops_only():
+    spill = "\tscratch_store_dword off, v5, off offset:4\n"
+    straight = kernel(spill + "\tv_mov_b32_e32 v1, v2")
+    assert isa_check.scan_scratch_in_loops(straight) == []
+    loop = kernel("\ts_mov_b32 s4, 8\n.LBB0_1:\n" + spill + "\ts_sub_u32 s4, s4, 1\n\ts_cmp_lg_u32 s4, 0\n"
+                  "\ts_cbranch_scc1 .LBB0_1\n\tscratch_load_dword v5, off, off offset:4")
+    hits = isa_check.scan_scratch_in_loops(loop)
+    assert len(hits) == 1 and hits[0][1] == 1          # the reload behind the loop does not count
+    # a loop of several blocks (the access sits in a block that only the back edge closes)
+    nested = kernel("\ts_mov_b32 s4, 8\n.LBB0_1:\n\ts_cbranch_scc0 .LBB0_3\n.LBB0_2:\n" + spill +
+                    ".LBB0_3:\n\ts_sub_u32 s4, s4, 1\n\ts_cmp_lg_u32 s4, 0\n\ts_cbranch_scc1 .LBB0_1")
+    assert len(isa_check.scan_scratch_in_loops(nested)) == 1
+    # allowed by name
+    assert isa_check.scan_scratch_in_loops(loop, allowed={"k0": "test"}) == []
