@@ -141,8 +141,12 @@ __device__ __forceinline__ void rms_bwd_fetch(Pack<T, VEC> (&px)[ITERS], Pack<T,
         px[j] = ld_pack_nt<T, VEC>(x + row * (int64_t)N + col);
         pd[j] = ld_pack_nt<T, VEC>(dy + row * (int64_t)N + col);
       } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) px[j].v[e] = pd[j].v[e] = (T)0.f;
+        // (whole packs, not element by element: a pack that is written both as one 16-byte value and as 16-bit
+        // elements is left in scratch memory by the compiler)
+        Pack<T, VEC> zero;
+        __builtin_memset(&zero, 0, sizeof(zero));
+        px[j] = zero;
+        pd[j] = zero;
       }
     }
   }

@@ -319,8 +319,6 @@ def _blocks_in_loops(succ):
 
 # Kernels whose loops are known to touch scratch memory, with the reason each is tolerated.
 SCRATCH_IN_LOOP_ALLOWED = {
-    # rms_norm backward for rows of 8193..16384 elements: 1024 threads x 2 packs leave 128 registers a thread
-    "rms_bwd_rows_kernel": "three values of a 1024-thread variant live in scratch",
     # stream-K on the element-by-element stager: the last resort for operands contiguous along neither axis
     "gemm_streamk_kernel": "the element-wise stager of the last-resort stream-K kernel spills",
 }
