@@ -44,25 +44,55 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
   const bool row_ok = row < M;
   const T* xr = x + row * xs;
 
+  // What the tail of the kernel needs is requested before the row is read.  Fetched where it is used, the weight
+  // pack costs every workgroup a round trip to L2 behind the reduction, when it has no other request in flight, and
+  // each kernel argument first touched there a round trip to the scalar cache.  Up to two packs a thread (4 registers
+  // each for 16-bit types); longer rows keep the late fetch.
+  constexpr bool EARLY_W = ITERS <= 2 && sizeof(T) * VEC == 16;
+  u32x4 pw_early[EARLY_W ? ITERS : 1];
+  if constexpr (EARLY_W) {
+    const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      pw_early[j] = *reinterpret_cast<const u32x4*>(wp + (col < N ? col : 0));  // columns past the end are never stored
+    }
+  }
+  asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));
+
+  // All packs of the thread are requested before the first is used.  The loads are unconditional (a pack past the
+  // end of the row or of the matrix is read from the start of x and discarded): with a branch around each load the
+  // compiler finishes pack j, wait included, before it requests pack j + 1, one trip to memory per pack.
+  Pack<T, VEC> px[ITERS], pr[FUSED ? ITERS : 1];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    const bool ok = row_ok && col < N;
+    px[j] = ld_pack_nt<T, VEC>(ok ? xr + col : x);
+    if constexpr (FUSED) pr[j] = ld_pack_nt<T, VEC>(ok ? res + row * rs + col : x);
+  }
+  if constexpr (FUSED && ITERS == 1 && sizeof(T) * VEC == 16) {
+    // with one pack of each, the scheduler otherwise starts converting x before it has requested the residual;
+    // the empty asm needs both registers, so both requests go out first
+    asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&px[0])), "+v"(*reinterpret_cast<u32x4*>(&pr[0])));
+  }
   float v[ITERS][VEC];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
     if (row_ok && col < N) {
-      Pack<T, VEC> px = ld_pack_nt<T, VEC>(xr + col);
       if constexpr (FUSED) {
-        Pack<T, VEC> pr = ld_pack_nt<T, VEC>(res + row * rs + col);
         Pack<T, VEC> po;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          v[j][e] = (float)px.v[e] + (float)pr.v[e];
+          v[j][e] = (float)px[j].v[e] + (float)pr[j].v[e];
           po.v[e] = (T)v[j][e];
         }
         st_pack_nt<T, VEC>(res + row * rs + col, po);
       } else {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[j][e] = (float)px.v[e];
+        for (int e = 0; e < VEC; ++e) v[j][e] = (float)px[j].v[e];
       }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) ss += v[j][e] * v[j][e];
@@ -84,7 +114,16 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
     if (col < N) {
       Pack<T, VEC> po;
       if (w != nullptr) {
-        Pack<T, VEC> pw = ld_pack<T, VEC>(w + col);
+        Pack<T, VEC> pw;
+        if constexpr (EARLY_W) {
+          // (the registers pass through an empty asm so that the conversion to fp32, and with it the wait for the
+          // load, stays down here)
+          u32x4 raw = pw_early[j];
+          asm volatile("" : "+v"(raw));
+          pw = *reinterpret_cast<Pack<T, VEC>*>(&raw);
+        } else {
+          pw = ld_pack<T, VEC>(w + col);
+        }
 #pragma unroll
         for (int e = 0; e < VEC; ++e) po.v[e] = (T)(v[j][e] * rrms * (float)pw.v[e]);
       } else {

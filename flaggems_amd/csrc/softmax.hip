@@ -51,21 +51,27 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
   const bool row_ok = row < M;
   const TI* xr = in + row * (int64_t)N;
 
+  // All packs of the thread are requested before the first is used.  The loads are unconditional (a pack past the
+  // end of the row or of the matrix is read from the start of the input and discarded): with a branch around each
+  // load the compiler finishes pack j, wait included, before it requests pack j + 1, one trip to memory per pack.
+  Pack<TI, VEC> px[ITERS];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    px[j] = ld_pack_nt<TI, VEC>(row_ok && col < N ? xr + col : in);
+  }
+  // the output pointer is fetched with the other kernel arguments, not by a scalar load behind the last reduction
+  asm volatile("" : : "s"(out));
   float v[ITERS][VEC];
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
-    if (row_ok && col < N) {
-      Pack<TI, VEC> px = ld_pack_nt<TI, VEC>(xr + col);
+    const bool ok = row_ok && col < N;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        v[j][e] = (float)px.v[e];
-        m = fmaxf(m, v[j][e]);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) v[j][e] = -INFINITY;
+    for (int e = 0; e < VEC; ++e) {
+      v[j][e] = ok ? (float)px[j].v[e] : -INFINITY;
+      m = fmaxf(m, v[j][e]);
     }
   }
   // fmaxf drops NaN operands, but exp(NaN - m) below puts the NaN into the row sum, so a NaN
