@@ -70,23 +70,36 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
   const bool row_ok = row < M;
   const TI* ar = a + row * (int64_t)N;
   const TI* gr = g + row * (int64_t)N;
+  // All packs of the thread are requested before the first is used; the loads are unconditional (a pack past the end
+  // of the row or of the matrix is read from the start of the input and discarded).  With a branch around each pair
+  // of loads the compiler finishes pack j, wait included, before it requests pack j + 1.
+  Pack<TI, VEC> pa[ITERS], pg[ITERS];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int col = (j * TPR + t) * VEC;
+    const bool ok = row_ok && col < N;
+    pa[j] = ld_pack_nt<TI, VEC>(ok ? ar + col : a);
+    pg[j] = ld_pack_nt<TI, VEC>(ok ? gr + col : g);
+  }
+  asm volatile("" : : "s"(out));  // fetched with the other kernel arguments, not behind the reduction
+  if constexpr (sizeof(TI) * VEC == 16) {
+    // (the registers pass through an empty asm: without it the compiler moves a load whose value is only needed
+    // behind the reduction down to that use, where it costs a trip to memory of its own)
+#pragma unroll
+    for (int j = 0; j < ITERS; ++j)
+      asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&pa[j])), "+v"(*reinterpret_cast<u32x4*>(&pg[j])));
+  }
   float va[ITERS][VEC], vg[ITERS][VEC];
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
-    if (row_ok && col < N) {
-      const Pack<TI, VEC> pa = ld_pack_nt<TI, VEC>(ar + col);
-      const Pack<TI, VEC> pg = ld_pack_nt<TI, VEC>(gr + col);
+    const bool ok = row_ok && col < N;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        va[j][e] = (float)pa.v[e];
-        vg[j][e] = (float)pg.v[e];
-        s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) va[j][e] = vg[j][e] = 0.f;
+    for (int e = 0; e < VEC; ++e) {
+      va[j][e] = ok ? (float)pa[j].v[e] : 0.f;
+      vg[j][e] = ok ? (float)pg[j].v[e] : 0.f;
+      s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
     }
   }
   s = row_sum<TPR>(s, smem, row_in_block, t);
