@@ -345,7 +345,44 @@ def check_file(path):
              for k, n, first in scan_scratch_in_loops(text)])
 
 
+def memory_trace(text, name_part):
+    """One line per kernel whose name contains name_part: its vector-memory traffic in program order.
+    L load, D LDS-direct load, S store, A atomic, | barrier, (n) a wait that leaves n operations in flight,
+    k a scalar load issued after the first 40 instructions (a kernel argument fetched late), . a branch.
+    A well-formed streaming kernel reads `LL..L(n)..(0)|..|S..S`: every request before the first wait."""
+    lines = []
+    for km in _KERNEL.finditer(text):
+        if name_part not in km.group(1):
+            continue
+        out = []
+        for i, (op, _, line) in enumerate(_instructions(km.group(2))):
+            if op.startswith("global_load_lds") or (op.startswith("buffer_load") and line.endswith("lds")):
+                out.append("D")
+            elif op.startswith(("global_load", "buffer_load", "flat_load", "scratch_load")):
+                out.append("L")
+            elif op.startswith(("global_store", "buffer_store", "flat_store", "scratch_store")):
+                out.append("S")
+            elif op.startswith(("global_atomic", "buffer_atomic", "flat_atomic")):
+                out.append("A")
+            elif op == "s_barrier":
+                out.append("|")
+            elif op == "s_waitcnt" and "vmcnt" in line:
+                out.append("(%s)" % re.search(r"vmcnt\((\d+)\)", line).group(1))
+            elif op.startswith(("s_load", "s_buffer_load")) and i > 40:
+                out.append("k")
+            elif op.startswith(("s_cbranch", "s_branch")):
+                out.append(".")
+        lines.append("%s\n    %s" % (km.group(1), "".join(out)))
+    return lines
+
+
 if __name__ == "__main__":
+    if len(sys.argv) >= 4 and sys.argv[1] == "--trace":
+        # python isa_check.py --trace <part of a kernel name> <device .s files>
+        for p in sys.argv[3:]:
+            with open(p) as f:
+                print("\n".join(memory_trace(f.read(), sys.argv[2])))
+        sys.exit(0)
     bad = 0
     for p in sys.argv[1:]:
         found = check_file(p)

@@ -1,0 +1,54 @@
+"""Shape of the memory traffic of the row kernels at the benchmark configurations, read from the device assembly that
+the library's build keeps (flaggems_amd/csrc/build/*.s): every load is requested before the first wait, and no kernel
+argument is fetched late.  A branch around a load, or a value first touched behind a reduction, silently turns one trip
+to memory per row into several; the results stay right, so only a look at the generated code shows it.
+Skipped when the build's assembly is not there (the tests may run against a prebuilt library)."""
+import importlib.util
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BUILD = os.path.join(ROOT, "flaggems_amd", "csrc", "build")
+_spec = importlib.util.spec_from_file_location("fg_isa_check", os.path.join(ROOT, "flaggems_amd", "csrc", "isa_check.py"))
+isa_check = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(isa_check)
+
+# (source, kernel instantiation, what it serves)
+CASES = [
+    ("softmax", "softmax_rows_kernelIDF16bDF16bLi8ELi2ELi128ELb0", "softmax [131072, 2048] bf16"),
+    ("softmax", "softmax_rows_kernelIDF16bDF16bLi8ELi8ELi1024ELb0", "softmax, eight packs a thread"),
+    ("norm", "rms_rows_kernelIDF16bLi8ELi1ELi512ELb1", "fused_add_rms_norm [4096, 4096] bf16"),
+    ("norm", "rms_rows_kernelIfLi4ELi2ELi512ELb1", "fused_add_rms_norm [4096, 4096] fp32"),
+    ("norm", "rms_rows_kernelIDF16bLi8ELi1ELi512ELb0", "rms_norm [16384, 4096] bf16"),
+    ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi1ELi256ELi0", "softmax backward [131072, 2048] bf16"),
+    ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi4ELi1024ELi0", "softmax backward, four packs a thread"),
+    ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi2ELi1024ELi1", "log_softmax backward, two packs a thread"),
+]
+
+
+def _trace(source, kernel):
+    path = os.path.join(BUILD, "%s-hip-amdgcn-amd-amdhsa-gfx950.s" % source)
+    if not os.path.exists(path):
+        pytest.skip("no device assembly at %s (run flaggems_amd/csrc/build.py)" % path)
+    with open(path) as f:
+        lines = isa_check.memory_trace(f.read(), kernel)
+    assert len(lines) == 1, (kernel, len(lines))
+    return lines[0].split("\n")[1].strip().replace(".", "")
+
+
+@pytest.mark.parametrize("source,kernel,what", CASES)
+def test_every_request_goes_out_before_the_first_wait(source, kernel, what):
+    trace = _trace(source, kernel)
+    assert "k" not in trace, "%s: a kernel argument is fetched late: %s" % (what, trace)
+    head = re.match(r"^[L|]+", trace).group(0)
+    assert "L" not in trace[len(head):], "%s: a load is issued behind a wait: %s" % (what, trace)
+    assert trace.count("L") >= 1 and trace.rstrip("|").endswith("S"), trace
+
+
+def test_the_trace_reads_a_known_kernel():
+    text = ("k0:   ; @k0\n\ts_load_dwordx2 s[0:1], s[4:5], 0x0\n\tglobal_load_dwordx4 v[0:3], v8, s[0:1]\n"
+            "\ts_waitcnt vmcnt(0)\n\ts_cbranch_scc1 .LBB0_1\n.LBB0_1:\n\tglobal_load_dwordx4 v[4:7], v8, s[0:1]\n"
+            "\ts_barrier\n\ts_waitcnt vmcnt(0) lgkmcnt(0)\n\tglobal_store_dwordx4 v8, v[0:3], s[2:3]\n\ts_endpgm\n.Lfunc_end0:\n")
+    assert isa_check.memory_trace(text, "k0") == ["k0\n    L(0).L|(0)S"]
