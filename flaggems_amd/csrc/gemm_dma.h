@@ -171,9 +171,15 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
-        if (bias != nullptr) {
-          T4 t = brow[j];
-          if (!bcast && r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+        if (bcast) {
+          // (a branch of its own: merged with the per-element case below, the wait for that case's load lands
+          // behind the join and this case, which loads nothing, waits there for every store still in flight)
+          const T4 t = brow[j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
+        } else if (bias != nullptr) {
+          T4 t = T4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          if (r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
         } else if (scale) {
