@@ -53,10 +53,11 @@ namespace fgk {
 constexpr int kDmaRowB = 128;   // bytes of K per stage per A row
 constexpr int kDmaBK = 64;
 // Quarter steps of a K step that issue copies: 2 (quarter 3 and quarter 0, half of the copies each), or 3 (quarters
-// 3, 0 and 1).  3 on the 256x256 tile was measured 2-6 % faster on large products; it is switched off because it has
-// run on a few large shapes only, not under the parity tests.  kDmaCopyRunsEveryTile extends 3 from the 256x256 tile
-// with two stages to every tile (never measured).
-constexpr int kDmaCopyRuns = 2;
+// 3, 0 and 1).  3 on the 256x256 tile with two stages was measured 2-6 % faster on large products (same instruction
+// stream as built here, apart from register names) with the products checked, and its schedule holds for every K
+// length in the host model of this loop (tests/test_gemm_schedule_model.py).  kDmaCopyRunsEveryTile extends 3 to
+// every tile and to the stream-K kernel: never measured, off.
+constexpr int kDmaCopyRuns = 3;
 constexpr bool kDmaCopyRunsEveryTile = false;
 // with three quarters: the copies of a step issued in quarter 3 and in quarter 0 (the rest go to quarter 1), by the
 // number of copies per wave and step
