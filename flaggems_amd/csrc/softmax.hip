@@ -208,12 +208,20 @@ __global__ __launch_bounds__(256) void softmax_short_kernel(const TI* __restrict
   if (row >= M) return;  // the whole wave leaves
   const TI* xr = in + row * (int64_t)N;
   TO* yr = out + row * (int64_t)N;
+  // unconditional loads (a column past the end reads the row's first element and is discarded): with a branch
+  // around each the compiler waits for one before it requests the next, up to ITERS trips to memory per row
+  TI raw[ITERS];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    raw[j] = xr[c < N ? c : 0];
+  }
   float v[ITERS];
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    v[j] = c < N ? (float)xr[c] : -INFINITY;
+    v[j] = c < N ? (float)raw[j] : -INFINITY;
     m = fmaxf(m, v[j]);
   }
   m = wave_max(m);
