@@ -367,13 +367,23 @@ __global__ __launch_bounds__(256) void bwd_short_kernel(const TI* __restrict__ a
   const TI* ar = a + row * (int64_t)N;
   const TI* gr = g + row * (int64_t)N;
   TO* orow = out + row * (int64_t)N;
+  // unconditional loads (a column past the end reads column 0 and is discarded): with a branch around each the
+  // compiler waits for one before it requests the next, a trip to memory per element
+  TI araw[ITERS], graw[ITERS];
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    const int cc = c < N ? c : 0;
+    araw[j] = ar[cc];
+    graw[j] = gr[cc];
+  }
   float x[ITERS], d[ITERS];
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    x[j] = c < N ? (float)ar[c] : 0.f;
-    d[j] = c < N ? (float)gr[c] : 0.f;
+    x[j] = c < N ? (float)araw[j] : 0.f;
+    d[j] = c < N ? (float)graw[j] : 0.f;
     s += MODE == BWD_SOFTMAX ? x[j] * d[j] : d[j];
   }
   s = wave_sum(s);

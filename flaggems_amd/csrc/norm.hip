@@ -147,14 +147,27 @@ __global__ __launch_bounds__(256) void rms_short_kernel(const T* x, T* res, cons
   const T* xr = x + row * xs;
   T* rr = FUSED ? res + row * rs : nullptr;
   T* yr = y + row * ys;
+  // unconditional loads, the weights included (a column past the end reads column 0 and is discarded): with a
+  // branch around each the compiler waits for one before it requests the next, a trip to memory per element
+  T xraw[ITERS], rraw[FUSED ? ITERS : 1], wraw[ITERS];
+  const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
+  asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));  // the tail's arguments are fetched with the others
+#pragma unroll
+  for (int j = 0; j < ITERS; ++j) {
+    const int c = j * 64 + lane;
+    const int cc = c < N ? c : 0;
+    xraw[j] = xr[cc];
+    if constexpr (FUSED) rraw[j] = rr[cc];
+    wraw[j] = wp[cc];
+  }
   float v[ITERS];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    v[j] = c < N ? (float)xr[c] : 0.f;
+    v[j] = c < N ? (float)xraw[j] : 0.f;
     if constexpr (FUSED) {
-      if (c < N) v[j] += (float)rr[c];
+      if (c < N) v[j] += (float)rraw[j];
     }
     ss += v[j] * v[j];
   }
@@ -168,7 +181,7 @@ __global__ __launch_bounds__(256) void rms_short_kernel(const T* x, T* res, cons
     const int c = j * 64 + lane;
     if (c < N) {
       if constexpr (FUSED) rr[c] = (T)v[j];
-      yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)w[c] : 1.0f));
+      yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)wraw[j] : 1.0f));
     }
   }
 }

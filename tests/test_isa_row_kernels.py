@@ -25,6 +25,9 @@ CASES = [
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi1ELi256ELi0", "softmax backward [131072, 2048] bf16"),
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi4ELi1024ELi0", "softmax backward, four packs a thread"),
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi2ELi1024ELi1", "log_softmax backward, two packs a thread"),
+    ("softmax", "softmax_short_kernelIDF16bDF16bLb0ELi16", "softmax, a wave per row of up to 1024 elements"),
+    ("backward", "bwd_short_kernelIDF16bDF16bLi0ELi8", "softmax backward, a wave per row of up to 512 elements"),
+    ("norm", "rms_short_kernelIDF16bLb0ELi8", "rms_norm, a wave per unaligned row of up to 512 elements"),
 ]
 
 
