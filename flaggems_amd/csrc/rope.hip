@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
 
   const bool is_q = h < a.Hq;
   const int hh = is_q ? h : h - a.Hq;
-  // the strides are selected by value: selecting a pointer into the argument block makes each stride a vector load
-  // from memory, two trips in front of everything else
+  // the strides are selected by value: selecting a pointer into the argument block makes them a vector load from
+  // memory, a trip of its own in front of the row
   const int64_t is[3] = {is_q ? a.qs[0] : a.ks[0], is_q ? a.qs[1] : a.ks[1], is_q ? a.qs[2] : a.ks[2]};
   const int64_t os[3] = {is_q ? a.qos[0] : a.kos[0], is_q ? a.qos[1] : a.kos[1], is_q ? a.qos[2] : a.kos[2]};
   const T* src = (const T*)(is_q ? a.q : a.k) + tok * is[0] + hh * is[1];
