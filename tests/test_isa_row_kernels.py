@@ -55,3 +55,23 @@ def test_the_trace_reads_a_known_kernel():
             "\ts_waitcnt vmcnt(0)\n\ts_cbranch_scc1 .LBB0_1\n.LBB0_1:\n\tglobal_load_dwordx4 v[4:7], v8, s[0:1]\n"
             "\ts_barrier\n\ts_waitcnt vmcnt(0) lgkmcnt(0)\n\tglobal_store_dwordx4 v8, v[0:3], s[2:3]\n\ts_endpgm\n.Lfunc_end0:\n")
     assert isa_check.memory_trace(text, "k0") == ["k0\n    L(0).L|(0)S"]
+
+
+def _groups(trace):
+    """Runs of loads between waits: 'LL(1)(0)LLL(0)S' -> [2, 3]."""
+    return [len(g) for g in re.findall(r"L+", trace)]
+
+
+def test_rope_reads_position_then_everything_else_in_one_batch():
+    trace = _trace("rope", "rope_kernelIDF16bDF16bLi8ELb0")
+    first = trace.index("L")
+    assert "k" not in trace[first:], trace            # every argument is fetched before the first load
+    groups = _groups(trace)
+    # the position (one load in each arm of the int64 / int32 branch), then cos, sin and the two halves of the row
+    assert groups[-1] == 4 and sum(groups[:-1]) == 2, trace
+
+
+def test_cache_scatter_requests_the_row_with_the_slot():
+    trace = _trace("kvcache", "cache_scatter_kernelIDv4_jl")
+    assert "k" not in trace[trace.index("L"):], trace
+    assert _groups(trace)[0] == 5, trace              # four pieces of the row and the slot, one wait for all
