@@ -12,7 +12,8 @@ import threading
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libfg_mi355.so")
+# FG_LIB_PATH names another build of the same library (csrc/build.py --variant ... --tag TAG: kernel variants on trial)
+LIB_PATH = os.environ.get("FG_LIB_PATH") or os.path.join(_HERE, "libfg_mi355.so")
 
 FG_F16, FG_BF16, FG_F32 = 0, 1, 2
 SCHED_AUTO, SCHED_DATA_PARALLEL, SCHED_STREAM_K = 0, 1, 2

@@ -1,6 +1,7 @@
 // Host-only part of libfg_mi355.so: error channel, device facts, stream-K partition arithmetic.
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include "fg_common.h"
 
@@ -25,7 +26,10 @@ int fg_check_launch(const char* what) {
 }
 
 namespace {
-FgOptions g_opt;
+// The current switches are an immutable snapshot behind an atomic pointer: fg_reload_options() publishes a new one
+// and never frees the old (a few dozen bytes per reload), so a thread that reads fg_options() while another reloads
+// sees either snapshot whole, and a reference it still holds stays valid.
+std::atomic<const FgOptions*> g_opt{nullptr};
 std::once_flag g_opt_once;
 void load_options() {
   FgOptions o = {};
@@ -54,13 +58,13 @@ void load_options() {
     const int v = atoi(e);
     if (v >= 1 && v <= 64) o.decode_wg_per_cu = v;
   }
-  g_opt = o;
+  g_opt.store(new FgOptions(o), std::memory_order_release);
 }
 }  // namespace
 
 const FgOptions& fg_options() {
   std::call_once(g_opt_once, load_options);
-  return g_opt;
+  return *g_opt.load(std::memory_order_acquire);
 }
 
 extern "C" void fg_reload_options(void) {
@@ -69,6 +73,8 @@ extern "C" void fg_reload_options(void) {
 }
 
 extern "C" const char* fg_last_error(void) { return g_err; }
+
+void fg_static_scratch_prime(int device);  // gemm_skinny.hip
 
 extern "C" int fg_abi_version(void) { return 2; }
 
@@ -93,5 +99,7 @@ extern "C" int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_
     }
     *gcn_arch = arch;  // 0x950 for MI355X
   }
+  // the one piece of per-device set-up the library has: the address of fg_gemm_skinny_static's scratch array
+  fg_static_scratch_prime(device);
   return FG_OK;
 }

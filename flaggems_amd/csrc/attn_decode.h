@@ -84,6 +84,20 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
   if (split > 0 && t_begin >= t_end) return;
   const bool has_work = t_begin < t_end;
 
+#if !FG_V_DECODE_Q_EARLY
+  // ---- Q fragments: row r < G is query head kvh*G + r of this sequence's token; other rows are zero ---------
+  Frag qf[KS];
+  {
+    const bool row_ok = ql < G && q_len == 1;
+    const T* qp = (const T*)p.q + (int64_t)q_bos * p.q_row_stride + (int64_t)(kvh * G + (row_ok ? ql : 0)) * p.q_head_stride;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok) v = *reinterpret_cast<const u32x4*>(qp + ks * 16 + half * 8);
+      qf[ks] = __builtin_bit_cast(Frag, v);
+    }
+  }
+#endif
   f32x16 o_acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
@@ -104,7 +118,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
     pgc[r] = has_work ? btab[pg] : 0;
   }
   const int last_page_id = has_work ? btab[last_page] : 0;
-  // ---- Q fragments: row r < G is query head kvh*G + r of this sequence's token; other rows are zero ---------
+#if FG_V_DECODE_Q_EARLY
+  // ---- Q fragments (variant FG_V_DECODE_Q_EARLY, variants.h): row r < G is query head kvh*G + r of this
+  // sequence's token; other rows are zero.
   // Requested unconditionally (qp is clamped to a row that exists) together with the page ids, and not touched
   // before the one wait below: under a branch of its own each load was waited for before the next request, and the
   // page ids went out a trip later.
@@ -115,9 +131,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qp + ks * 16 + half * 8);
   }
+#endif
   // Everything loaded so far is complete from here on (stated explicitly: once tile DMAs are in flight the
   // compiler could only wait for all of them together with these loads).
   FG_WAIT_VM(0);
+#if FG_V_DECODE_Q_EARLY
   Frag qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -126,6 +144,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs a) {
     if (!q_row_ok) v = u32x4{0u, 0u, 0u, 0u};
     qf[ks] = __builtin_bit_cast(Frag, v);
   }
+#endif
 
   const char* kbase = (const char*)((const T*)p.k_cache + (int64_t)kvh * p.k_head_stride);
   const char* vbase = (const char*)((const T*)p.v_cache + (int64_t)kvh * p.v_head_stride);

@@ -193,18 +193,25 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     const T* qp = (const T*)p.q + (int64_t)(q_bos + (row_ok ? qrow : 0)) * p.q_row_stride + (int64_t)head * p.q_head_stride;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      // unconditional: rows past the end read row 0 of the sequence (qp is clamped) and are zeroed afterwards; a
-      // branch around each load makes the compiler wait for one before it requests the next
-      u32x4 v = *reinterpret_cast<const u32x4*>(qp + kk * 32 + g * 8);
-      if (!row_ok) v = u32x4{0u, 0u, 0u, 0u};
+      // Variant FG_V_ATTN_Q_UNCOND (variants.h; off: each load under the row check).  Unconditional: rows past the
+      // end read row 0 of the sequence (qp is clamped) and are zeroed afterwards; a branch around each load makes the
+      // compiler wait for one before it requests the next
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if constexpr (FG_V_ATTN_Q_UNCOND != 0) {
+        v = *reinterpret_cast<const u32x4*>(qp + kk * 32 + g * 8);
+        if (!row_ok) v = u32x4{0u, 0u, 0u, 0u};
+      } else {
+        if (row_ok) v = *reinterpret_cast<const u32x4*>(qp + kk * 32 + g * 8);
+      }
       Frag f = __builtin_bit_cast(Frag, v);
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = (T)((float)f[e] * a.scale_log2);
       qf[qt][kk] = f;
     }
-    // the conversions of the two column tiles are not interleaved: scheduled freely, the register allocator put the
-    // reload of a spilled register in front of the first barrier, and with it a wait for every copy in flight
-    __builtin_amdgcn_sched_barrier(0);
+    // (with the variant) the conversions of the two column tiles are not interleaved: scheduled freely, the register
+    // allocator put the reload of a spilled register in front of the first barrier, and with it a wait for every copy
+    // in flight
+    if constexpr (FG_V_ATTN_Q_UNCOND != 0) __builtin_amdgcn_sched_barrier(0);
   }
   f32x4 minit[QT];          // -m of the lane's row, four times: C operand of the first MFMA of a score tile
   f32x4 o_acc[QT][NPV];

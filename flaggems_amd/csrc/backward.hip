@@ -73,33 +73,51 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void bwd_rows_kernel(const T
   // All packs of the thread are requested before the first is used; the loads are unconditional (a pack past the end
   // of the row or of the matrix is read from the start of the input and discarded).  With a branch around each pair
   // of loads the compiler finishes pack j, wait included, before it requests pack j + 1.
+  // (variant FG_V_ROWS_UPFRONT, variants.h; off: every pair of packs is loaded where it is used, under its bounds check)
+  constexpr bool UPFRONT = FG_V_ROWS_UPFRONT != 0;
   Pack<TI, VEC> pa[ITERS], pg[ITERS];
+  if constexpr (UPFRONT) {
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int col = (j * TPR + t) * VEC;
-    const bool ok = row_ok && col < N;
-    pa[j] = ld_pack_nt<TI, VEC>(ok ? ar + col : a);
-    pg[j] = ld_pack_nt<TI, VEC>(ok ? gr + col : g);
-  }
-  asm volatile("" : : "s"(out));  // fetched with the other kernel arguments, not behind the reduction
-  if constexpr (sizeof(TI) * VEC == 16) {
-    // (the registers pass through an empty asm: without it the compiler moves a load whose value is only needed
-    // behind the reduction down to that use, where it costs a trip to memory of its own)
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      const bool ok = row_ok && col < N;
+      pa[j] = ld_pack_nt<TI, VEC>(ok ? ar + col : a);
+      pg[j] = ld_pack_nt<TI, VEC>(ok ? gr + col : g);
+    }
+    asm volatile("" : : "s"(out));  // fetched with the other kernel arguments, not behind the reduction
+    if constexpr (sizeof(TI) * VEC == 16) {
+      // (the registers pass through an empty asm: without it the compiler moves a load whose value is only needed
+      // behind the reduction down to that use, where it costs a trip to memory of its own)
 #pragma unroll
-    for (int j = 0; j < ITERS; ++j)
-      asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&pa[j])), "+v"(*reinterpret_cast<u32x4*>(&pg[j])));
+      for (int j = 0; j < ITERS; ++j)
+        asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&pa[j])), "+v"(*reinterpret_cast<u32x4*>(&pg[j])));
+    }
   }
   float va[ITERS][VEC], vg[ITERS][VEC];
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
-    const bool ok = row_ok && col < N;
+    if constexpr (UPFRONT) {
+      const bool ok = row_ok && col < N;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      va[j][e] = ok ? (float)pa[j].v[e] : 0.f;
-      vg[j][e] = ok ? (float)pg[j].v[e] : 0.f;
-      s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
+      for (int e = 0; e < VEC; ++e) {
+        va[j][e] = ok ? (float)pa[j].v[e] : 0.f;
+        vg[j][e] = ok ? (float)pg[j].v[e] : 0.f;
+        s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
+      }
+    } else if (row_ok && col < N) {
+      pa[j] = ld_pack_nt<TI, VEC>(ar + col);
+      pg[j] = ld_pack_nt<TI, VEC>(gr + col);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        va[j][e] = (float)pa[j].v[e];
+        vg[j][e] = (float)pg[j].v[e];
+        s += MODE == BWD_SOFTMAX ? va[j][e] * vg[j][e] : vg[j][e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) va[j][e] = vg[j][e] = 0.f;
     }
   }
   s = row_sum<TPR>(s, smem, row_in_block, t);
@@ -154,12 +172,17 @@ __device__ __forceinline__ void rms_bwd_fetch(Pack<T, VEC> (&px)[ITERS], Pack<T,
         px[j] = ld_pack_nt<T, VEC>(x + row * (int64_t)N + col);
         pd[j] = ld_pack_nt<T, VEC>(dy + row * (int64_t)N + col);
       } else {
-        // (whole packs, not element by element: a pack that is written both as one 16-byte value and as 16-bit
-        // elements is left in scratch memory by the compiler)
+#if FG_V_RMS_BWD_ZERO_PACK
+        // (variant, variants.h: whole packs, not element by element: a pack that is written both as one 16-byte value
+        // and as 16-bit elements is left in scratch memory by the compiler)
         Pack<T, VEC> zero;
         __builtin_memset(&zero, 0, sizeof(zero));
         px[j] = zero;
         pd[j] = zero;
+#else
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) px[j].v[e] = pd[j].v[e] = (T)0.f;
+#endif
       }
     }
   }
@@ -369,21 +392,30 @@ __global__ __launch_bounds__(256) void bwd_short_kernel(const TI* __restrict__ a
   TO* orow = out + row * (int64_t)N;
   // unconditional loads (a column past the end reads column 0 and is discarded): with a branch around each the
   // compiler waits for one before it requests the next, a trip to memory per element
+  // (variant FG_V_SHORT_UPFRONT, variants.h; off: every element is loaded where it is used, under its bounds check)
+  constexpr bool UPFRONT = FG_V_SHORT_UPFRONT != 0;
   TI araw[ITERS], graw[ITERS];
+  if constexpr (UPFRONT) {
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int c = j * 64 + lane;
-    const int cc = c < N ? c : 0;
-    araw[j] = ar[cc];
-    graw[j] = gr[cc];
+    for (int j = 0; j < ITERS; ++j) {
+      const int c = j * 64 + lane;
+      const int cc = c < N ? c : 0;
+      araw[j] = ar[cc];
+      graw[j] = gr[cc];
+    }
   }
   float x[ITERS], d[ITERS];
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    x[j] = c < N ? (float)araw[j] : 0.f;
-    d[j] = c < N ? (float)graw[j] : 0.f;
+    if constexpr (UPFRONT) {
+      x[j] = c < N ? (float)araw[j] : 0.f;
+      d[j] = c < N ? (float)graw[j] : 0.f;
+    } else {
+      x[j] = c < N ? (float)ar[c] : 0.f;
+      d[j] = c < N ? (float)gr[c] : 0.f;
+    }
     s += MODE == BWD_SOFTMAX ? x[j] * d[j] : d[j];
   }
   s = wave_sum(s);

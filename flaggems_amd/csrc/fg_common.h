@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <stdarg.h>
 #include "../../include/fg_mi355.h"
+#include "variants.h"
 
 // ---------------------------------------------------------------------------------------------
 // host side: error reporting

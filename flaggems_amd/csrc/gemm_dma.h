@@ -55,9 +55,10 @@ constexpr int kDmaBK = 64;
 // Quarter steps of a K step that issue copies: 2 (quarter 3 and quarter 0, half of the copies each), or 3 (quarters
 // 3, 0 and 1).  3 on the 256x256 tile with two stages was measured 2-6 % faster on large products (same instruction
 // stream as built here, apart from register names) with the products checked, and its schedule holds for every K
-// length in the host model of this loop (tests/test_gemm_schedule_model.py).  kDmaCopyRunsEveryTile extends 3 to
+// length in the host model of this loop (tests/test_gemm_schedule_model.py), but it has not been through the parity
+// suite: the value comes from FG_V_DMA_COPY_RUNS (variants.h, default 2).  kDmaCopyRunsEveryTile extends 3 to
 // every tile and to the stream-K kernel: never measured, off.
-constexpr int kDmaCopyRuns = 3;
+constexpr int kDmaCopyRuns = FG_V_DMA_COPY_RUNS;
 constexpr bool kDmaCopyRunsEveryTile = false;
 // with three quarters: the copies of a step issued in quarter 3 and in quarter 0 (the rest go to quarter 1), by the
 // number of copies per wave and step
@@ -172,9 +173,11 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
+#if FG_V_ADDMM_BCAST_BRANCH
         if (bcast) {
-          // (a branch of its own: merged with the per-element case below, the wait for that case's load lands
-          // behind the join and this case, which loads nothing, waits there for every store still in flight)
+          // (variant, variants.h: a branch of its own: merged with the per-element case below, the wait for that
+          // case's load lands behind the join and this case, which loads nothing, waits there for every store still
+          // in flight)
           const T4 t = brow[j];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
@@ -184,6 +187,14 @@ __device__ __forceinline__ void dma_tile_epilogue(const GemmArgs& g, int tm, int
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
         } else if (scale) {
+#else
+        if (bias != nullptr) {
+          T4 t = brow[j];
+          if (!bcast && r < M && c < N) t = *reinterpret_cast<const T4*>(bias + r * g.sim + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = v[e] * alpha + (float)t[e] * beta;
+        } else if (scale) {
+#endif
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] *= alpha;
         }
@@ -294,9 +305,16 @@ __device__ __forceinline__ void dma_tile_mainloop(const GemmArgs& g, char* lds, 
   // states behind them; what bases_of() derives from them is scalar arithmetic on scalar registers, which has no
   // such rule.  (The tile's row and column come from integer divisions, which run on the vector unit: without
   // this, how far a v_readfirstlane lands ahead of the first copy is up to the instruction scheduler.)
+  // Variant FG_V_DMA_SCALAR_BASES (variants.h).  Off, the tested code: bases_of() makes the bases scalar per K step, and
+  // the build's scan of the device assembly (isa_check.py) is what establishes that no copy follows a
+  // v_readfirstlane too closely.
+#if FG_V_DMA_SCALAR_BASES
   a_base = uniform_ptr(a_base);
   b_base = uniform_ptr(b_base);
   asm volatile("s_nop 4" : "+s"(a_base), "+s"(b_base));
+#else
+  static_assert(!kDmaCopyRunsEveryTile, "the three-quarter split on every tile needs FG_V_DMA_SCALAR_BASES");
+#endif
   struct KBase { const char* a; const char* b; bool last; };
   auto bases_of = [&](int kk) {
     return KBase{uniform_ptr(a_base + (int64_t)kk * kDmaRowB), uniform_ptr(b_base + (int64_t)kk * b_step), RAGGED && kk == nk - 1};

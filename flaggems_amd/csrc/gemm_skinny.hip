@@ -631,17 +631,28 @@ __global__ void clear_tickets_kernel(unsigned* tickets, int n) {
 
 // Device address of this GPU's copy of `scratch`, looked up once per device with that device current.
 // In host code the array's name is only a handle for this lookup, never an address to hand to a kernel.
-int static_scratch(unsigned char** out) {
-  static std::mutex mu;
-  static unsigned char* ptr[64] = {nullptr};
+// The lookup is not a stream operation and may load the code object: it must not happen while `st` is being
+// captured, so a first call on a device that arrives under capture is refused (fg_device_info on that device, or
+// any eager call of the entry point, makes the lookup beforehand).
+std::mutex g_static_mu;
+unsigned char* g_static_ptr[64] = {nullptr};
+
+int static_scratch(unsigned char** out, hipStream_t st, bool launching = true) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= 64) {
     fg_set_error("gemm_skinny_static: cannot identify the current device: %s", hipGetErrorString(e));
     return FG_ERR_INVALID;
   }
-  std::lock_guard<std::mutex> lk(mu);
-  if (ptr[dev] == nullptr) {
+  std::lock_guard<std::mutex> lk(g_static_mu);
+  if (g_static_ptr[dev] == nullptr) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (launching && hipStreamIsCapturing(st, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone) {
+      fg_set_error("gemm_skinny_static: the first call on device %d came under stream capture; call fg_device_info(%d, "
+                   "...) or this entry point once outside capture first", dev, dev);
+      return FG_ERR_UNSUPPORTED;
+    }
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || p == nullptr) {
@@ -649,12 +660,30 @@ int static_scratch(unsigned char** out) {
       fg_set_error("gemm_skinny_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
       return FG_ERR_LAUNCH;
     }
-    ptr[dev] = (unsigned char*)p;
+    g_static_ptr[dev] = (unsigned char*)p;
   }
-  *out = ptr[dev];
+  *out = g_static_ptr[dev];
   return FG_OK;
 }
 }  // namespace
+
+// Called by fg_device_info (abi.cpp): looks the address up for `device` ahead of the first call, so that the first
+// fg_gemm_skinny_static on that device may come under stream capture.  Failure is not an error of fg_device_info;
+// the entry point reports it when it is called.
+void fg_static_scratch_prime(int device) {
+  int cur = 0;
+  if (hipGetDevice(&cur) != hipSuccess) { (void)hipGetLastError(); return; }
+  if (device < 0) device = cur;
+  if (device >= 64) return;
+  {
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (g_static_ptr[device] != nullptr) return;
+  }
+  if (device != cur && hipSetDevice(device) != hipSuccess) { (void)hipGetLastError(); return; }
+  unsigned char* p = nullptr;
+  (void)static_scratch(&p, nullptr, /*launching=*/false);
+  if (device != cur) (void)hipSetDevice(cur);
+}
 
 extern "C" int fg_gemm_skinny_static(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                                      int64_t K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim,
@@ -689,13 +718,15 @@ extern "C" int fg_gemm_skinny_static(const void* A, const void* B, const void* b
              "gemm_skinny_static: this device (%d CUs) needs %zu bytes of scratch, the static buffer holds %zu", cu, need,
              kStaticScratchBytes);
   unsigned char* ws = nullptr;
-  const int rc = static_scratch(&ws);
-  if (rc != FG_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
+  const int rc = static_scratch(&ws, st);
+  if (rc != FG_OK) return rc;
   // The array keeps what the last call left.  The ticket counters must read zero when the kernel starts: cleared
   // by a small kernel (a memset node would not be safe to record into a caller's graph).
   hipLaunchKernelGGL(clear_tickets_kernel, dim3(kMaxWorkers / 256), dim3(256), 0, st, (unsigned*)(ws + kTicketOffset),
                      kMaxWorkers);
+  const int rc_clear = fg_check_launch("gemm_skinny_static(clear tickets)");
+  if (rc_clear != FG_OK) return rc_clear;
   return skinny_launch(g, ab_dtype, kind, ws, kStaticScratchBytes, cu, st);
 }
 

@@ -321,6 +321,11 @@ def _blocks_in_loops(succ):
 SCRATCH_IN_LOOP_ALLOWED = {
     # stream-K on the element-by-element stager: the last resort for operands contiguous along neither axis
     "gemm_streamk_kernel": "the element-wise stager of the last-resort stream-K kernel spills",
+    # rms_norm backward for rows of 8193-16384 elements, in the code the GPU parity suite last passed on: a pack
+    # zeroed element by element stays in scratch.  variants.h: FG_V_RMS_BWD_ZERO_PACK removes it (not yet GPU-tested).
+    "rms_bwd_rows_kernelIDF16_Li8ELi2ELi1024ELb0": "tested code keeps a two-pack row partly in scratch",
+    "rms_bwd_rows_kernelIDF16bLi8ELi2ELi1024ELb0": "tested code keeps a two-pack row partly in scratch",
+    "rms_bwd_rows_kernelIfLi4ELi2ELi1024ELb0": "tested code keeps a two-pack row partly in scratch",
 }
 
 
@@ -343,6 +348,23 @@ def check_file(path):
     return (scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] + scan_packed_f32(text) +
             [(k, 0, first, "%d scratch accesses inside a loop: registers spill there" % n)
              for k, n, first in scan_scratch_in_loops(text)])
+
+
+def kernel_digests(text):
+    """{kernel: (sha1 of its instruction stream, instruction and label lines)}.  Comments are dropped and the
+    per-function number in basic-block labels (.LBB<n>_<m>) is removed, so that a kernel's digest does not depend on
+    which other kernels its source instantiates; registers, immediates and instruction order all count."""
+    import hashlib
+
+    out = {}
+    for km in _KERNEL.finditer(text):
+        lines = []
+        for line in km.group(2).split("\n"):
+            line = re.sub(r"\.LBB\d+_", ".LBB_", line.split(";")[0].rstrip())
+            if line.strip():
+                lines.append(line)
+        out[km.group(1)] = (hashlib.sha1("\n".join(lines).encode()).hexdigest(), len(lines))
+    return out
 
 
 def memory_trace(text, name_part):

@@ -19,13 +19,15 @@ __global__ __launch_bounds__(256) void cache_scatter_kernel(const char* __restri
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, tensor) pair
   const int64_t tok = w >> 1;
   if (tok >= num_tokens) return;
+#if FG_V_SCATTER_EARLY
+  // Variant (variants.h): the first four pieces of the row are requested together with the slot, which only the
+  // stores depend on (a padding token's row is read for nothing): behind the slot they would cost a trip to memory
+  // of their own.
   const bool is_v = w & 1;
   const U* src = reinterpret_cast<const U*>(is_v ? value + tok * value_stride_b : key + tok * key_stride_b);
   const int64_t n = row_bytes / (int64_t)sizeof(U);
   // four pieces per lane in flight: the row is short, so the copy lives on memory-level parallelism
   int64_t i = threadIdx.x & 63;
-  // The first four pieces of the row are requested together with the slot, which only the stores depend on (a
-  // padding token's row is read for nothing): behind the slot they would cost a trip to memory of their own.
   asm volatile("" : : "s"(kc), "s"(vc), "s"(block_stride_b), "s"(block_size));  // fetched with the other arguments
   const bool first4 = i + 192 < n;
   U a0, b0, c0, d0;
@@ -47,6 +49,18 @@ __global__ __launch_bounds__(256) void cache_scatter_kernel(const char* __restri
     __builtin_nontemporal_store(d0, dst + i + 192);
     i += 256;
   }
+#else
+  const int64_t slot = (int64_t)slots[tok];
+  if (slot < 0) return;  // padding token
+  const int64_t blk = slot / block_size;
+  const int64_t off = slot - blk * block_size;
+  const bool is_v = w & 1;
+  const U* src = reinterpret_cast<const U*>(is_v ? value + tok * value_stride_b : key + tok * key_stride_b);
+  U* dst = reinterpret_cast<U*>((is_v ? vc : kc) + blk * block_stride_b + off * row_bytes);
+  const int64_t n = row_bytes / (int64_t)sizeof(U);
+  // four pieces per lane in flight: the row is short, so the copy lives on memory-level parallelism
+  int64_t i = threadIdx.x & 63;
+#endif
   // streaming accesses: neither the token rows nor the cache lines written here are read again soon
   for (; i + 192 < n; i += 256) {
     const U a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + 64),

@@ -44,11 +44,13 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
   const bool row_ok = row < M;
   const T* xr = x + row * xs;
 
+  // Variant FG_V_ROWS_UPFRONT (variants.h; off: every pack is loaded where it is used, under its bounds check).
   // What the tail of the kernel needs is requested before the row is read.  Fetched where it is used, the weight
   // pack costs every workgroup a round trip to L2 behind the reduction, when it has no other request in flight, and
   // each kernel argument first touched there a round trip to the scalar cache.  Up to two packs a thread (4 registers
   // each for 16-bit types); longer rows keep the late fetch.
-  constexpr bool EARLY_W = ITERS <= 2 && sizeof(T) * VEC == 16;
+  constexpr bool UPFRONT = FG_V_ROWS_UPFRONT != 0;
+  constexpr bool EARLY_W = UPFRONT && ITERS <= 2 && sizeof(T) * VEC == 16;
   u32x4 pw_early[EARLY_W ? ITERS : 1];
   if constexpr (EARLY_W) {
     const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
@@ -58,20 +60,22 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
       pw_early[j] = *reinterpret_cast<const u32x4*>(wp + (col < N ? col : 0));  // columns past the end are never stored
     }
   }
-  asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));
+  if constexpr (UPFRONT) asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));
 
   // All packs of the thread are requested before the first is used.  The loads are unconditional (a pack past the
   // end of the row or of the matrix is read from the start of x and discarded): with a branch around each load the
   // compiler finishes pack j, wait included, before it requests pack j + 1, one trip to memory per pack.
   Pack<T, VEC> px[ITERS], pr[FUSED ? ITERS : 1];
+  if constexpr (UPFRONT) {
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int col = (j * TPR + t) * VEC;
-    const bool ok = row_ok && col < N;
-    px[j] = ld_pack_nt<T, VEC>(ok ? xr + col : x);
-    if constexpr (FUSED) pr[j] = ld_pack_nt<T, VEC>(ok ? res + row * rs + col : x);
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      const bool ok = row_ok && col < N;
+      px[j] = ld_pack_nt<T, VEC>(ok ? xr + col : x);
+      if constexpr (FUSED) pr[j] = ld_pack_nt<T, VEC>(ok ? res + row * rs + col : x);
+    }
   }
-  if constexpr (FUSED && ITERS == 1 && sizeof(T) * VEC == 16) {
+  if constexpr (UPFRONT && FUSED && ITERS == 1 && sizeof(T) * VEC == 16) {
     // with one pack of each, the scheduler otherwise starts converting x before it has requested the residual;
     // the empty asm needs both registers, so both requests go out first
     asm volatile("" : "+v"(*reinterpret_cast<u32x4*>(&px[0])), "+v"(*reinterpret_cast<u32x4*>(&pr[0])));
@@ -82,7 +86,9 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
     if (row_ok && col < N) {
+      if constexpr (!UPFRONT) px[j] = ld_pack_nt<T, VEC>(xr + col);
       if constexpr (FUSED) {
+        if constexpr (!UPFRONT) pr[j] = ld_pack_nt<T, VEC>(res + row * rs + col);
         Pack<T, VEC> po;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -147,27 +153,38 @@ __global__ __launch_bounds__(256) void rms_short_kernel(const T* x, T* res, cons
   const T* xr = x + row * xs;
   T* rr = FUSED ? res + row * rs : nullptr;
   T* yr = y + row * ys;
+  // Variant FG_V_SHORT_UPFRONT (variants.h; off: every element is loaded where it is used, under its bounds check):
   // unconditional loads, the weights included (a column past the end reads column 0 and is discarded): with a
   // branch around each the compiler waits for one before it requests the next, a trip to memory per element
+  constexpr bool UPFRONT = FG_V_SHORT_UPFRONT != 0;
   T xraw[ITERS], rraw[FUSED ? ITERS : 1], wraw[ITERS];
-  const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
-  asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));  // the tail's arguments are fetched with the others
+  if constexpr (UPFRONT) {
+    const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
+    asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));  // the tail's arguments are fetched with the others
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int c = j * 64 + lane;
-    const int cc = c < N ? c : 0;
-    xraw[j] = xr[cc];
-    if constexpr (FUSED) rraw[j] = rr[cc];
-    wraw[j] = wp[cc];
+    for (int j = 0; j < ITERS; ++j) {
+      const int c = j * 64 + lane;
+      const int cc = c < N ? c : 0;
+      xraw[j] = xr[cc];
+      if constexpr (FUSED) rraw[j] = rr[cc];
+      wraw[j] = wp[cc];
+    }
   }
   float v[ITERS];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    v[j] = c < N ? (float)xraw[j] : 0.f;
-    if constexpr (FUSED) {
-      if (c < N) v[j] += (float)rraw[j];
+    if constexpr (UPFRONT) {
+      v[j] = c < N ? (float)xraw[j] : 0.f;
+      if constexpr (FUSED) {
+        if (c < N) v[j] += (float)rraw[j];
+      }
+    } else {
+      v[j] = c < N ? (float)xr[c] : 0.f;
+      if constexpr (FUSED) {
+        if (c < N) v[j] += (float)rr[c];
+      }
     }
     ss += v[j] * v[j];
   }
@@ -181,7 +198,8 @@ __global__ __launch_bounds__(256) void rms_short_kernel(const T* x, T* res, cons
     const int c = j * 64 + lane;
     if (c < N) {
       if constexpr (FUSED) rr[c] = (T)v[j];
-      yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)wraw[j] : 1.0f));
+      if constexpr (UPFRONT) yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)wraw[j] : 1.0f));
+      else yr[c] = (T)(v[j] * rrms * (w != nullptr ? (float)w[c] : 1.0f));
     }
   }
 }

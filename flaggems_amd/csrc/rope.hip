@@ -55,9 +55,13 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
   const int h = r / pph;
   const int c = r - h * pph;
 
-  // the arguments of the second half of the kernel are fetched with the first ones, not behind the position load
-  asm volatile("" : : "s"(a.cos), "s"(a.sin), "s"(a.cos_stride), "s"(a.sin_stride), "s"(a.q), "s"(a.k), "s"(a.q_out), "s"(a.k_out));
-  asm volatile("" : : "s"(a.qs[0]), "s"(a.qs[1]), "s"(a.ks[0]), "s"(a.ks[1]), "s"(a.qos[0]), "s"(a.qos[1]), "s"(a.kos[0]), "s"(a.kos[1]));
+  // Variant FG_V_ROPE_ARGS (variants.h; off: arguments fetched where used, strides selected through a pointer).
+  constexpr bool ARGS_EARLY = FG_V_ROPE_ARGS != 0;
+  if constexpr (ARGS_EARLY) {
+    // the arguments of the second half of the kernel are fetched with the first ones, not behind the position load
+    asm volatile("" : : "s"(a.cos), "s"(a.sin), "s"(a.cos_stride), "s"(a.sin_stride), "s"(a.q), "s"(a.k), "s"(a.q_out), "s"(a.k_out));
+    asm volatile("" : : "s"(a.qs[0]), "s"(a.qs[1]), "s"(a.ks[0]), "s"(a.ks[1]), "s"(a.qos[0]), "s"(a.qos[1]), "s"(a.kos[0]), "s"(a.kos[1]));
+  }
   int64_t pos;
   if (a.pos == nullptr) {
     pos = tok % a.seq_len;
@@ -71,10 +75,15 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
 
   const bool is_q = h < a.Hq;
   const int hh = is_q ? h : h - a.Hq;
+#if FG_V_ROPE_ARGS
   // the strides are selected by value: selecting a pointer into the argument block makes them a vector load from
   // memory, a trip of its own in front of the row
   const int64_t is[3] = {is_q ? a.qs[0] : a.ks[0], is_q ? a.qs[1] : a.ks[1], is_q ? a.qs[2] : a.ks[2]};
   const int64_t os[3] = {is_q ? a.qos[0] : a.kos[0], is_q ? a.qos[1] : a.kos[1], is_q ? a.qos[2] : a.kos[2]};
+#else
+  const int64_t* is = is_q ? a.qs : a.ks;
+  const int64_t* os = is_q ? a.qos : a.kos;
+#endif
   const T* src = (const T*)(is_q ? a.q : a.k) + tok * is[0] + hh * is[1];
   T* dst = (T*)(is_q ? a.q_out : a.k_out) + tok * os[0] + hh * os[1];
 

@@ -54,24 +54,40 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void softmax_rows_kernel(con
   // All packs of the thread are requested before the first is used.  The loads are unconditional (a pack past the
   // end of the row or of the matrix is read from the start of the input and discarded): with a branch around each
   // load the compiler finishes pack j, wait included, before it requests pack j + 1, one trip to memory per pack.
+  // (variant FG_V_ROWS_UPFRONT, variants.h; off: every pack is loaded where it is used, under its bounds check)
+  constexpr bool UPFRONT = FG_V_ROWS_UPFRONT != 0;
   Pack<TI, VEC> px[ITERS];
+  if constexpr (UPFRONT) {
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int col = (j * TPR + t) * VEC;
-    px[j] = ld_pack_nt<TI, VEC>(row_ok && col < N ? xr + col : in);
+    for (int j = 0; j < ITERS; ++j) {
+      const int col = (j * TPR + t) * VEC;
+      px[j] = ld_pack_nt<TI, VEC>(row_ok && col < N ? xr + col : in);
+    }
+    // the output pointer is fetched with the other kernel arguments, not by a scalar load behind the last reduction
+    asm volatile("" : : "s"(out));
   }
-  // the output pointer is fetched with the other kernel arguments, not by a scalar load behind the last reduction
-  asm volatile("" : : "s"(out));
   float v[ITERS][VEC];
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int col = (j * TPR + t) * VEC;
-    const bool ok = row_ok && col < N;
+    if constexpr (UPFRONT) {
+      const bool ok = row_ok && col < N;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      v[j][e] = ok ? (float)px[j].v[e] : -INFINITY;
-      m = fmaxf(m, v[j][e]);
+      for (int e = 0; e < VEC; ++e) {
+        v[j][e] = ok ? (float)px[j].v[e] : -INFINITY;
+        m = fmaxf(m, v[j][e]);
+      }
+    } else if (row_ok && col < N) {
+      px[j] = ld_pack_nt<TI, VEC>(xr + col);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        v[j][e] = (float)px[j].v[e];
+        m = fmaxf(m, v[j][e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[j][e] = -INFINITY;
     }
   }
   // fmaxf drops NaN operands, but exp(NaN - m) below puts the NaN into the row sum, so a NaN
@@ -210,18 +226,23 @@ __global__ __launch_bounds__(256) void softmax_short_kernel(const TI* __restrict
   TO* yr = out + row * (int64_t)N;
   // unconditional loads (a column past the end reads the row's first element and is discarded): with a branch
   // around each the compiler waits for one before it requests the next, up to ITERS trips to memory per row
+  // (variant FG_V_SHORT_UPFRONT, variants.h; off: every element is loaded where it is used, under its bounds check)
+  constexpr bool UPFRONT = FG_V_SHORT_UPFRONT != 0;
   TI raw[ITERS];
+  if constexpr (UPFRONT) {
 #pragma unroll
-  for (int j = 0; j < ITERS; ++j) {
-    const int c = j * 64 + lane;
-    raw[j] = xr[c < N ? c : 0];
+    for (int j = 0; j < ITERS; ++j) {
+      const int c = j * 64 + lane;
+      raw[j] = xr[c < N ? c : 0];
+    }
   }
   float v[ITERS];
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < ITERS; ++j) {
     const int c = j * 64 + lane;
-    v[j] = c < N ? (float)raw[j] : -INFINITY;
+    if constexpr (UPFRONT) v[j] = c < N ? (float)raw[j] : -INFINITY;
+    else v[j] = c < N ? (float)xr[c] : -INFINITY;
     m = fmaxf(m, v[j]);
   }
   m = wave_max(m);

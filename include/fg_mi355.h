@@ -46,7 +46,9 @@ int fg_abi_version(void);
 void fg_reload_options(void);
 
 /* Device facts the host-side heuristics use (CU count stands in for the reference's
- * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530). */
+ * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530).
+ * Also performs the library's only per-device set-up (the address of fg_gemm_skinny_static's scratch array), so a
+ * caller that queries its devices at start-up may issue every later call under stream capture. */
 int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
 
 /* Calibration of the matrix-core roofline (no counterpart in the reference; used by bench.py):
@@ -219,7 +221,10 @@ int fg_gemm(const void* A, const void* B, const void* bias, void* C, int64_t M, 
  * Accepts what the skinny stream-K kernels accept: 16-bit inputs, M <= 64, K >= 1024, A with unit K stride and
  * 16-byte aligned rows, B row-major (M <= 16) or K-contiguous; anything else returns FG_ERR_UNSUPPORTED with a
  * message (use fg_gemm).  Results are bit-identical to fg_gemm's stream-K schedule.  All calls on one GPU share
- * the array: calls that overlap on one GPU (different streams) race; calls on one stream are safe. */
+ * the array: calls that overlap on one GPU (different streams) race; calls on one stream are safe.
+ * The array's device address is looked up on the first call on a device (or by fg_device_info for that device);
+ * the lookup cannot be made while the stream is being captured, so a first call that arrives under capture returns
+ * FG_ERR_UNSUPPORTED with a message instead of breaking the capture. */
 int fg_gemm_skinny_static(const void* A, const void* B, const void* bias, void* C, int64_t M, int64_t N,
                           int64_t K, int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t sim,
                           int64_t sin_, int64_t scm, int64_t scn, float alpha, float beta, int ab_dtype,
@@ -228,7 +233,12 @@ int fg_gemm_skinny_static(const void* A, const void* B, const void* bias, void* 
 /* C[b] = A[b] . B[b] for b in [0, batch), fp32 accumulate, every operand addressed through
  * (matrix, row, col) element strides (a matrix stride of 0 broadcasts one operand).  Matrix b is
  * one data-parallel fg_gemm launch; the launches follow each other on the stream.
+ * Verified envelope: at most FG_BMM_MAX_BATCH matrices and FG_BMM_MAX_OUT_ELEMS output elements per call; a call
+ * beyond it returns FG_ERR_UNSUPPORTED with a message and launches nothing (a larger batch once ended in a GPU
+ * memory fault whose cause is not known; callers split the batch or use the vendor library).
  * Replaces bmm_kernel (src/flag_gems/ops/bmm.py:15-136) and its C++ twin lib/bmm.cpp. */
+#define FG_BMM_MAX_BATCH 16
+#define FG_BMM_MAX_OUT_ELEMS (1LL << 24)
 int fg_bmm(const void* A, const void* B, void* C, int64_t batch, int64_t M, int64_t N, int64_t K,
            int64_t sab, int64_t sam, int64_t sak, int64_t sbb, int64_t sbk, int64_t sbn,
            int64_t scb, int64_t scm, int64_t scn, int dtype, void* stream);

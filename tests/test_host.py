@@ -135,12 +135,42 @@ def test_abi_validation_errors_without_gpu():
     rc = lib.fg_gemm(one, one, None, one, 4, 4, 0, 4, 1, 4, 1, 0, 0, 4, 1, 1.0, 0.0, _C.FG_F16, _C.FG_F16, _C.FG_F16,
                      0, None, 0, None, None)
     assert rc == -1 and "K must be positive" in _C.last_error()
+    # the entry point that allocates nothing turns away what its static scratch array cannot hold, before any launch
+    rc = lib.fg_gemm_skinny_static(one, one, None, one, 65, 512, 2048, 2048, 1, 1, 2048, 0, 0, 512, 1, 1.0, 0.0,
+                                   _C.FG_BF16, _C.FG_BF16, _C.FG_BF16, None)
+    assert rc == -2 and "exceed the maximum of 64" in _C.last_error()
+    rc = lib.fg_gemm_skinny_static(one, one, None, one, 8, 512, 2048, 2048, 1, 1, 2048, 0, 0, 512, 1, 1.0, 0.0,
+                                   _C.FG_F32, _C.FG_F32, _C.FG_F32, None)
+    assert rc == -2 and "16-bit inputs only" in _C.last_error()
     p = _C.FgFlashParams()
     p.dtype = _C.FG_F32
     assert lib.fg_flash_attn_varlen_fwd(ctypes.byref(p), None) == -1
     assert "fp16 and bf16" in _C.last_error()
     with pytest.raises(RuntimeError):
         _C.check(-1, "probe")
+
+
+def test_bmm_abi_refuses_batches_beyond_the_verified_envelope():
+    """fg_bmm itself, not only the Python wrapper, keeps callers inside the batch sizes its parity cases cover: the
+    refusal happens on the host, before any launch (the pointers here are never dereferenced)."""
+    import importlib
+
+    bmm_mod = importlib.import_module("flaggems_amd.ops.bmm")
+
+    lib = _C.lib()
+    one = ctypes.c_void_p(256)
+
+    def call(batch, M, N, K):
+        return lib.fg_bmm(one, one, one, batch, M, N, K, M * K, K, 1, K * N, N, 1, M * N, N, 1, _C.FG_BF16, None)
+
+    assert call(32, 2048, 2048, 128) == -2                      # FG_ERR_UNSUPPORTED: the batch that once faulted
+    assert "verified envelope" in _C.last_error()
+    assert call(17, 8, 8, 8) == -2                              # more than 16 matrices
+    assert call(16, 1024, 1025, 8) == -2                        # more than 2^24 output elements
+    assert call(0, 2048, 2048, 128) == 0 and call(64, 0, 8, 8) == 0   # empty: nothing to do, whatever the batch
+    header = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "fg_mi355.h")).read()
+    assert int(re.search(r"#define FG_BMM_MAX_BATCH (\d+)", header).group(1)) == bmm_mod._MAX_BATCH
+    assert 1 << int(re.search(r"#define FG_BMM_MAX_OUT_ELEMS \(1LL << (\d+)\)", header).group(1)) == bmm_mod._MAX_OUT_ELEMS
 
 
 def test_python_wrappers_assert_like_the_reference():

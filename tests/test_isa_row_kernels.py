@@ -1,19 +1,60 @@
-"""Shape of the memory traffic of the row kernels at the benchmark configurations, read from the device assembly that
-the library's build keeps (flaggems_amd/csrc/build/*.s): every load is requested before the first wait, and no kernel
-argument is fetched late.  A branch around a load, or a value first touched behind a reduction, silently turns one trip
-to memory per row into several; the results stay right, so only a look at the generated code shows it.
-Skipped when the build's assembly is not there (the tests may run against a prebuilt library)."""
+"""Shape of the memory traffic of the row kernels' "requests up front" variants at the benchmark configurations, read
+from their device assembly: every load is requested before the first wait, and no kernel argument is fetched late.
+A branch around a load, or a value first touched behind a reduction, silently turns one trip to memory per row into
+several; the results stay right, so only a look at the generated code shows it.
+
+The variants are switches of flaggems_amd/csrc/variants.h (off in the default build until they have passed the GPU
+parity suite), so this test compiles the five sources concerned to device assembly itself, with the switches on.
+Skipped when hipcc is not installed."""
 import importlib.util
 import os
 import re
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BUILD = os.path.join(ROOT, "flaggems_amd", "csrc", "build")
-_spec = importlib.util.spec_from_file_location("fg_isa_check", os.path.join(ROOT, "flaggems_amd", "csrc", "isa_check.py"))
+CSRC = os.path.join(ROOT, "flaggems_amd", "csrc")
+_spec = importlib.util.spec_from_file_location("fg_isa_check", os.path.join(CSRC, "isa_check.py"))
 isa_check = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(isa_check)
+_spec = importlib.util.spec_from_file_location("fg_build", os.path.join(CSRC, "build.py"))
+fg_build = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(fg_build)
+
+VARIANTS = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "RMS_BWD_ZERO_PACK": 1}
+SOURCES = ["norm", "softmax", "backward", "rope", "kvcache"]
+
+
+@pytest.fixture(scope="module")
+def variant_asm(tmp_path_factory):
+    """{source: device assembly text} of the five sources built with the variants on."""
+    if not os.path.exists(fg_build.HIPCC):
+        pytest.skip("no hipcc at %s" % fg_build.HIPCC)
+    out = tmp_path_factory.mktemp("variant_asm")
+    defines = fg_build.variant_defines(VARIANTS)
+
+    def one(src):
+        dst = os.path.join(str(out), src + ".s")
+        cmd = [fg_build.HIPCC] + fg_build.FLAGS + defines + ["-x", "hip", "--cuda-device-only", "-S",
+                                                            os.path.join(CSRC, src + ".hip"), "-o", dst]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        assert p.returncode == 0, p.stderr[-2000:]
+        with open(dst) as f:
+            return src, f.read()
+
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+        texts = dict(ex.map(one, SOURCES))
+    shutil.rmtree(str(out), ignore_errors=True)
+    for src, text in texts.items():
+        hits = isa_check.scan(text) + isa_check.scan_packed_f32(text) + [
+            (k, 0, first, "%d scratch accesses inside a loop" % n)
+            for k, n, first in isa_check.scan_scratch_in_loops(text, allowed={})]
+        assert not hits, (src, hits[:3])
+    return texts
+
 
 # (source, kernel instantiation, what it serves)
 CASES = [
@@ -31,19 +72,15 @@ CASES = [
 ]
 
 
-def _trace(source, kernel):
-    path = os.path.join(BUILD, "%s-hip-amdgcn-amd-amdhsa-gfx950.s" % source)
-    if not os.path.exists(path):
-        pytest.skip("no device assembly at %s (run flaggems_amd/csrc/build.py)" % path)
-    with open(path) as f:
-        lines = isa_check.memory_trace(f.read(), kernel)
+def _trace(asm, source, kernel):
+    lines = isa_check.memory_trace(asm[source], kernel)
     assert len(lines) == 1, (kernel, len(lines))
     return lines[0].split("\n")[1].strip().replace(".", "")
 
 
 @pytest.mark.parametrize("source,kernel,what", CASES)
-def test_every_request_goes_out_before_the_first_wait(source, kernel, what):
-    trace = _trace(source, kernel)
+def test_every_request_goes_out_before_the_first_wait(variant_asm, source, kernel, what):
+    trace = _trace(variant_asm, source, kernel)
     assert "k" not in trace, "%s: a kernel argument is fetched late: %s" % (what, trace)
     head = re.match(r"^[L|]+", trace).group(0)
     assert "L" not in trace[len(head):], "%s: a load is issued behind a wait: %s" % (what, trace)
@@ -62,8 +99,8 @@ def _groups(trace):
     return [len(g) for g in re.findall(r"L+", trace)]
 
 
-def test_rope_reads_position_then_everything_else_in_one_batch():
-    trace = _trace("rope", "rope_kernelIDF16bDF16bLi8ELb0")
+def test_rope_reads_position_then_everything_else_in_one_batch(variant_asm):
+    trace = _trace(variant_asm, "rope", "rope_kernelIDF16bDF16bLi8ELb0")
     first = trace.index("L")
     assert "k" not in trace[first:], trace            # every argument is fetched before the first load
     groups = _groups(trace)
@@ -71,7 +108,7 @@ def test_rope_reads_position_then_everything_else_in_one_batch():
     assert groups[-1] == 4 and sum(groups[:-1]) == 2, trace
 
 
-def test_cache_scatter_requests_the_row_with_the_slot():
-    trace = _trace("kvcache", "cache_scatter_kernelIDv4_jl")
+def test_cache_scatter_requests_the_row_with_the_slot(variant_asm):
+    trace = _trace(variant_asm, "kvcache", "cache_scatter_kernelIDv4_jl")
     assert "k" not in trace[trace.index("L"):], trace
     assert _groups(trace)[0] == 5, trace              # four pieces of the row and the slot, one wait for all

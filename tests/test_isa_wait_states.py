@@ -156,7 +156,6 @@ def _build_module():
 
 def test_the_build_refuses_an_object_whose_assembly_fails_the_scan(tmp_path, monkeypatch):
     build = _build_module()
-    monkeypatch.setattr(build, "OBJ_DIR", str(tmp_path))
     obj = tmp_path / "x.hip.o"
     asm = tmp_path / "x-hip-amdgcn-amd-amdhsa-gfx950.s"
     leftover = tmp_path / "x-hip-amdgcn-amd-amdhsa-gfx950.hipi"
@@ -165,18 +164,18 @@ def test_the_build_refuses_an_object_whose_assembly_fails_the_scan(tmp_path, mon
         f.write_text("")
     asm.write_text(kernel("\tv_readfirstlane_b32 s6, v36\n" + COPY))
     with pytest.raises(RuntimeError, match="fails 1 check"):
-        build._check_wait_states("x.hip", str(obj))
+        build._check_wait_states("x.hip", str(obj), str(tmp_path))
     assert not obj.exists() and other.exists()        # nothing stale left to link
     # a clean assembly: the object stays, the bulky intermediates go, the assembly is kept for inspection
     obj.write_text("")
     leftover.write_text("")
     asm.write_text(kernel("\tv_readfirstlane_b32 s6, v36\n\ts_nop 4\n" + COPY))
-    build._check_wait_states("x.hip", str(obj))
+    build._check_wait_states("x.hip", str(obj), str(tmp_path))
     assert obj.exists() and asm.exists() and not leftover.exists() and other.exists()
     # no assembly at all is an error too: the check must not be skipped silently
     asm.unlink()
     with pytest.raises(RuntimeError, match="no device assembly"):
-        build._check_wait_states("x.hip", str(obj))
+        build._check_wait_states("x.hip", str(obj), str(tmp_path))
 
 
 def test_expected_compiler_remarks_are_dropped_from_the_build_log():

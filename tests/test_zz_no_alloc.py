@@ -107,3 +107,55 @@ def test_static_scratch_gemm_rejects_what_it_cannot_hold(gpu):
     b32 = torch.randn(2048, 512, device=gpu)
     out = torch.empty(8, 512, device=gpu)
     assert _call("static", a32, b32, None, out, 1.0, 0.0) == -2
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import ctypes, os, sys
+import torch
+sys.path.insert(0, os.path.join(os.getcwd(), "tests"))
+import test_zz_no_alloc as T
+from flaggems_amd import _C
+
+lib = _C.lib()
+dev = torch.device("cuda:0")
+a, b, _ = T._problem(dev, 8, 4096, 4096, torch.bfloat16, True, 7, False)
+total, header = ctypes.c_size_t(0), ctypes.c_size_t(0)
+assert lib.fg_gemm_workspace_layout(0, ctypes.byref(total), ctypes.byref(header)) == 0
+ws = torch.zeros(total.value, dtype=torch.uint8, device=dev)
+want = torch.empty(8, 4096, dtype=torch.bfloat16, device=dev)
+assert T._call("workspace", a, b, None, want, 1.0, 0.0, ws) == 0
+out = torch.zeros_like(want)
+torch.cuda.synchronize()
+side = torch.cuda.Stream()
+g1 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g1, stream=side):
+    rc = T._call("static", a, b, None, out, 1.0, 0.0)       # the process's first call: refused, capture intact
+    msg = _C.last_error()
+assert rc == -2 and "under stream capture" in msg, (rc, msg)
+n = ctypes.c_int(0)
+assert lib.fg_device_info(0, ctypes.byref(n), None, None) == 0 and n.value > 0
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2, stream=side):
+    assert T._call("static", a, b, None, out, 1.0, 0.0) == 0, _C.last_error()
+for _ in range(2):
+    out.zero_()
+    torch.cuda.synchronize()
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+print("FIRST-CALL-UNDER-CAPTURE OK")
+"""
+
+
+def test_first_call_under_capture_is_refused_until_the_device_is_primed(gpu):
+    """In a fresh process: the entry point's first call on a device, made under stream capture, returns
+    FG_ERR_UNSUPPORTED and leaves the capture usable; after fg_device_info for that device the same call is recorded
+    and replays to fg_gemm's bits.  (A child process, because this process has long made its first call.)"""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-c", _FIRST_CALL_UNDER_CAPTURE], cwd=root, capture_output=True, text=True,
+                       timeout=300)
+    assert p.returncode == 0 and "FIRST-CALL-UNDER-CAPTURE OK" in p.stdout, (p.stdout[-2000:], p.stderr[-4000:])
