@@ -29,7 +29,8 @@ def get_higher_dtype(a, b):
 # later.  Only the header has to read zero when a launch starts, and the kernels return it to zero.  It is
 # cleared when the buffer is made and, once per graph capture that uses the buffer, by a fill kernel recorded
 # into that graph, so that every replay starts from a cleared header whichever graph of the stream ran (or was
-# only recorded) before it.
+# only recorded) before it.  A buffer whose first use falls inside a capture has only a recorded clear; its first
+# eager use clears it for real.
 _workspaces = {}
 _layouts = {}
 _capture_id = ctypes.c_ulonglong(0)
@@ -50,10 +51,17 @@ def _workspace(device, stream):
             layout = _layouts[device.index] = (total.value, header.value)
         buf = torch.empty(layout[0], dtype=torch.uint8, device=device)
         buf[:layout[1]].zero_()
-        entry = _workspaces[key] = [buf, capture, layout[1]]
+        # entry: buffer, capture id last seen, header bytes, whether a clear has ever RUN (one issued under capture
+        # is only recorded into that graph)
+        entry = _workspaces[key] = [buf, capture, layout[1], capture == 0]
     elif capture != entry[1]:
         if capture != 0:
             entry[0][:entry[2]].zero_()
+        elif not entry[3]:
+            # the buffer was made under capture and this is its first eager use: no clear has run yet unless that
+            # graph was replayed, so the header may hold whatever the allocation held
+            entry[0][:entry[2]].zero_()
+            entry[3] = True
         entry[1] = capture
     return entry[0]
 

@@ -282,3 +282,45 @@ def test_custom_op_namespace_schemas():
     # a CPU tensor finds no kernel: the namespace is served on the CUDA key only, as in the reference
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.flag_gems.mm(torch.ones(2, 2), torch.ones(2, 2))
+
+
+def test_gemm_workspace_made_under_capture_is_cleared_on_first_eager_use(monkeypatch):
+    """Bookkeeping of the cached stream-K scratch buffer (flaggems_amd/ops/_gemm.py), with a stand-in library that
+    reports capture ids: a buffer first made while its stream is being captured has had its clear only recorded, so
+    the first eager use clears the header itself; later eager uses do not touch it; a new capture records a clear."""
+    from flaggems_amd.ops import _gemm
+
+    state = {"capture": 7}
+
+    class Lib:
+        def fg_stream_capture_id(self, stream, out):
+            out._obj.value = state["capture"]
+            return 0
+
+        def fg_gemm_workspace_layout(self, dev, total, header):
+            total._obj.value, header._obj.value = 4096, 256
+            return 0
+
+    monkeypatch.setattr(_C, "lib", lambda: Lib())
+    monkeypatch.setattr(_gemm, "_workspaces", {})
+    monkeypatch.setattr(_gemm, "_layouts", {})
+    dev = torch.device("cpu")
+    buf = _gemm._workspace(dev, 123)                  # made "under capture 7"
+    entry = _gemm._workspaces[(dev.index, 123)]
+    assert entry[1] == 7 and entry[3] is False
+    buf.fill_(0xFF)                                   # the recorded clear never ran
+    assert _gemm._workspace(dev, 123) is buf and (buf[:256] == 0xFF).all()   # same capture: nothing new recorded
+    state["capture"] = 0
+    assert _gemm._workspace(dev, 123) is buf
+    assert (buf[:256] == 0).all() and (buf[256:] == 0xFF).all() and entry[3] is True
+    buf[:256].fill_(5)                                # kernels own the header between eager calls
+    assert _gemm._workspace(dev, 123) is buf and (buf[:256] == 5).all()
+    state["capture"] = 9                              # a new capture on the stream records its own clear
+    _gemm._workspace(dev, 123)
+    assert (buf[:256] == 0).all() and entry[1] == 9
+    state["capture"] = 0
+    buf[:256].fill_(5)
+    _gemm._workspace(dev, 123)                        # back to eager: already cleared once for real, left alone
+    assert (buf[:256] == 5).all()
+    buf2 = _gemm._workspace(dev, 456)                 # a buffer made eagerly is cleared on the spot
+    assert (buf2[:256] == 0).all() and _gemm._workspaces[(dev.index, 456)][3] is True
