@@ -136,7 +136,8 @@ def main():
         return ts[len(ts) // 2]
 
     # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs scaled by what the
-    # same counters read for a plain 512 MiB copy (profiles/hbm_traffic_*.txt hold the runs and their commands)
+    # same counters read for a plain 512 MiB copy (profiles/hbm_traffic_all_configs.txt holds the runs and their
+    # commands); measured on the kernels the default build ships (tests/golden/device_code_manifest.txt pins them)
     TRAFFIC = {
         "softmax_c2": 1073780000,
         "fused_add_rms_norm_c1": 134340000,
@@ -173,8 +174,6 @@ def main():
         def cpu():
             O.softmax(sample, -1)
 
-        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
-        # read for a plain 512 MiB copy (profiles/hbm_traffic_softmax_mm_attention.txt)
         return dict(run=run, work=2 * M * N * 2, bound="hbm", dtype="bf16", traffic=TRAFFIC.get("softmax_c2"),
                     workload="softmax dim=-1 [131072,2048] bf16, N(0,4) with 1% -inf (BASELINE.json configs[1])",
                     cpu=(cpu, 2 * 32768 * N * 2, "oracle softmax (torch CPU, fp64 upcast) on the first 32768 rows"))

@@ -13,7 +13,8 @@
  *     thread-local message of the last failure.  No C++ exception crosses this boundary.
  *
  * Each declaration cites the reference interface it stands in for (paths are relative to
- * the FlagGems source tree).
+ * the FlagGems source tree).  The operator entry points come first; a "Diagnostics" section at the
+ * end holds the few host-side hooks of the library's own tests and benchmark.
  */
 #ifndef FG_MI355_H
 #define FG_MI355_H
@@ -41,22 +42,11 @@ const char* fg_last_error(void);
 /* ABI version of this header (bumped on any signature change). */
 int fg_abi_version(void);
 
-/* Re-reads the FG_* measurement and test switches from the environment.  The library reads them once, on first
- * use; no entry point consults the environment per call.  No counterpart in the reference. */
-void fg_reload_options(void);
-
 /* Device facts the host-side heuristics use (CU count stands in for the reference's
  * multi_processor_count: src/flag_gems/ops/mm.py:24, src/flag_gems/ops/flash_api.py:524-530).
  * Also performs the library's only per-device set-up (the address of fg_gemm_skinny_static's scratch array), so a
  * caller that queries its devices at start-up may issue every later call under stream capture. */
 int fg_device_info(int device, int* num_cu, int* lds_bytes, int* gcn_arch);
-
-/* Calibration of the matrix-core roofline (no counterpart in the reference; used by bench.py):
- * every wave of `blocks` 256-thread workgroups issues 64 * iters MFMA 16x16x32 bf16 on operand
- * fragments read once from `operands` (8 * 256 * 16 bytes).  `out` receives blocks * 256 floats;
- * *flops the floating-point operations of the launch.  The sustained rate depends on the operand
- * bits (power): random operands give the ceiling a real bf16 GEMM can approach on this part. */
-int fg_mfma_probe(const void* operands, float* out, int blocks, int iters, double* flops, void* stream);
 
 /* rms_norm forward.  y[m,:] = x[m,:] * rsqrt(mean(x[m,:]^2) + eps) * w, fp32 arithmetic,
  * one rounding on store; inv_rms[m] (fp32) is written when non-NULL; w may be NULL (= ones).
@@ -177,26 +167,6 @@ size_t fg_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int ab_dtype, in
  * src/flag_gems/ops/mm_streamk.py:488-491. */
 int fg_gemm_workspace_layout(int device, size_t* max_bytes /*host*/, size_t* header_bytes /*host*/);
 
-/* What fg_gemm's automatic schedule selects for 16-bit operands that qualify for the direct-to-LDS kernels (16-byte
- * aligned rows, unit stride along K or N, K a multiple of 64) on a device of `num_cu` compute units (<= 0: the
- * current device's): the workgroup tile of the data-parallel launch with its modelled duration in microseconds, and
- * the number of workgroups and modelled duration of the stream-K launch on 128x128 tiles (*streamk_workers = 0 when
- * the problem does not qualify for it: more tiles than CUs or fewer than four K steps per CU).  *streamk_chosen tells
- * which of the two the automatic schedule takes when a workspace is given.  Host arithmetic only when num_cu > 0: no
- * device is touched.  Any output pointer may be NULL.
- * Stands in for the tuned-configuration lookup of src/flag_gems/ops/mm.py:54-62 and the schedule test
- * streamk_scenario, src/flag_gems/ops/mm.py:186-197. */
-int fg_gemm_plan(int64_t M, int64_t N, int64_t K, int num_cu, int* tile_m /*host*/, int* tile_n /*host*/,
-                 double* dp_us /*host*/, int* streamk_workers /*host*/, double* streamk_us /*host*/,
-                 int* streamk_chosen /*host*/);
-
-/* The order in which a data-parallel launch of tiles_m x tiles_n workgroup tiles walks its grid: workgroup id i
- * computes tile (tile_m[i], tile_n[i]); both arrays hold tiles_m * tiles_n entries.  Workgroup i runs on XCD i mod 8,
- * so the order decides which A and B panels share an L2.  b_k_contiguous selects the variant used for B = W^T
- * (non-zero) or row-major B.  Host arithmetic only; the kernels call the same function.
- * Stands in for the grouped ordering of mm_kernel_general, src/flag_gems/ops/mm.py:83-91 (GROUP_M grouping of the program ids). */
-int fg_gemm_tile_order(int tiles_m, int tiles_n, int b_k_contiguous, int* tile_m /*host*/, int* tile_n /*host*/);
-
 /* *id = 0 when `stream` is not capturing into a HIP graph, otherwise a non-zero number unique to the capture in
  * progress.  Host code uses it to record one clearing of the workspace header per captured graph.  No counterpart
  * in the reference (its Triton launches allocate and clear per call). */
@@ -296,6 +266,45 @@ int fg_flash_attn_varlen_fwd(const FgFlashParams* p /*host*/, void* stream);
  * src/flag_gems/ops/flash_api.py:752-800).  The forward never needs it: without it (NULL or too
  * small) it runs unsplit.  Uninitialised memory is fine; one stream at a time. */
 size_t fg_flash_attn_workspace_bytes(const FgFlashParams* p /*host*/, int device);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Diagnostics.  Not part of the operator interface: nothing above depends on a caller using them, and a binder of
+ * the operators can leave them out.  They exist for the library's own tests and benchmark: host-side views of
+ * decisions the kernels and launchers make (so that those can be checked without a GPU), the matrix-core
+ * calibration loop, and the re-reading of the FG_* switches.  None has a counterpart in the reference's operator
+ * interface; where a comment names reference code, it is the logic the reported decision stands in for.
+ * ------------------------------------------------------------------------------------------------------------ */
+
+/* Re-reads the FG_* measurement and test switches from the environment.  The library reads them once, on first
+ * use; no entry point consults the environment per call.  No counterpart in the reference. */
+void fg_reload_options(void);
+
+/* Calibration of the matrix-core roofline (no counterpart in the reference; used by bench.py):
+ * every wave of `blocks` 256-thread workgroups issues 64 * iters MFMA 16x16x32 bf16 on operand
+ * fragments read once from `operands` (8 * 256 * 16 bytes).  `out` receives blocks * 256 floats;
+ * *flops the floating-point operations of the launch.  The sustained rate depends on the operand
+ * bits (power): random operands give the ceiling a real bf16 GEMM can approach on this part. */
+int fg_mfma_probe(const void* operands, float* out, int blocks, int iters, double* flops, void* stream);
+
+/* What fg_gemm's automatic schedule selects for 16-bit operands that qualify for the direct-to-LDS kernels (16-byte
+ * aligned rows, unit stride along K or N, K a multiple of 64) on a device of `num_cu` compute units (<= 0: the
+ * current device's): the workgroup tile of the data-parallel launch with its modelled duration in microseconds, and
+ * the number of workgroups and modelled duration of the stream-K launch on 128x128 tiles (*streamk_workers = 0 when
+ * the problem does not qualify for it: more tiles than CUs or fewer than four K steps per CU).  *streamk_chosen tells
+ * which of the two the automatic schedule takes when a workspace is given.  Host arithmetic only when num_cu > 0: no
+ * device is touched.  Any output pointer may be NULL.
+ * Stands in for the tuned-configuration lookup of src/flag_gems/ops/mm.py:54-62 and the schedule test
+ * streamk_scenario, src/flag_gems/ops/mm.py:186-197. */
+int fg_gemm_plan(int64_t M, int64_t N, int64_t K, int num_cu, int* tile_m /*host*/, int* tile_n /*host*/,
+                 double* dp_us /*host*/, int* streamk_workers /*host*/, double* streamk_us /*host*/,
+                 int* streamk_chosen /*host*/);
+
+/* The order in which a data-parallel launch of tiles_m x tiles_n workgroup tiles walks its grid: workgroup id i
+ * computes tile (tile_m[i], tile_n[i]); both arrays hold tiles_m * tiles_n entries.  Workgroup i runs on XCD i mod 8,
+ * so the order decides which A and B panels share an L2.  b_k_contiguous selects the variant used for B = W^T
+ * (non-zero) or row-major B.  Host arithmetic only; the kernels call the same function.
+ * Stands in for the grouped ordering of mm_kernel_general, src/flag_gems/ops/mm.py:83-91 (GROUP_M grouping of the program ids). */
+int fg_gemm_tile_order(int tiles_m, int tiles_n, int b_k_contiguous, int* tile_m /*host*/, int* tile_n /*host*/);
 
 #ifdef __cplusplus
 }
