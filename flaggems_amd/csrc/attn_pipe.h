@@ -216,6 +216,18 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   f32x4 minit[QT];          // -m of the lane's row, four times: C operand of the first MFMA of a score tile
   f32x4 o_acc[QT][NPV];
   float m_run[QT], l_run[QT];
+  // Variant FG_V_ATTN_ROWSUM_MFMA (variants.h): the row sums come from the matrix pipe.  One more MFMA per column
+  // tile and half-tile step multiplies a fragment of ones with P^T, exactly the B operand of the PV products: every
+  // element of its 16 x 16 result in column q is the sum over the 32 keys of P[key][q], so each lane holds the WHOLE
+  // row sum of its column (four times), summed from the P values as rounded for the PV product.  It replaces sixteen
+  // vector additions per step, on a kernel whose vector ALU is as busy as its matrix pipe.
+  // Head dim 128 only: at head dim 64 the eight extra accumulator registers take the kernel from three waves per
+  // SIMD to two.
+  constexpr bool ROWSUM_MFMA = FG_V_ATTN_ROWSUM_MFMA != 0 && D == 128;
+  f32x4 l_acc[ROWSUM_MFMA ? QT : 1];
+  Frag ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = (T)1.0f;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     minit[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -223,6 +235,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     for (int dt = 0; dt < NPV; ++dt) o_acc[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     m_run[qt] = -INFINITY;
     l_run[qt] = 0.f;   // the lane's share of the row sum
+    if constexpr (ROWSUM_MFMA) l_acc[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
   // ---- DMA geometry: one page id per wave and tile, kept in two registers ------------------------------
@@ -348,7 +361,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
     if constexpr (QK) {
       a_static_for<0, RING>([&](auto ic) { read_k(ic, sk_c, AInt<NXT>{}); });
     }
-    if constexpr (EXP) {
+    if constexpr (EXP && !ROWSUM_MFMA) {
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt) psum[qt] = 0.f;
     }
@@ -384,8 +397,10 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
             const float p1 = __builtin_amdgcn_exp2f(s_buf[CUR][t2][qt][2 * w + 1]);
             typedef T T2 __attribute__((ext_vector_type(2)));
             const T2 pk = {(T)p0, (T)p1};
-            psum[qt] += p0 + p1;
-            asm volatile("" : "+v"(psum[qt]));  // (keeps the addition in this slot: left free it sinks behind phase B)
+            if constexpr (!ROWSUM_MFMA) {
+              psum[qt] += p0 + p1;
+              asm volatile("" : "+v"(psum[qt]));  // (keeps the addition in this slot: left free it sinks behind phase B)
+            }
             u32x4 words = __builtin_bit_cast(u32x4, pf[qt]);
             words[t2 * 2 + w] = __builtin_bit_cast(uint32_t, pk);
             pf[qt] = __builtin_bit_cast(Frag, words);
@@ -394,7 +409,7 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (EXP) {
+    if constexpr (EXP && !ROWSUM_MFMA) {
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt) l_run[qt] += psum[qt];
     }
@@ -421,6 +436,10 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
         o_acc[qt][i] = AttnMfma<T>::mma16(__builtin_bit_cast(Frag, both), pf[qt], o_acc[qt][i]);
         if constexpr (qt == QT - 1 && i + RING < NPV) read_v(AInt<i + RING>{}, sv_c, cur_c);
       });
+      if constexpr (ROWSUM_MFMA && i < QT) {
+        // slot i carries the row-sum product of column tile i: the first two slots of the phase hold no vector work
+        l_acc[i < QT ? i : 0] = AttnMfma<T>::mma16(ones, pf[i < QT ? i : 0], l_acc[i < QT ? i : 0]);
+      }
       if constexpr (MAX && i >= 2) {
         // the 8 score pairs over the slots from the third on
         constexpr int per = (8 + NPV - 3) / (NPV - 2);
@@ -500,7 +519,12 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
       for (int dt = 0; dt < NPV; ++dt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) o_acc[qt][dt][r] *= alpha;
-      l_run[qt] *= alpha;
+      if constexpr (ROWSUM_MFMA) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) l_acc[qt][r] *= alpha;
+      } else {
+        l_run[qt] *= alpha;
+      }
       if (moved) m_run[qt] = (fresh ? 0.f : m_run[qt]) + delta;
       const float mm = m_run[qt] == -INFINITY ? 0.f : -m_run[qt];
       minit[qt] = f32x4{mm, mm, mm, mm};
@@ -572,7 +596,9 @@ __global__ __launch_bounds__(256, 2) void attn_varlen_pipe_kernel(AttnArgs a) {
   // ---- epilogue: lane (g, c) holds O^T[16 dt + 4 g + r][q = 16 QT + c] ---------------------------------
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    const float l_row = xquad_sum(l_run[qt]);
+    float l_row;
+    if constexpr (ROWSUM_MFMA) l_row = l_acc[qt][0];   // already the sum over all keys of the row
+    else l_row = xquad_sum(l_run[qt]);
     const int qrow = row0 + qt * 16 + c;
     if (qrow >= q_len) continue;
     const bool empty = l_row == 0.f || l_row != l_row;

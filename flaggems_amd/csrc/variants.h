@@ -38,6 +38,13 @@
 #define FG_V_ATTN_Q_UNCOND 0
 #endif
 
+// attn_varlen_pipe_kernel: the softmax row sums are taken by one extra MFMA per column tile and half-tile step (a
+// fragment of ones times P^T) instead of sixteen vector additions per step; the normaliser then sums P as rounded for
+// the PV product.  Tested code: lane-local fp32 sums on the vector ALU, added across lane groups in the epilogue.
+#ifndef FG_V_ATTN_ROWSUM_MFMA
+#define FG_V_ATTN_ROWSUM_MFMA 0
+#endif
+
 // attn_decode_kernel: Q requested together with the page ids, in front of the one wait before the first tile copies.
 // Tested code: Q loaded at the top of the kernel under the row check.
 #ifndef FG_V_DECODE_Q_EARLY
