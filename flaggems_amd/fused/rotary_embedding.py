@@ -57,8 +57,10 @@ def apply_rotary_pos_emb(
         position_ids = position_ids.reshape(-1)
         seq_len = 0
 
-    q = q.view(-1, q.shape[-2], q.shape[-1])
-    k = k.view(-1, k.shape[-2], k.shape[-1])
+    flat = len(q_shape) == 3  # already (tokens, heads, head_dim), what a serving engine passes: no views to make
+    if not flat:
+        q = q.view(-1, q.shape[-2], q.shape[-1])
+        k = k.view(-1, k.shape[-2], k.shape[-1])
     n_tokens, q_heads, head_dim = q.shape
     k_heads = k.shape[1]
 
@@ -70,17 +72,20 @@ def apply_rotary_pos_emb(
 
     if n_tokens > 0 and head_dim > 0:
         I3 = _C.I64x3
+        qs, ks = I3(*q.stride()), I3(*k.stride())
         with _C.device_guard(q.device):
             rc = _C.lib().fg_rope(
                 q_embed.data_ptr(), k_embed.data_ptr(), q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                 position_ids.data_ptr() if position_ids is not None else None,
                 1 if (position_ids is not None and position_ids.dtype == torch.int64) else 0,
                 n_tokens, seq_len, q_heads, k_heads, head_dim,
-                I3(*q.stride()), I3(*k.stride()), I3(*q_embed.stride()), I3(*k_embed.stride()),
+                qs, ks, qs if inplace else I3(*q_embed.stride()), ks if inplace else I3(*k_embed.stride()),
                 position_ids.stride(0) if position_ids is not None else 0,
                 cos.stride(0) if cos.ndim > 1 else 0, sin.stride(0) if sin.ndim > 1 else 0, cos.shape[0],
                 1 if rotary_interleaved else 0, _C.dtype_id(q.dtype), _C.dtype_id(cos.dtype),
                 _C.current_stream(q.device),
             )
         _C.check(rc, "fg_rope")
+    if flat:
+        return q_embed, k_embed
     return q_embed.view(q_shape), k_embed.view(k_shape)

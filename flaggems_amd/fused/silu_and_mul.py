@@ -11,6 +11,12 @@ logger = logging.getLogger("flag_gems.fused.silu_and_mul")
 def _rows_view(t):
     """(rows, cols, row_stride) when t is a stack of unit-stride rows with one uniform row stride
     (contiguous tensors, and the halves of a gate-up projection, qualify); otherwise None."""
+    if t.ndim == 2:  # the usual case, spelled out: one stride() call instead of a walk over the dims
+        row_stride, col_stride = t.stride()
+        rows, cols = t.shape
+        if (col_stride == 1 or cols == 1) and row_stride >= cols:
+            return rows, cols, row_stride
+        return None
     if t.ndim == 0:
         return 1, 1, 1
     if t.stride(-1) != 1 and t.shape[-1] != 1:

@@ -67,11 +67,17 @@ def _workspace(device, stream):
 
 
 _last_schedule = ctypes.c_int(0)
+_last_schedule_ref = ctypes.byref(_last_schedule)
 
 
 def last_schedule():
     """Schedule the most recent gemm call on this process used (1 data-parallel, 2 stream-K)."""
     return _last_schedule.value
+
+
+# fg_gemm_workspace_bytes is a pure function of its arguments (shape, dtype, schedule and the device's CU count):
+# its answers are kept, so that a decode-size call pays for one transition into the library, not two.
+_ws_need = {}
 
 
 def gemm(a, b, bias, c, alpha=1.0, beta=0.0, schedule=_C.SCHED_AUTO):
@@ -83,18 +89,28 @@ def gemm(a, b, bias, c, alpha=1.0, beta=0.0, schedule=_C.SCHED_AUTO):
     with _C.device_guard(dev):
         stream = _C.current_stream(dev)
         ab = _C.dtype_id(a.dtype)
-        ws_bytes = lib.fg_gemm_workspace_bytes(M, N, K, ab, schedule, dev.index)
-        ws = _workspace(dev, stream) if ws_bytes else None
+        key = (M, N, K, ab, schedule, dev.index)
+        ws_bytes = _ws_need.get(key)
+        if ws_bytes is None:
+            if len(_ws_need) > 4096:
+                _ws_need.clear()
+            ws_bytes = _ws_need[key] = lib.fg_gemm_workspace_bytes(M, N, K, ab, schedule, dev.index)
+        if ws_bytes:
+            ws = _workspace(dev, stream)
+            wptr, wlen = ws.data_ptr(), ws.numel()
+        else:
+            wptr, wlen = None, 0
         if bias is not None:
-            bptr, sim, sin_, bdt = bias.data_ptr(), bias.stride(0), bias.stride(1), _C.dtype_id(bias.dtype)
+            (sim, sin_), bptr, bdt = bias.stride(), bias.data_ptr(), _C.dtype_id(bias.dtype)
         else:
             bptr, sim, sin_, bdt = None, 0, 0, ab
+        sam, sak = a.stride()
+        sbk, sbn = b.stride()
+        scm, scn = c.stride()
         rc = lib.fg_gemm(
-            a.data_ptr(), b.data_ptr(), bptr, c.data_ptr(), M, N, K,
-            a.stride(0), a.stride(1), b.stride(0), b.stride(1), sim, sin_, c.stride(0), c.stride(1),
-            alpha, beta, ab, _C.dtype_id(c.dtype), bdt, schedule,
-            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            ctypes.byref(_last_schedule), stream,
+            a.data_ptr(), b.data_ptr(), bptr, c.data_ptr(), M, N, K, sam, sak, sbk, sbn, sim, sin_, scm, scn,
+            alpha, beta, ab, _C.dtype_id(c.dtype), bdt, schedule, wptr, wlen, _last_schedule_ref, stream,
         )
-    _C.check(rc, "fg_gemm")
+    if rc != 0:
+        _C.check(rc, "fg_gemm")
     return c

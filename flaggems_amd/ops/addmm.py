@@ -47,11 +47,12 @@ def _vendor_addmm(bias, mat1, mat2, beta, alpha, out=None):
 def _run(bias, mat1, mat2, beta, alpha, out):
     M, K = mat1.shape
     N = mat2.shape[1]
-    logger.debug(
-        "GEMS ADDMM, [shape info]: [-, %s, %s, %s](batch, M, N, K), "
-        "[A column-major]: %s, [B column-major]: %s, [bias column-major]: %s",
-        M, N, K, mat1.stride(0) == 1, mat2.stride(0) == 1, bias.stride(0) == 1 if bias.dim() else True,
-    )
+    if logger.isEnabledFor(logging.DEBUG):
+        logger.debug(
+            "GEMS ADDMM, [shape info]: [-, %s, %s, %s](batch, M, N, K), "
+            "[A column-major]: %s, [B column-major]: %s, [bias column-major]: %s",
+            M, N, K, mat1.stride(0) == 1, mat2.stride(0) == 1, bias.stride(0) == 1 if bias.dim() else True,
+        )
     if M == 0 or N == 0:
         return out
     mat1 = mat1.contiguous()

@@ -19,6 +19,21 @@ def maybe_contiguous(x):
     return x.contiguous() if x is not None and x.stride(-1) != 1 else x
 
 
+# The reference's forward returns three tensors that only dropout gives a meaning (philox state, an unused slot, the
+# attention probabilities).  Dropout is not part of this path, so they are placeholders: made once per device and
+# handed out again, instead of three allocations on every call.
+_placeholders = {}
+
+
+def _dropout_placeholders(device):
+    hit = _placeholders.get(device)
+    if hit is None:
+        hit = _placeholders[device] = (torch.empty((2,), dtype=torch.int64, device=device),
+                                       torch.empty((), dtype=torch.int64, device=device),
+                                       torch.empty((), device=device))
+    return hit
+
+
 def mha_varlan_fwd(
     q, k, v, out, cu_seqlens_q, cu_seqlens_k, seqused_k, leftpad_k, page_table, alibi_slopes,
     max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal,
@@ -100,10 +115,10 @@ def mha_varlan_fwd(
             p.seqused_k = seqused_k.data_ptr()
             p.block_table = page_table.data_ptr()
             p.alibi_slopes = alibi_slopes.data_ptr() if alibi_slopes is not None else None
-            p.q_row_stride, p.q_head_stride = q.stride(0), q.stride(1)
-            p.o_row_stride, p.o_head_stride = out.stride(0), out.stride(1)
-            p.k_page_stride, p.k_row_stride, p.k_head_stride = k.stride(0), k.stride(1), k.stride(2)
-            p.v_page_stride, p.v_row_stride, p.v_head_stride = v.stride(0), v.stride(1), v.stride(2)
+            p.q_row_stride, p.q_head_stride, _ = q.stride()
+            p.o_row_stride, p.o_head_stride, _ = out.stride()
+            p.k_page_stride, p.k_row_stride, p.k_head_stride, _ = k.stride()
+            p.v_page_stride, p.v_row_stride, p.v_head_stride, _ = v.stride()
             p.block_table_stride = page_table.stride(0)
             p.alibi_batch_stride = alibi_batch_stride
             p.total_q = total_q
@@ -122,9 +137,7 @@ def mha_varlan_fwd(
                 p.workspace, p.workspace_bytes = ws.data_ptr(), ws_bytes
             rc = _C.lib().fg_flash_attn_varlen_fwd(ctypes.byref(p), _C.current_stream(q.device))
             _C.check(rc, "fg_flash_attn_varlen_fwd")
-        philox_args = torch.empty((2,), dtype=torch.int64, device=q.device)
-        unused = torch.empty((), dtype=torch.int64, device=q.device)
-        probs = torch.empty((), device=q.device)
+        philox_args, unused, probs = _dropout_placeholders(q.device)
     return out, q, k, v, lse, philox_args, unused, probs
 
 
@@ -180,8 +193,7 @@ def flash_attn_varlen_func(
     else:
         assert len(window_size) == 2
         real_window_size = (window_size[0], window_size[1])
-    q, k, v = [maybe_contiguous(x) for x in (q, k, v)]
-    dummy_cu_seqlens_k = torch.empty_like(cu_seqlens_q)
+    q, k, v = maybe_contiguous(q), maybe_contiguous(k), maybe_contiguous(v)
     if fa_version != 2:
         raise RuntimeError("Only FA2 is implemented.")
     if num_splits > 0:
@@ -190,7 +202,9 @@ def flash_attn_varlen_func(
     max_seqlen_k = max_seqlen_k.item() if hasattr(max_seqlen_k, "item") else max_seqlen_k
     out, q, k, v, softmax_lse, *_ = mha_varlan_fwd(
         q, k, v, out, cu_seqlens_q,
-        dummy_cu_seqlens_k if cu_seqlens_k is None else cu_seqlens_k,
+        # (the reference passes an uninitialised tensor shaped like cu_seqlens_q here; only its shape and dtype are
+        # looked at, so cu_seqlens_q itself serves without an allocation)
+        cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k,
         seqused_k, None, block_table, alibi_slopes, max_seqlen_q, max_seqlen_k, dropout_p,
         softmax_scale, False, causal, real_window_size[0], real_window_size[1], softcap,
         return_softmax_lse and dropout_p > 0, None,

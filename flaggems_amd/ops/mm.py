@@ -11,11 +11,15 @@ logger = logging.getLogger("flag_gems.ops.mm")
 
 def _prepare(a, b):
     # same contiguity rule as the reference: copy only when both strides exceed one
-    if a.stride(0) > 1 and a.stride(1) > 1:
+    sa0, sa1 = a.stride()
+    sb0, sb1 = b.stride()
+    if sa0 > 1 and sa1 > 1:
         a = a.contiguous()
-    if b.stride(0) > 1 and b.stride(1) > 1:
+    if sb0 > 1 and sb1 > 1:
         b = b.contiguous()
     assert a.shape[1] == b.shape[0], "incompatible dimensions"
+    if sa1 == 1:
+        return a, b  # A is contiguous along K already (the usual case): nothing below applies
     # A column-major A (the X^T of a weight gradient) misses the direct-to-LDS and skinny kernels, which want
     # A contiguous along K; one transposing copy of A (the library's own kernel) costs far less than the
     # slower main loop once the output is 256 columns wide, or 64 when A has few rows.  Measured, bf16:
@@ -55,10 +59,11 @@ def _vendor_mm(a, b, out=None):
 def _run(a, b, c):
     M, K = a.shape
     N = b.shape[1]
-    logger.debug(
-        "GEMS MM, [shape info]: [-, %s, %s, %s](batch, M, N, K), [A column-major]: %s, [B column-major]: %s",
-        M, N, K, a.stride(0) == 1, b.stride(0) == 1,
-    )
+    if logger.isEnabledFor(logging.DEBUG):
+        logger.debug(
+            "GEMS MM, [shape info]: [-, %s, %s, %s](batch, M, N, K), [A column-major]: %s, [B column-major]: %s",
+            M, N, K, a.stride(0) == 1, b.stride(0) == 1,
+        )
     if M == 0 or N == 0:
         return c
     if K == 0:

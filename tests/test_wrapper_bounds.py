@@ -441,3 +441,35 @@ def test_the_checks_notice_a_wrong_stride_a_long_row_and_a_foreign_pointer(hx):
     lib.fg_rms_norm(x.data_ptr() + 2, None, y.data_ptr(), None, 8, 64, 64, 64, 1e-5, _C.FG_BF16, 0)   # not a data_ptr()
     with pytest.raises(AssertionError, match="did not come from"):
         hx.check_all()
+
+
+def test_repeated_calls_take_the_short_host_path(hx):
+    """Decode-size calls are host-bound unless the wrapper stays short: the workspace query of a GEMM shape is asked
+    of the library once, attention hands out its dropout placeholders instead of allocating them, and rotary
+    embedding on (tokens, heads, dim) tensors in place returns its arguments without making views."""
+    from flaggems_amd.ops import _gemm
+
+    _gemm._ws_need.clear()
+    a, w = _r(8, 256), _r(64, 256)
+    for _ in range(3):
+        flag_gems.mm(a, w.t())
+    flag_gems.mm(_r(9, 256), w.t())
+    names = [n for n, _ in hx.rec.calls]
+    assert names.count("fg_gemm") == 4 and names.count("fg_gemm_workspace_bytes") == 2
+    _gemm._ws_need.clear()
+
+    q1, kc, vc, cu1, sk1, bt1, _, mk1 = _paged_case([(1, 70), (1, 3)], 8, 2, 64, 16, 16)
+    from flaggems_amd.ops.attention import mha_varlan_fwd
+
+    r1 = mha_varlan_fwd(q1, kc, vc, None, cu1, cu1, sk1, None, bt1, None, 1, mk1, 0.0, 0.125, False, True, -1, -1, 0.0, False, None)
+    r2 = mha_varlan_fwd(q1, kc, vc, None, cu1, cu1, sk1, None, bt1, None, 1, mk1, 0.0, 0.125, False, True, -1, -1, 0.0, False, None)
+    assert all(x is y for x, y in zip(r1[5:], r2[5:])) and r1[0] is not r2[0] and r1[4] is not r2[4]
+
+    q, k = _r(5, 8, 64), _r(5, 2, 64)
+    cos, sin = _r(16, 32, dtype=torch.float32), _r(16, 32, dtype=torch.float32)
+    pos = torch.arange(5)
+    qo, ko = flag_gems.apply_rotary_pos_emb(q, k, cos, sin, pos, False, inplace=True)
+    assert qo is q and ko is k
+    qo, ko = flag_gems.apply_rotary_pos_emb(q, k, cos, sin, pos, False)
+    assert qo.shape == q.shape and qo.data_ptr() != q.data_ptr()
+    hx.check_all()
