@@ -267,6 +267,33 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kernel(SkinnyArgs a) {
 // Wide outputs (N >= 8192) take 32-column tiles on a ring of 4 slots instead: the same bytes in flight, but
 // every A fragment (which all workgroups fetch from L2 at the same time) feeds two column blocks, and a
 // workgroup restarts its pipeline half as often.
+#if FG_V_SKINNY_ASM_A
+// Variant FG_V_SKINNY_ASM_A (variants.h).  The A fragments of gemm_skinny_kc_kernel are loaded into a ring of
+// registers RING - 1 steps ahead of their use, so a register written in one trip of the main loop is read in the next.
+// The compiler places the waits for the loads it emits, and across the loop's back edge it waits for EVERY operation
+// in flight (s_waitcnt vmcnt(0) in front of the first use of a trip): once per RING steps the wave has nothing on
+// its way.  Here the loads are written as asm, which the compiler does not count, and the wait that makes a slot's
+// registers valid is the counted one the copies into LDS already use.  The wait names the slot's registers as
+// operands, so no use of them can be scheduled in front of it; the build's scan of the device assembly
+// (isa_check.py, scan_vmem_loads) follows the VM counter through the loop and fails on any instruction that touches
+// a register whose load may still be outstanding.
+__device__ __forceinline__ void kc_load_a(u32x4& dst, const char* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+template <int N, int NAL> __device__ __forceinline__ void kc_wait_vm_pin(u32x4 (&r)[NAL]) {
+  static_assert(NAL == 2 || NAL == 4 || NAL == 8, "two loads per 16-row block");
+  if constexpr (NAL == 2) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(r[0]), "+v"(r[1]) : "n"(N) : "memory");
+  } else if constexpr (NAL == 4) {
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(N) : "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
+                 : "n"(N) : "memory");
+  }
+}
+#endif
+
 constexpr int kcStepK = 64;
 constexpr int kcLdsBytes = kWaves * 8 * 16 * kcStepK * 2;  // 128 KB: 8 slots of 16 rows, or 4 slots of 32 rows, per wave
 
@@ -379,8 +406,16 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
           constexpr int i = decltype(ic)::value;
           __builtin_amdgcn_global_load_lds(FGK_GLBP(bsrc[i] + koff), FGK_LDSP(slot), 16, i * 1024, 0);
         });
+#if FG_V_SKINNY_ASM_A
+        if constexpr (A_LINES) {
 #pragma unroll
-        for (int j = 0; j < NAL; ++j) af[p][j] = *reinterpret_cast<const u32x4*>(asrc[j] + koff);
+          for (int j = 0; j < NAL; ++j) kc_load_a(af[p][j], asrc[j] + koff);
+        } else
+#endif
+        {
+#pragma unroll
+          for (int j = 0; j < NAL; ++j) af[p][j] = *reinterpret_cast<const u32x4*>(asrc[j] + koff);
+        }
       };
       auto compute = [&](auto pc) {
         constexpr int p = decltype(pc)::value;
@@ -423,7 +458,11 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
         static_for<0, RING>([&](auto pc) {
           constexpr int p = decltype(pc)::value;
           issue(i + p + RING - 1, IntC<(p + RING - 1) % RING>{});
-          FGK_WAIT_VM(OPS * (RING - 1));
+#if FG_V_SKINNY_ASM_A
+          if constexpr (A_LINES) kc_wait_vm_pin<OPS * (RING - 1)>(af[p]);
+          else
+#endif
+            FGK_WAIT_VM(OPS * (RING - 1));
           compute(pc);
           __builtin_amdgcn_sched_barrier(0);
         });
@@ -432,6 +471,9 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_kc_kernel(SkinnyArgs a) {
       FGK_WAIT_VM(0);
       const int rest = nmine - i;
       static_for<0, RING - 1>([&](auto pc) {
+#if FG_V_SKINNY_ASM_A
+        if constexpr (A_LINES) kc_wait_vm_pin<0>(af[decltype(pc)::value]);  // (names the registers: no use moves above it)
+#endif
         if (decltype(pc)::value < rest) compute(pc);
       });
     }

@@ -238,6 +238,95 @@ def scan_lds_reads(text):
     return hits
 
 
+# ---- vector-memory loads against the VM counter ------------------------------------------------------------------
+# The same question for vector-memory loads whose wait the compiler did not place: a global_load written as asm hands
+# the compiler a destination register that it believes valid at once, and the s_waitcnt vmcnt(N) that really makes it
+# so is counted by hand.  gfx9 has one counter for loads, stores and LDS-direct loads; operations of one kind return in
+# order, so after vmcnt(N) everything but the N youngest has returned.  State: destination sets of the outstanding
+# operations, oldest first (an empty set for stores, LDS-direct loads and atomics without return).  Any instruction
+# that reads or writes a register whose load may still be outstanding is reported, except a later load into the same
+# register (loads return in order).  Compiler-placed waits satisfy this by construction, which makes every kernel of
+# the library a known-answer case for the scan.
+_VMEM_PREFIX = ("global_", "buffer_", "flat_", "scratch_")
+
+
+def _vm_wait_count(ops):
+    text = " ".join(ops)
+    m = re.search(r"vmcnt\((\d+)\)", text)
+    if m is not None:
+        return int(m.group(1))
+    if "cnt(" in text:
+        return None  # names other counters only
+    m2 = re.match(r"^(0x[0-9a-fA-F]+|\d+)$", text.strip())
+    if m2 is None:
+        return None
+    imm = int(m2.group(1), 0)
+    return (imm & 0xF) | (((imm >> 14) & 0x3) << 4)  # bits 3:0 and 15:14 hold the VM counter on gfx9
+
+
+def _vm_step(state, op, ops, line, report):
+    """state: {vgpr: fewest operations known to be younger than the outstanding load into it}.  A load is complete
+    once vmcnt(N) has been waited for with N <= that number; where paths join, the smaller number is kept."""
+    if op == "s_waitcnt":
+        n = _vm_wait_count(ops)
+        if n is None or not state:
+            return state
+        return {r: c for r, c in state.items() if c < n}
+    is_vmem = op.startswith(_VMEM_PREFIX)
+    if not state and not is_vmem:
+        return state
+    is_load = is_vmem and "_load" in op and "_lds" not in op and "lds" not in [o.split()[-1] for o in ops if o]
+    returns = is_load or (is_vmem and "atomic" in op and any(o.split()[-1] in ("glc", "sc0") for o in ops if o))
+    dst = _vgprs(ops[0].split()[0]) if returns and ops else frozenset()
+    if state:
+        used = frozenset().union(*[_vgprs(o.split()[0]) for o in ops if o]) if ops else frozenset()
+        srcs = frozenset().union(*[_vgprs(o.split()[0]) for o in ops[1:] if o]) if returns and len(ops) > 1 else used
+        # (a later load into a register with a load outstanding is no hazard by itself: loads return in order)
+        hit = [r for r in (srcs if is_load else used) if r in state]
+        if hit:
+            report(line, "touches v%s while the vector-memory load into it may be outstanding" % sorted(hit))
+    if is_vmem:
+        state = {r: c + 1 for r, c in state.items() if c + 1 < 63}  # six-bit counter: 63 younger ones mean it is back
+        for r in dst:
+            state[r] = 0
+    return state
+
+
+def scan_vmem_loads(text, only=None):
+    """Uses of a register before the vector-memory load that writes it is known to have returned:
+    (kernel, line, reason).  `only`: scan kernels whose name contains this string."""
+    hits = []
+    for km in _KERNEL.finditer(text):
+        kernel, blocks = km.group(1), _blocks(km.group(2))
+        if only is not None and only not in kernel:
+            continue
+        succ = _successors(blocks)
+        entry = [None] * len(blocks)   # state at block entry (None: not reached yet)
+        entry[0] = {}
+        work = [0]
+        found = set()
+        while work:
+            b = work.pop()
+            state = dict(entry[b])
+            for op, ops, line in blocks[b][1]:
+                state = _vm_step(state, op, ops, line, lambda l, why: found.add((l, why)))
+            for nb in succ[b]:
+                old = entry[nb]
+                if old is None:
+                    entry[nb] = dict(state)
+                    work.append(nb)
+                    continue
+                changed = False
+                for r, c in state.items():
+                    if r not in old or c < old[r]:
+                        old[r] = c
+                        changed = True
+                if changed:
+                    work.append(nb)
+        hits += [(kernel, l, why) for l, why in sorted(found)]
+    return hits
+
+
 # Packed fp32 arithmetic is switched off for this library (a compiler flag removes the feature, and no source writes
 # the instructions by hand); this confirms it on what was actually generated.
 _PACKED_F32 = ("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32")
@@ -345,7 +434,8 @@ def scan_scratch_in_loops(text, allowed=SCRATCH_IN_LOOP_ALLOWED):
 def check_file(path):
     with open(path) as f:
         text = f.read()
-    return (scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] + scan_packed_f32(text) +
+    return (scan(text) + [(k, 0, line, why) for k, line, why in scan_lds_reads(text)] +
+            [(k, 0, line, why) for k, line, why in scan_vmem_loads(text)] + scan_packed_f32(text) +
             [(k, 0, first, "%d scratch accesses inside a loop: registers spill there" % n)
              for k, n, first in scan_scratch_in_loops(text)])
 

@@ -141,6 +141,87 @@ __global__ __launch_bounds__(TPR < 256 ? 256 : TPR) void rms_rows_kernel(
   }
 }
 
+#if FG_V_RMS_TWO_ROWS
+// Variant FG_V_RMS_TWO_ROWS (variants.h): rows of one 16-byte pack per thread on 256 to 1024 threads, two rows per
+// workgroup.  A matrix of a few thousand rows is a handful of rounds of workgroups on this part (a CU holds 2048
+// threads: [4096, 4096] bf16 at 512 threads a row is four rounds), and every round pays its start and its drain.  Two
+// rows per workgroup halve the rounds; both rows' packs and the weight pack are requested before anything is
+// used, so a thread has four requests in flight instead of two, and the two row sums share one LDS exchange (two
+// barriers per workgroup instead of two per row).  Arithmetic and rounding are those of rms_rows_kernel.
+template <typename T, int VEC, int TPR, bool FUSED>
+__global__ __launch_bounds__(TPR) void rms_rows2_kernel(const T* x, T* res, const T* __restrict__ w, T* y,
+                                                       float* __restrict__ inv_rms, int64_t M, int N, int64_t xs,
+                                                       int64_t rs, int64_t ys, float eps) {
+  static_assert(TPR >= 256 && TPR % 64 == 0 && sizeof(T) * VEC == 16, "one 16-byte pack per thread, whole waves");
+  constexpr int WPR = TPR / 64;
+  __shared__ float smem[2][WPR];
+  const int t = threadIdx.x;
+  const int64_t row0 = (int64_t)blockIdx.x * 2;
+  const int col = t * VEC;
+  const bool col_ok = col < N;
+  bool ok[2];
+  Pack<T, VEC> px[2], pr[FUSED ? 2 : 1];
+  const T* wp = w != nullptr ? w : x;  // no weight: any readable address, the value is not used
+  const u32x4 wraw = *reinterpret_cast<const u32x4*>(wp + (col_ok ? col : 0));
+  asm volatile("" : : "s"(eps), "s"(y), "s"(ys), "s"(inv_rms));  // the tail's arguments are fetched with the others
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    ok[r] = row0 + r < M && col_ok;
+    // unconditional loads: a pack past the end of the row or of the matrix is read from the start of x and discarded
+    px[r] = ld_pack_nt<T, VEC>(ok[r] ? x + (row0 + r) * xs + col : x);
+    if constexpr (FUSED) pr[r] = ld_pack_nt<T, VEC>(ok[r] ? res + (row0 + r) * rs + col : x);
+  }
+  float v[2][VEC], ss[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    ss[r] = 0.f;
+    if constexpr (FUSED) {
+      Pack<T, VEC> po;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        v[r][e] = ok[r] ? (float)px[r].v[e] + (float)pr[r].v[e] : 0.f;
+        po.v[e] = (T)v[r][e];
+      }
+      if (ok[r]) st_pack_nt<T, VEC>(res + (row0 + r) * rs + col, po);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[r][e] = ok[r] ? (float)px[r].v[e] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ss[r] += v[r][e] * v[r][e];
+    ss[r] = wave_sum(ss[r]);
+  }
+  // (a row's sum is added up over its waves in wave order, as row_sum does)
+  if ((t & 63) == 0) {
+    smem[0][t >> 6] = ss[0];
+    smem[1][t >> 6] = ss[1];
+  }
+  __syncthreads();
+  Pack<T, VEC> pw = *reinterpret_cast<const Pack<T, VEC>*>(&wraw);
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) s += smem[r][i];
+    const float rrms = 1.0f / sqrtf(s / (float)N + eps);
+    if (row0 + r >= M) continue;
+    if constexpr (!FUSED) {
+      if (inv_rms != nullptr && t == 0) inv_rms[row0 + r] = rrms;
+    }
+    if (!col_ok) continue;
+    Pack<T, VEC> po;
+    if (w != nullptr) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) po.v[e] = (T)(v[r][e] * rrms * (float)pw.v[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) po.v[e] = (T)(v[r][e] * rrms);
+    }
+    st_pack_nt<T, VEC>(y + (row0 + r) * ys + col, po);
+  }
+}
+#endif
+
 // Any N, any alignment: one 256-thread block per row, element-wise coalesced access, two passes.
 // Short rows that defeat 16-byte access (N <= 512): one wave per row, element j * 64 + lane in register j.
 template <typename T, bool FUSED, int ITERS>
@@ -298,6 +379,16 @@ __global__ __launch_bounds__(BLOCK) void rms_looped_kernel(const T* x, T* res,
 template <typename T, int VEC, int ITERS, int TPR, bool FUSED>
 void launch_rows(const T* x, T* res, const T* w, T* y, float* inv_rms, int64_t M, int N, int64_t xs, int64_t rs,
                  int64_t ys, float eps, hipStream_t st) {
+#if FG_V_RMS_TWO_ROWS
+  if constexpr (ITERS == 1 && TPR >= 256) {
+    // matrices of up to a few rounds of workgroups: beyond that the rounds overlap and one row per workgroup is as good
+    if (M >= 2 && M <= 32768) {
+      hipLaunchKernelGGL((rms_rows2_kernel<T, VEC, TPR, FUSED>), dim3((unsigned)fg_cdiv(M, 2)), dim3(TPR), 0, st, x, res,
+                         w, y, inv_rms, M, N, xs, rs, ys, eps);
+      return;
+    }
+  }
+#endif
   constexpr int BLOCK = TPR < 256 ? 256 : TPR;
   constexpr int RPB = BLOCK / TPR;
   const int64_t grid = fg_cdiv(M, RPB);

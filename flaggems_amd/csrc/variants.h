@@ -14,6 +14,13 @@
 #define FG_V_ROWS_UPFRONT 0
 #endif
 
+// rms_norm / fused_add_rms_norm, rows of one pack per thread on 256-1024 threads, up to 32768 rows: two rows per
+// workgroup (rms_rows2_kernel), all requests of both rows up front, one LDS exchange for both row sums.  Halves the
+// rounds of workgroups of a small matrix ([4096, 4096]: four rounds -> two).  Tested code: one row per workgroup.
+#ifndef FG_V_RMS_TWO_ROWS
+#define FG_V_RMS_TWO_ROWS 0
+#endif
+
 // rms_short_kernel, softmax_short_kernel, bwd_short_kernel (one wave per short or unaligned row): elements loaded
 // unconditionally from clamped columns before the first use.  Tested code: each element under its own bounds check.
 #ifndef FG_V_SHORT_UPFRONT
@@ -55,6 +62,13 @@
 // keeps the two-pack variant (rows of 8193-16384 elements) out of scratch memory.  Tested code: zeroed element by element.
 #ifndef FG_V_RMS_BWD_ZERO_PACK
 #define FG_V_RMS_BWD_ZERO_PACK 0
+#endif
+
+// gemm_skinny_kc_kernel with more than 8 rows of A: the A fragments are loaded by asm and made valid by the counted
+// wait the LDS copies already use, instead of compiler-placed waits, which drain everything in flight once per trip of
+// the main loop (every RING steps).  Tested code: plain loads, compiler-placed waits.
+#ifndef FG_V_SKINNY_ASM_A
+#define FG_V_SKINNY_ASM_A 0
 #endif
 
 // dma_tile_epilogue: the broadcast-bias case of addmm takes a branch of its own.

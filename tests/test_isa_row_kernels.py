@@ -24,8 +24,9 @@ _spec = importlib.util.spec_from_file_location("fg_build", os.path.join(CSRC, "b
 fg_build = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(fg_build)
 
-VARIANTS = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "RMS_BWD_ZERO_PACK": 1}
-SOURCES = ["norm", "softmax", "backward", "rope", "kvcache"]
+VARIANTS = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "RMS_BWD_ZERO_PACK": 1,
+            "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1}
+SOURCES = ["norm", "softmax", "backward", "rope", "kvcache", "gemm_skinny"]
 
 
 @pytest.fixture(scope="module")
@@ -49,7 +50,7 @@ def variant_asm(tmp_path_factory):
         texts = dict(ex.map(one, SOURCES))
     shutil.rmtree(str(out), ignore_errors=True)
     for src, text in texts.items():
-        hits = isa_check.scan(text) + isa_check.scan_packed_f32(text) + [
+        hits = isa_check.scan(text) + isa_check.scan_packed_f32(text) + isa_check.scan_vmem_loads(text) + [
             (k, 0, first, "%d scratch accesses inside a loop" % n)
             for k, n, first in isa_check.scan_scratch_in_loops(text, allowed={})]
         assert not hits, (src, hits[:3])
@@ -63,6 +64,8 @@ CASES = [
     ("norm", "rms_rows_kernelIDF16bLi8ELi1ELi512ELb1", "fused_add_rms_norm [4096, 4096] bf16"),
     ("norm", "rms_rows_kernelIfLi4ELi2ELi512ELb1", "fused_add_rms_norm [4096, 4096] fp32"),
     ("norm", "rms_rows_kernelIDF16bLi8ELi1ELi512ELb0", "rms_norm [16384, 4096] bf16"),
+    ("norm", "rms_rows2_kernelIDF16bLi8ELi512ELb1", "fused_add_rms_norm [4096, 4096] bf16, two rows per workgroup"),
+    ("norm", "rms_rows2_kernelIfLi4ELi1024ELb1", "fused_add_rms_norm [4096, 4096] fp32, two rows per workgroup"),
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi1ELi256ELi0", "softmax backward [131072, 2048] bf16"),
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi4ELi1024ELi0", "softmax backward, four packs a thread"),
     ("backward", "bwd_rows_kernelIDF16bDF16bLi8ELi2ELi1024ELi1", "log_softmax backward, two packs a thread"),
@@ -85,6 +88,23 @@ def test_every_request_goes_out_before_the_first_wait(variant_asm, source, kerne
     head = re.match(r"^[L|]+", trace).group(0)
     assert "L" not in trace[len(head):], "%s: a load is issued behind a wait: %s" % (what, trace)
     assert trace.count("L") >= 1 and trace.rstrip("|").endswith("S"), trace
+
+
+def test_skinny_gemm_with_asm_loads_never_drains_the_ring(variant_asm):
+    """FG_V_SKINNY_ASM_A: the main loop of the K-contiguous skinny GEMM for more than eight rows holds counted waits
+    only (the build of the default code waits for everything in flight once per trip), and the VM-counter scan, which
+    the fixture has already run over the whole file, finds every register valid where it is used."""
+    text = variant_asm["gemm_skinny"]
+    for dtype in ("DF16b", "DF16_"):
+        km = [k for k in isa_check._KERNEL.finditer(text) if "gemm_skinny_kc_kernelI%sLi16ELi8ELb1ELi1E" % dtype in k.group(1)]
+        assert len(km) == 1
+        blocks = isa_check._blocks(km[0].group(2))
+        loop = isa_check._blocks_in_loops(isa_check._successors(blocks))
+        main = max(loop, key=lambda b: sum(1 for op, _, _ in blocks[b][1] if op.startswith("v_mfma")))
+        waits = [isa_check._vm_wait_count(ops) for op, ops, _ in blocks[main][1] if op == "s_waitcnt"]
+        waits = [w for w in waits if w is not None]
+        assert waits == [28] * 8, waits   # eight steps a trip, each leaving the 7 x 4 younger operations in flight
+    assert isa_check.scan_lds_reads(text) == []
 
 
 def test_the_trace_reads_a_known_kernel():

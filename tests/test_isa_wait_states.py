@@ -211,3 +211,49 @@ def test_scratch_accesses_are_reported_inside_loops_only():
     assert len(isa_check.scan_scratch_in_loops(nested)) == 1
     # allowed by name
     assert isa_check.scan_scratch_in_loops(loop, allowed={"k0": "test"}) == []
+
+
+# ---- vector-memory loads against the VM counter (scan_vmem_loads) ------------------------------------------------
+LOAD = "\tglobal_load_dwordx4 v[8:11], v[20:21], off"
+STORE = "\tglobal_store_dwordx4 v[20:21], v[30:33], off"
+
+
+@pytest.mark.parametrize("younger,wait,expect", [(0, 0, 0), (2, 2, 0), (2, 3, 1), (2, 1, 0), (5, 63, 1)])
+def test_a_vm_wait_retires_all_but_the_youngest(younger, wait, expect):
+    """A load, `younger` stores behind it, a wait for all but `wait` operations, then a use of the loaded register."""
+    body = LOAD + "\n" + (STORE + "\n") * younger + "\ts_waitcnt vmcnt(%d)\n\tv_add_u32_e32 v1, v8, v3" % wait
+    assert len(isa_check.scan_vmem_loads(kernel(body))) == expect
+
+
+def test_a_use_without_any_wait_and_an_overwrite_are_reported():
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\tv_mov_b32_e32 v40, v11"))) == 1
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\tv_mov_b32_e32 v9, v40"))) == 1    # written under the load
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\tv_mov_b32_e32 v20, v40"))) == 0   # the address is free at once
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\tds_bpermute_b32 v50, v51, v10"))) == 1
+
+
+def test_loads_return_in_order_lds_direct_loads_and_stores_count():
+    again = "\tglobal_load_dwordx4 v[8:11], v[22:23], off"
+    assert isa_check.scan_vmem_loads(kernel(LOAD + "\n" + again + "\n\ts_waitcnt vmcnt(0)\n\tv_mov_b32_e32 v1, v8")) == []
+    body = LOAD + "\n" + COPY + "\n" + STORE + "\n\ts_waitcnt vmcnt(2)\n\tv_mov_b32_e32 v1, v8"
+    assert isa_check.scan_vmem_loads(kernel(body)) == []
+    body = LOAD + "\n" + COPY + "\n" + STORE + "\n\ts_waitcnt vmcnt(3)\n\tv_mov_b32_e32 v1, v8"
+    assert len(isa_check.scan_vmem_loads(kernel(body))) == 1
+    # a wait that names only the LDS counter retires nothing here; a bare immediate carries the count in bits 3:0, 15:14
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\ts_waitcnt lgkmcnt(0)\n\tv_mov_b32_e32 v1, v8"))) == 1
+    assert isa_check.scan_vmem_loads(kernel(LOAD + "\n\ts_waitcnt 0x0f70\n\tv_mov_b32_e32 v1, v8")) == []
+    assert len(isa_check.scan_vmem_loads(kernel(LOAD + "\n\ts_waitcnt 0x0f71\n\tv_mov_b32_e32 v1, v8"))) == 1
+
+
+def test_the_vm_counter_is_followed_around_a_loop_and_through_both_arms():
+    # a ring of two registers: the load of one trip is used in the next, behind a wait that leaves one load in flight
+    ring = ("\tglobal_load_dwordx4 v[8:11], v[20:21], off\n.LBB0_1:\n\tglobal_load_dwordx4 v[12:15], v[20:21], off\n"
+            "\ts_waitcnt vmcnt(%d)\n\tv_mov_b32_e32 v1, v8\n\tglobal_load_dwordx4 v[8:11], v[20:21], off\n"
+            "\ts_waitcnt vmcnt(%d)\n\tv_mov_b32_e32 v1, v12\n\ts_cbranch_scc1 .LBB0_1")
+    assert isa_check.scan_vmem_loads(kernel(ring % (1, 1))) == []
+    assert len(isa_check.scan_vmem_loads(kernel(ring % (2, 1)))) == 1
+    assert len(isa_check.scan_vmem_loads(kernel(ring % (1, 2)))) == 1
+    arms = (LOAD + "\n\ts_cbranch_scc1 .LBB0_2\n\ts_waitcnt vmcnt(0)\n\ts_branch .LBB0_3\n.LBB0_2:\n" + STORE +
+            "\n.LBB0_3:\n\tv_mov_b32_e32 v1, v8")
+    assert len(isa_check.scan_vmem_loads(kernel(arms))) == 1        # one arm does not wait
+    assert isa_check.scan_vmem_loads(kernel(arms.replace(STORE, "\ts_waitcnt vmcnt(0)"))) == []
