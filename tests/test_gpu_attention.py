@@ -59,34 +59,6 @@ def test_flash_attn_varlen_reference_grid(gpu, dtype, Hq, Hk, D, num_blocks, ali
     check(gpu, [(1, 1328), (5, 18), (129, 463)], Hq, Hk, D, 32, num_blocks, dtype, alibi=alibi, softcap=softcap)
 
 
-# The reference's single-token grid as it stands (tests/test_attention_ops.py:998-1085,
-# test_flash_attn_varlen_func_swap_qg: every sequence has one query token, so the reference takes its "swap query
-# groups and sequence" path, ops/flash_api.py:318-345): lengths [(1, 1328), (1, 18), (1, 463)], 8 query heads on 2 KV
-# heads, head dim 128, pages of 32, 2048 pages, soft cap off and 10.0, both 16-bit types, causal, seed 1234567890.
-@pytest.mark.parametrize("seq_lens", [[(1, 1328), (1, 18), (1, 463)]])
-@pytest.mark.parametrize("num_heads", [(8, 2)])
-@pytest.mark.parametrize("head_size", [128])
-@pytest.mark.parametrize("block_size", [32])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("soft_cap", [None, 10.0])
-@pytest.mark.parametrize("num_blocks", [2048])
-def test_flash_attn_varlen_func_swap_qg(gpu, seq_lens, num_heads, head_size, block_size, dtype, soft_cap, num_blocks):
-    q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, seq_lens, num_heads[0], num_heads[1], head_size, block_size,
-                                                    num_blocks, dtype)
-    scale = head_size ** -0.5
-    out = flag_gems.ops.flash_attn_varlen_func(
-        q=q, k=kc, v=vc, cu_seqlens_q=cu, seqused_k=sk, max_seqlen_q=max(qlens), max_seqlen_k=max(klens),
-        softmax_scale=scale, causal=True, window_size=(-1, -1), block_table=bt,
-        softcap=soft_cap if soft_cap is not None else 0, fa_version=2,
-    )
-    assert out.shape == q.shape and out.dtype == dtype
-    # the reference compares in the tensors' own dtype: its oracle rounds the probabilities to the value dtype
-    ref = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, soft_cap=soft_cap)
-    torch.testing.assert_close(out.cpu(), ref.to(dtype), atol=ATOL, rtol=RTOL)
-    ref32 = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, soft_cap=soft_cap, compute_dtype=torch.float32)
-    torch.testing.assert_close(out.float().cpu(), ref32, atol=ATOL, rtol=RTOL)
-
-
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("Hq,Hk", [(6, 2), (3, 1), (32, 8)])
 @pytest.mark.parametrize("D", [32, 48, 64, 72, 80, 96, 112, 120])

@@ -168,37 +168,3 @@ def test_two_graphs_on_one_stream_replayed_out_of_order(gpu):
             g.replay()
             torch.cuda.synchronize()
         assert torch.equal(got1, want1) and torch.equal(got2, want2)
-
-
-def test_workspace_made_under_capture_then_used_eagerly(gpu):
-    """The workspace of a stream is first made during a capture, so its clearing is only recorded; the next call on
-    that stream is eager and comes before any replay.  It must not start from whatever the allocation held."""
-    from flaggems_amd.ops import _gemm
-
-    a1, w1 = _sk_inputs(gpu, 16, 1024, 4096, 5)
-    a2, w2 = _sk_inputs(gpu, 384, 4096, 4096, 6)
-    want1 = _streamk_mm(a1, w1.t())
-    want2 = _streamk_mm(a2, w2.t())
-    torch.cuda.synchronize()
-    side = _fresh_stream(gpu)
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        got1 = _streamk_mm(a1, w1.t())
-    entry = _gemm._workspaces[(gpu.index, side.cuda_stream)]
-    assert entry[3] is False          # no clear of this buffer has run yet
-    entry[0][:entry[2]].fill_(0xFF)   # what stale memory would look like to the ticket counters
-    torch.cuda.synchronize()
-    with torch.cuda.stream(side):
-        eager = _streamk_mm(a2, w2.t())
-    torch.cuda.synchronize()
-    assert entry[3] is True
-    assert torch.equal(eager, want2)
-    for _ in range(2):
-        got1.zero_()
-        graph.replay()
-        torch.cuda.synchronize()
-        assert torch.equal(got1, want1)
-        with torch.cuda.stream(side):
-            again = _streamk_mm(a2, w2.t())
-        torch.cuda.synchronize()
-        assert torch.equal(again, want2)

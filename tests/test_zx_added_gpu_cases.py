@@ -1,0 +1,74 @@
+"""GPU cases added after the last complete run of the GPU suite.  They collect behind the long-standing parity tests
+(pytest takes files in alphabetical order) so that a problem in a case that has never run cannot hide, under `-x`, the
+result of the ones that have; the tests of the entry point that allocates nothing still come last."""
+import pytest
+import torch
+
+import flag_gems
+from oracle import torch_ref as O
+from test_gpu_attention import ATOL, RTOL, make_case
+from test_gpu_zgraph import _fresh_stream, _sk_inputs, _streamk_mm
+
+pytestmark = pytest.mark.gpu
+
+
+# The reference's single-token grid as it stands (tests/test_attention_ops.py:998-1085,
+# test_flash_attn_varlen_func_swap_qg: every sequence has one query token, so the reference takes its "swap query
+# groups and sequence" path, ops/flash_api.py:318-345): lengths [(1, 1328), (1, 18), (1, 463)], 8 query heads on 2 KV
+# heads, head dim 128, pages of 32, 2048 pages, soft cap off and 10.0, both 16-bit types, causal, seed 1234567890.
+@pytest.mark.parametrize("seq_lens", [[(1, 1328), (1, 18), (1, 463)]])
+@pytest.mark.parametrize("num_heads", [(8, 2)])
+@pytest.mark.parametrize("head_size", [128])
+@pytest.mark.parametrize("block_size", [32])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("soft_cap", [None, 10.0])
+@pytest.mark.parametrize("num_blocks", [2048])
+def test_flash_attn_varlen_func_swap_qg(gpu, seq_lens, num_heads, head_size, block_size, dtype, soft_cap, num_blocks):
+    q, kc, vc, cu, sk, bt, qlens, klens = make_case(gpu, seq_lens, num_heads[0], num_heads[1], head_size, block_size,
+                                                    num_blocks, dtype)
+    scale = head_size ** -0.5
+    out = flag_gems.ops.flash_attn_varlen_func(
+        q=q, k=kc, v=vc, cu_seqlens_q=cu, seqused_k=sk, max_seqlen_q=max(qlens), max_seqlen_k=max(klens),
+        softmax_scale=scale, causal=True, window_size=(-1, -1), block_table=bt,
+        softcap=soft_cap if soft_cap is not None else 0, fa_version=2,
+    )
+    assert out.shape == q.shape and out.dtype == dtype
+    # the reference compares in the tensors' own dtype: its oracle rounds the probabilities to the value dtype
+    ref = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, soft_cap=soft_cap)
+    torch.testing.assert_close(out.cpu(), ref.to(dtype), atol=ATOL, rtol=RTOL)
+    ref32 = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, soft_cap=soft_cap, compute_dtype=torch.float32)
+    torch.testing.assert_close(out.float().cpu(), ref32, atol=ATOL, rtol=RTOL)
+
+
+def test_workspace_made_under_capture_then_used_eagerly(gpu):
+    """The workspace of a stream is first made during a capture, so its clearing is only recorded; the next call on
+    that stream is eager and comes before any replay.  It must not start from whatever the allocation held."""
+    from flaggems_amd.ops import _gemm
+
+    a1, w1 = _sk_inputs(gpu, 16, 1024, 4096, 5)
+    a2, w2 = _sk_inputs(gpu, 384, 4096, 4096, 6)
+    want1 = _streamk_mm(a1, w1.t())
+    want2 = _streamk_mm(a2, w2.t())
+    torch.cuda.synchronize()
+    side = _fresh_stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        got1 = _streamk_mm(a1, w1.t())
+    entry = _gemm._workspaces[(gpu.index, side.cuda_stream)]
+    assert entry[3] is False          # no clear of this buffer has run yet
+    entry[0][:entry[2]].fill_(0xFF)   # what stale memory would look like to the ticket counters
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        eager = _streamk_mm(a2, w2.t())
+    torch.cuda.synchronize()
+    assert entry[3] is True
+    assert torch.equal(eager, want2)
+    for _ in range(2):
+        got1.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got1, want1)
+        with torch.cuda.stream(side):
+            again = _streamk_mm(a2, w2.t())
+        torch.cuda.synchronize()
+        assert torch.equal(again, want2)

@@ -129,9 +129,12 @@ torch.cuda.synchronize()
 side = torch.cuda.Stream()
 g1 = torch.cuda.CUDAGraph()
 with torch.cuda.graph(g1, stream=side):
+    out.zero_()                                              # (a fill kernel: the captured graph is not empty)
     rc = T._call("static", a, b, None, out, 1.0, 0.0)       # the process's first call: refused, capture intact
     msg = _C.last_error()
 assert rc == -2 and "under stream capture" in msg, (rc, msg)
+g1.replay()                                                  # the capture the refused call sat in is a working graph
+torch.cuda.synchronize()
 n = ctypes.c_int(0)
 assert lib.fg_device_info(0, ctypes.byref(n), None, None) == 0 and n.value > 0
 g2 = torch.cuda.CUDAGraph()
