@@ -1,0 +1,392 @@
+"""Cases the interpreted device runs through the C-ABI: each builds seeded inputs with numpy, calls one entry point
+and returns the arrays a checker needs (inputs and outputs).  No torch here: the process that runs these must not
+have the real HIP runtime in its global symbol scope.  16-bit floats travel as bit patterns: bf16 as uint16, f16 as
+numpy float16.
+"""
+import ctypes as C
+
+import numpy as np
+
+from device import BF16, F16, F32, E
+
+DT = {"bf16": BF16, "f16": F16, "f32": F32}
+ITEM = {"bf16": 2, "f16": 2, "f32": 4}
+
+
+def bits(a, dtype):
+    """fp32 array -> storage array of `dtype` (round to nearest even)."""
+    a = np.asarray(a, np.float32)
+    if dtype == "bf16":
+        return E.bf16_round(a.ravel()).astype(np.uint16).reshape(a.shape)
+    if dtype == "f16":
+        with np.errstate(over="ignore"):
+            return a.astype(np.float16)
+    return a
+
+
+def storage(dtype):
+    return {"bf16": np.uint16, "f16": np.float16, "f32": np.float32}[dtype]
+
+
+def P(x):
+    return C.c_void_p(int(x))
+
+
+def I64(x):
+    return C.c_int64(int(x))
+
+
+def I32(x):
+    return C.c_int(int(x))
+
+
+def F(x):
+    return C.c_float(float(x))
+
+
+class Strided:
+    """A [rows, cols] matrix inside a wider allocation: row stride >= cols, the gap filled with a sentinel that a
+    checker verifies untouched."""
+
+    def __init__(self, dev, rows, cols, stride, dtype, data=None, name="buf"):
+        self.rows, self.cols, self.stride, self.dtype = rows, cols, stride, dtype
+        full = np.full((rows, stride), 0, dtype=storage(dtype))
+        full.view(np.uint16 if ITEM[dtype] == 2 else np.uint32)[:] = 0x7B7B if ITEM[dtype] == 2 else 0x7B7B7B7B
+        if data is not None:
+            full[:, :cols] = data
+        self.initial = full.copy()
+        n = (rows - 1) * stride + cols if rows else 0       # the allocation ends with the last row's last element
+        self.ptr = dev.upload(full.ravel()[:n], name) if n else dev.alloc(16, name)
+        self.dev, self.n = dev, n
+
+    def read(self):
+        flat = np.zeros(self.rows * self.stride, dtype=storage(self.dtype))
+        flat[:self.n] = self.dev.download(self.ptr, storage(self.dtype), (self.n,))
+        full = flat.reshape(self.rows, self.stride)
+        gap_ok = True
+        if self.stride > self.cols and self.rows:
+            a = full.view(np.uint16 if ITEM[self.dtype] == 2 else np.uint32)
+            b = self.initial.view(a.dtype)
+            gap = np.ones_like(a, dtype=bool)
+            gap[:, :self.cols] = False
+            gap.ravel()[self.n:] = False
+            gap_ok = bool((a[gap] == b[gap]).all())
+        return full[:, :self.cols].copy(), gap_ok
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# row-wise operators
+# ---------------------------------------------------------------------------------------------------------------
+def rms_norm(dev, rng, dtype, M, N, weight=True, inv=True, xs=None, ys=None, eps=1e-5):
+    xs, ys = xs or N, ys or N
+    x = bits(rng.standard_normal((M, N)), dtype)
+    w = bits(rng.standard_normal(N) * 0.5 + 1.0, dtype)
+    X = Strided(dev, M, N, xs, dtype, x, "x")
+    Y = Strided(dev, M, N, ys, dtype, None, "y")
+    pw = dev.upload(w, "w") if weight else 0
+    pi = dev.alloc(max(M, 1) * 4, "inv_rms") if inv else 0
+    rc = dev.call("fg_rms_norm", P(X.ptr), P(pw), P(Y.ptr), P(pi), I64(M), I64(N), I64(xs), I64(ys), F(eps), I32(DT[dtype]), P(0))
+    y, gap_ok = Y.read()
+    out = {"rc": rc, "x": x, "w": w, "y": y, "gap_ok": gap_ok, "x_after": X.read()[0]}
+    if inv:
+        out["inv_rms"] = dev.download(pi, np.float32, (M,))
+    return out
+
+
+def fused_add_rms_norm(dev, rng, dtype, M, N, weight=True, xs=None, rs=None, eps=1e-5):
+    xs, rs = xs or N, rs or N
+    x = bits(rng.standard_normal((M, N)), dtype)
+    r = bits(rng.standard_normal((M, N)), dtype)
+    w = bits(rng.standard_normal(N) * 0.5 + 1.0, dtype)
+    X = Strided(dev, M, N, xs, dtype, x, "x")
+    R = Strided(dev, M, N, rs, dtype, r, "residual")
+    pw = dev.upload(w, "w") if weight else 0
+    rc = dev.call("fg_fused_add_rms_norm", P(X.ptr), P(R.ptr), P(pw), I64(M), I64(N), I64(xs), I64(rs), F(eps), I32(DT[dtype]), P(0))
+    xo, g1 = X.read()
+    ro, g2 = R.read()
+    return {"rc": rc, "x": x, "residual": r, "w": w, "x_out": xo, "residual_out": ro, "gap_ok": g1 and g2}
+
+
+def softmax(dev, rng, dtype, M, N, K, log=False, out_dtype=None, scale=3.0):
+    out_dtype = out_dtype or dtype
+    x = bits(rng.standard_normal((M, N, K)) * scale, dtype)
+    px = dev.upload(x, "in")
+    po = dev.alloc(max(M * N * K, 1) * ITEM[out_dtype], "out")
+    rc = dev.call("fg_log_softmax" if log else "fg_softmax", P(px), P(po), I64(M), I64(N), I64(K), I32(DT[dtype]),
+                  I32(DT[out_dtype]), P(0))
+    return {"rc": rc, "x": x, "out": dev.download(po, storage(out_dtype), (M, N, K))}
+
+
+def softmax_backward(dev, rng, dtype, M, N, K, log=False, grad_in_dtype=None):
+    grad_in_dtype = grad_in_dtype or dtype
+    z = rng.standard_normal((M, N, K)) * 2.0
+    z = z - z.max(axis=1, keepdims=True)
+    p = np.exp(z) / np.exp(z).sum(axis=1, keepdims=True)
+    out = bits(np.log(p) if log else p, dtype)
+    g = bits(rng.standard_normal((M, N, K)), dtype)
+    po, pg = dev.upload(out, "out"), dev.upload(g, "grad_out")
+    pi = dev.alloc(max(M * N * K, 1) * ITEM[grad_in_dtype], "grad_in")
+    rc = dev.call("fg_log_softmax_backward" if log else "fg_softmax_backward", P(po), P(pg), P(pi), I64(M), I64(N), I64(K),
+                  I32(DT[dtype]), I32(DT[grad_in_dtype]), P(0))
+    return {"rc": rc, "out": out, "grad_out": g, "grad_in": dev.download(pi, storage(grad_in_dtype), (M, N, K))}
+
+
+def rms_norm_backward(dev, rng, dtype, M, N, weight=True, dw=True, eps=1e-5):
+    x = bits(rng.standard_normal((M, N)), dtype)
+    dy = bits(rng.standard_normal((M, N)), dtype)
+    w = bits(rng.standard_normal(N) * 0.5 + 1.0, dtype)
+    xf = x.astype(np.float32) if dtype != "bf16" else (x.astype(np.uint32) << 16).view(np.float32)
+    inv = (1.0 / np.sqrt((xf.astype(np.float64) ** 2).mean(axis=1) + eps)).astype(np.float32)
+    px, pdy, pinv = dev.upload(x, "x"), dev.upload(dy, "dy"), dev.upload(inv, "inv_rms")
+    pw = dev.upload(w, "w") if weight else 0
+    pdx = dev.alloc(M * N * ITEM[dtype], "dx")
+    dev.lib.fg_rms_norm_backward_partial_rows.restype = C.c_int64
+    rows = int(dev.call("fg_rms_norm_backward_partial_rows", I64(M), I64(N), I32(DT[dtype]), I32(0))) if dw else 0
+    ppart = dev.alloc(rows * N * 4 + 32, "dw_partial", fill=0x7B) if dw else 0
+    rc = dev.call("fg_rms_norm_backward", P(px), P(pdy), P(pinv), P(pw), P(pdx), P(ppart), I64(rows), I64(M), I64(N),
+                  I32(DT[dtype]), P(0))
+    out = {"rc": rc, "x": x, "dy": dy, "w": w, "inv_rms": inv, "dx": dev.download(pdx, storage(dtype), (M, N)),
+           "partial_rows": np.array(rows)}
+    if dw and rc == 0:
+        pdw = dev.alloc(N * ITEM[dtype], "dw")
+        out["rc_dw"] = dev.call("fg_rms_norm_backward_dw", P(ppart), I64(rows), I64(N), P(pdw), I32(DT[dtype]), P(0))
+        out["dw"] = dev.download(pdw, storage(dtype), (N,))
+        out["dw_partial"] = dev.download(ppart, np.float32, (rows, N))
+    return out
+
+
+def transpose2d(dev, rng, elem_bytes, rows, cols, src_stride=None, dst_stride=None):
+    src_stride, dst_stride = src_stride or cols, dst_stride or rows
+    dtype = "bf16" if elem_bytes == 2 else "f32"
+    data = rng.integers(0, 1 << 16, size=(rows, cols)).astype(np.uint16) if elem_bytes == 2 else \
+        rng.standard_normal((rows, cols)).astype(np.float32)
+    S = Strided(dev, rows, cols, src_stride, dtype, data, "src")
+    D = Strided(dev, cols, rows, dst_stride, dtype, None, "dst")
+    rc = dev.call("fg_transpose2d", P(S.ptr), P(D.ptr), I64(rows), I64(cols), I64(src_stride), I64(dst_stride), I32(elem_bytes), P(0))
+    d, gap_ok = D.read()
+    return {"rc": rc, "src": data, "dst": d, "gap_ok": gap_ok}
+
+
+def silu_and_mul(dev, rng, dtype, rows, cols, a_stride=None, b_stride=None, o_stride=None):
+    a_stride, b_stride, o_stride = a_stride or cols, b_stride or cols, o_stride or cols
+    a = bits(rng.standard_normal((rows, cols)) * 2, dtype)
+    b = bits(rng.standard_normal((rows, cols)), dtype)
+    A, B = Strided(dev, rows, cols, a_stride, dtype, a, "a"), Strided(dev, rows, cols, b_stride, dtype, b, "b")
+    O = Strided(dev, rows, cols, o_stride, dtype, None, "out")
+    rc = dev.call("fg_silu_and_mul", P(A.ptr), P(B.ptr), P(O.ptr), I64(rows), I64(cols), I64(a_stride), I64(b_stride), I64(o_stride),
+                  I32(DT[dtype]), P(0))
+    o, gap_ok = O.read()
+    return {"rc": rc, "a": a, "b": b, "out": o, "gap_ok": gap_ok}
+
+
+def rope(dev, rng, dtype, n_tokens, Hq, Hk, D, interleaved=False, pos="i64", inplace=True, cs_dtype="f32", max_pos=64,
+         seq_len=None, head_pad=0):
+    """q [n_tokens, Hq, D] with `head_pad` unused elements behind every head (a slice of a wider projection)."""
+    seq_len = seq_len or n_tokens
+    hs = D + head_pad
+    q = bits(rng.standard_normal((n_tokens, Hq, hs)), dtype)
+    k = bits(rng.standard_normal((n_tokens, Hk, hs)), dtype)
+    ang = rng.uniform(0, 6.28, size=(max_pos, D // 2))
+    cos, sin = bits(np.cos(ang), cs_dtype), bits(np.sin(ang), cs_dtype)
+    positions = rng.integers(0, max_pos, size=n_tokens)
+    pq, pk = dev.upload(q, "q"), dev.upload(k, "k")
+    pqo = pq if inplace else dev.alloc(q.nbytes, "q_out", fill=0x7B)
+    pko = pk if inplace else dev.alloc(k.nbytes, "k_out", fill=0x7B)
+    pc, ps = dev.upload(cos, "cos"), dev.upload(sin, "sin")
+    ppos = 0
+    if pos == "i64":
+        ppos = dev.upload(positions.astype(np.int64), "pos")
+    elif pos == "i32":
+        ppos = dev.upload(positions.astype(np.int32), "pos")
+    else:
+        positions = np.arange(n_tokens) % seq_len
+    arr = C.c_int64 * 3
+    qs, ks = arr(Hq * hs, hs, 1), arr(Hk * hs, hs, 1)
+    rc = dev.call("fg_rope", P(pqo), P(pko), P(pq), P(pk), P(pc), P(ps), P(ppos), I32(pos == "i64"), I64(n_tokens), I64(seq_len),
+                  I32(Hq), I32(Hk), I32(D), qs, ks, qs, ks, I64(1), I64(D // 2), I64(D // 2), I64(max_pos), I32(interleaved),
+                  I32(DT[dtype]), I32(DT[cs_dtype]), P(0))
+    return {"rc": rc, "q": q, "k": k, "cos": cos, "sin": sin, "positions": positions.astype(np.int64),
+            "q_out": dev.download(pqo, storage(dtype), q.shape), "k_out": dev.download(pko, storage(dtype), k.shape)}
+
+
+def reshape_and_cache_flash(dev, rng, elem_bytes, num_tokens, H, D, block_size, num_blocks, slot_i64=True, token_pad=0,
+                            block_pad=0):
+    st = np.uint16 if elem_bytes == 2 else (np.uint8 if elem_bytes == 1 else np.uint32)
+    ts = H * D + token_pad
+    bs = block_size * H * D + block_pad
+    key = rng.integers(0, 200, size=(num_tokens, ts)).astype(st)
+    val = rng.integers(0, 200, size=(num_tokens, ts)).astype(st)
+    slots = rng.permutation(num_blocks * block_size)[:num_tokens].astype(np.int64)
+    if num_tokens > 2:
+        slots[1] = -1
+    kc = rng.integers(200, 250, size=(num_blocks, bs)).astype(st)
+    vc = rng.integers(200, 250, size=(num_blocks, bs)).astype(st)
+    pk, pv = dev.upload(key.ravel()[:(num_tokens - 1) * ts + H * D], "key"), dev.upload(val.ravel()[:(num_tokens - 1) * ts + H * D], "value")
+    pkc, pvc = dev.upload(kc.ravel()[:(num_blocks - 1) * bs + block_size * H * D], "key_cache"), \
+        dev.upload(vc.ravel()[:(num_blocks - 1) * bs + block_size * H * D], "value_cache")
+    ps = dev.upload(slots if slot_i64 else slots.astype(np.int32), "slot_mapping")
+    rc = dev.call("fg_reshape_and_cache_flash", P(pk), P(pv), P(pkc), P(pvc), P(ps), I32(slot_i64), I64(num_tokens), I32(H), I32(D),
+                  I32(block_size), I64(ts), I64(ts), I64(bs), I32(elem_bytes), P(0))
+    n = (num_blocks - 1) * bs + block_size * H * D
+    kco, vco = kc.copy(), vc.copy()
+    kco.ravel()[:n] = dev.download(pkc, st, (n,))
+    vco.ravel()[:n] = dev.download(pvc, st, (n,))
+    return {"rc": rc, "key": key, "value": val, "slots": slots, "key_cache_before": kc, "value_cache_before": vc,
+            "key_cache": kco, "value_cache": vco, "dims": np.array([H, D, block_size, ts, bs])}
+
+
+def reshape_and_cache(dev, rng, elem_bytes, num_tokens, H, D, block_size, x, num_blocks, slot_i64=True):
+    st = np.uint16 if elem_bytes == 2 else np.uint32
+    key = rng.integers(0, 200, size=(num_tokens, H, D)).astype(st)
+    val = rng.integers(0, 200, size=(num_tokens, H, D)).astype(st)
+    slots = rng.permutation(num_blocks * block_size)[:num_tokens].astype(np.int64)
+    if num_tokens > 2:
+        slots[1] = -1
+        slots[2] = num_blocks * block_size + 3       # past the last block: skipped
+    kc = rng.integers(200, 250, size=(num_blocks, H, D // x, block_size, x)).astype(st)
+    vc = rng.integers(200, 250, size=(num_blocks, H, D, block_size)).astype(st)
+    pk, pv, pkc, pvc = dev.upload(key, "key"), dev.upload(val, "value"), dev.upload(kc, "key_cache"), dev.upload(vc, "value_cache")
+    ps = dev.upload(slots if slot_i64 else slots.astype(np.int32), "slot_mapping")
+    rc = dev.call("fg_reshape_and_cache", P(pk), P(pv), P(pkc), P(pvc), P(ps), I32(slot_i64), I64(num_tokens), I32(H), I32(D),
+                  I32(block_size), I32(x), I64(num_blocks), I64(H * D), I64(H * D), I32(elem_bytes), P(0))
+    return {"rc": rc, "key": key, "value": val, "slots": slots, "key_cache_before": kc, "value_cache_before": vc,
+            "key_cache": dev.download(pkc, st, kc.shape), "value_cache": dev.download(pvc, st, vc.shape)}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------------------------------------------
+def gemm(dev, rng, dtype, M, N, K, b_layout="kn", bias=None, alpha=1.0, beta=1.0, schedule=0, c_dtype=None, entry="fg_gemm",
+         a_pad=0):
+    """b_layout "kn": B row-major [K, N]; "nk": B stored [N, K] (K-contiguous, the weight layout).
+    bias: None, "row" ([N] broadcast over rows), "full" ([M, N])."""
+    c_dtype = c_dtype or dtype
+    a = bits(rng.standard_normal((M, K + a_pad)) * 0.5, dtype)
+    b = bits(rng.standard_normal((K, N)) * 0.5, dtype)
+    pa = dev.upload(a.ravel()[:(M - 1) * (K + a_pad) + K], "A")
+    if b_layout == "kn":
+        pb, sbk, sbn = dev.upload(b, "B"), N, 1
+    else:
+        pb, sbk, sbn = dev.upload(np.ascontiguousarray(b.T), "B"), 1, K
+    pc = dev.alloc(M * N * ITEM[c_dtype], "C", fill=0x7B)
+    pbias, sim, sin_ = 0, 0, 0
+    bias_arr = np.zeros(0, np.float32)
+    if bias == "row":
+        bias_arr = bits(rng.standard_normal(N), dtype)
+        pbias, sim, sin_ = dev.upload(bias_arr, "bias"), 0, 1
+    elif bias == "full":
+        bias_arr = bits(rng.standard_normal((M, N)), dtype)
+        pbias, sim, sin_ = dev.upload(bias_arr, "bias"), N, 1
+    used = C.c_int(-1)
+    out = {}
+    if entry == "fg_gemm":
+        dev.lib.fg_gemm_workspace_bytes.restype = C.c_size_t
+        need = int(dev.call("fg_gemm_workspace_bytes", I64(M), I64(N), I64(K), I32(DT[dtype]), I32(schedule), I32(0)))
+        pws = dev.alloc(need + 256, "workspace") if need else 0
+        rc = dev.call("fg_gemm", P(pa), P(pb), P(pbias), P(pc), I64(M), I64(N), I64(K), I64(K + a_pad), I64(1), I64(sbk), I64(sbn),
+                      I64(sim), I64(sin_), I64(N), I64(1), F(alpha), F(beta), I32(DT[dtype]), I32(DT[c_dtype]), I32(DT[dtype]),
+                      I32(schedule), P(pws), C.c_size_t(need), C.byref(used), P(0))
+        out["workspace_bytes"] = np.array(need)
+        if need:   # the header (ticket counters) must read zero again after the launch
+            hdr = C.c_size_t(0)
+            mx = C.c_size_t(0)
+            dev.call("fg_gemm_workspace_layout", I32(0), C.byref(mx), C.byref(hdr))
+            out["header_after"] = dev.download(pws, np.uint8, (min(int(hdr.value), need),))
+    else:
+        rc = dev.call("fg_gemm_skinny_static", P(pa), P(pb), P(pbias), P(pc), I64(M), I64(N), I64(K), I64(K + a_pad), I64(1),
+                      I64(sbk), I64(sbn), I64(sim), I64(sin_), I64(N), I64(1), F(alpha), F(beta), I32(DT[dtype]), I32(DT[c_dtype]),
+                      I32(DT[dtype]), P(0))
+    out.update({"rc": rc, "a": a[:, :K].copy(), "b": b, "bias": bias_arr, "c": dev.download(pc, storage(c_dtype), (M, N)),
+                "schedule_used": np.array(used.value)})
+    return out
+
+
+def bmm(dev, rng, dtype, batch, M, N, K):
+    a = bits(rng.standard_normal((batch, M, K)) * 0.5, dtype)
+    b = bits(rng.standard_normal((batch, K, N)) * 0.5, dtype)
+    pa, pb = dev.upload(a, "A"), dev.upload(b, "B")
+    pc = dev.alloc(batch * M * N * ITEM[dtype], "C", fill=0x7B)
+    rc = dev.call("fg_bmm", P(pa), P(pb), P(pc), I64(batch), I64(M), I64(N), I64(K), I64(M * K), I64(K), I64(1), I64(K * N), I64(N),
+                  I64(1), I64(M * N), I64(N), I64(1), I32(DT[dtype]), P(0))
+    return {"rc": rc, "a": a, "b": b, "c": dev.download(pc, storage(dtype), (batch, M, N))}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# attention over a paged KV cache
+# ---------------------------------------------------------------------------------------------------------------
+class FgFlashParams(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("out", C.c_void_p), ("lse", C.c_void_p),
+                ("cu_seqlens_q", C.c_void_p), ("seqused_k", C.c_void_p), ("block_table", C.c_void_p), ("alibi_slopes", C.c_void_p),
+                ("q_row_stride", C.c_int64), ("q_head_stride", C.c_int64), ("o_row_stride", C.c_int64), ("o_head_stride", C.c_int64),
+                ("k_page_stride", C.c_int64), ("k_row_stride", C.c_int64), ("k_head_stride", C.c_int64),
+                ("v_page_stride", C.c_int64), ("v_row_stride", C.c_int64), ("v_head_stride", C.c_int64),
+                ("block_table_stride", C.c_int64), ("alibi_batch_stride", C.c_int64), ("total_q", C.c_int64),
+                ("batch", C.c_int32), ("Hq", C.c_int32), ("Hk", C.c_int32), ("D", C.c_int32), ("page_size", C.c_int32),
+                ("max_seqlen_q", C.c_int32), ("max_seqlen_k", C.c_int32), ("is_causal", C.c_int32),
+                ("window_left", C.c_int32), ("window_right", C.c_int32), ("softmax_scale", C.c_float), ("softcap", C.c_float),
+                ("dtype", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_int64)]
+
+
+def attention(dev, rng, dtype, q_lens, k_lens, Hq, Hk, D, page_size, causal=True, window=(-1, -1), softcap=0.0, alibi=False,
+              lse=True, workspace=True, spare_pages=2):
+    """Sequences of q_lens[i] queries over k_lens[i] cached keys, pages handed out in a shuffled order."""
+    batch = len(q_lens)
+    total_q = int(sum(q_lens))
+    pages_per = [(k + page_size - 1) // page_size for k in k_lens]
+    num_pages = sum(pages_per) + spare_pages
+    max_pages = max(pages_per)
+    q = bits(rng.standard_normal((total_q, Hq, D)), dtype)
+    kc = bits(rng.standard_normal((num_pages, page_size, Hk, D)), dtype)
+    vc = bits(rng.standard_normal((num_pages, page_size, Hk, D)), dtype)
+    order = rng.permutation(num_pages)
+    table = np.zeros((batch, max_pages), dtype=np.int32)
+    at = 0
+    for i, n in enumerate(pages_per):
+        table[i, :n] = order[at:at + n]
+        at += n
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    used = np.asarray(k_lens, dtype=np.int32)
+    slopes = (rng.uniform(0.05, 0.5, size=(batch, Hq))).astype(np.float32)
+    p = FgFlashParams()
+    p.q, p.k_cache, p.v_cache = dev.upload(q, "q"), dev.upload(kc, "k_cache"), dev.upload(vc, "v_cache")
+    p.out = dev.alloc(q.nbytes, "out", fill=0x7B)
+    p.lse = dev.alloc(Hq * total_q * 4, "lse", fill=0x7B) if lse else 0
+    p.cu_seqlens_q, p.seqused_k, p.block_table = dev.upload(cu, "cu_seqlens_q"), dev.upload(used, "seqused_k"), dev.upload(table, "block_table")
+    p.alibi_slopes = dev.upload(slopes, "alibi_slopes") if alibi else 0
+    p.q_row_stride, p.q_head_stride, p.o_row_stride, p.o_head_stride = Hq * D, D, Hq * D, D
+    p.k_page_stride = p.v_page_stride = page_size * Hk * D
+    p.k_row_stride = p.v_row_stride = Hk * D
+    p.k_head_stride = p.v_head_stride = D
+    p.block_table_stride, p.alibi_batch_stride, p.total_q = max_pages, Hq if alibi else 0, total_q
+    p.batch, p.Hq, p.Hk, p.D, p.page_size = batch, Hq, Hk, D, page_size
+    p.max_seqlen_q, p.max_seqlen_k = int(max(q_lens)), int(max(k_lens))
+    p.is_causal, p.window_left, p.window_right = int(causal), window[0], window[1]
+    p.softmax_scale, p.softcap, p.dtype = float(D) ** -0.5, softcap, DT[dtype]
+    dev.lib.fg_flash_attn_workspace_bytes.restype = C.c_size_t
+    need = int(dev.call("fg_flash_attn_workspace_bytes", C.byref(p), I32(0))) if workspace else 0
+    p.workspace = dev.alloc(need, "workspace", fill=0x7B) if need else 0
+    p.workspace_bytes = need
+    rc = dev.call("fg_flash_attn_varlen_fwd", C.byref(p), P(0))
+    out = {"rc": rc, "q": q, "k_cache": kc, "v_cache": vc, "block_table": table, "q_lens": np.asarray(q_lens), "k_lens": np.asarray(k_lens),
+           "out": dev.download(p.out, storage(dtype), q.shape), "slopes": slopes, "workspace_bytes": np.array(need)}
+    if lse:
+        out["lse"] = dev.download(p.lse, np.float32, (Hq, total_q))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the interpreter's own guard: a call whose buffers are too small must be reported, not absorbed
+# ---------------------------------------------------------------------------------------------------------------
+def short_buffer(dev, rng, which):
+    """fg_rms_norm on [4, 2048] bf16 with one operand allocated 16 bytes short; returns the interpreter's message."""
+    M, N = 4, 2048
+    x = bits(rng.standard_normal((M, N)), "bf16")
+    w = bits(np.ones(N), "bf16")
+    px = dev.upload(x.ravel()[:M * N - (8 if which == "x" else 0)], "x")
+    pw = dev.upload(w[:N - (8 if which == "w" else 0)], "w")
+    py = dev.alloc((M * N - (8 if which == "y" else 0)) * 2, "y")
+    try:
+        rc = dev.call("fg_rms_norm", P(px), P(pw), P(py), P(0), I64(M), I64(N), I64(N), I64(N), F(1e-5), I32(BF16), P(0))
+        return {"rc": rc, "caught": np.array("")}
+    except E.EmuError as exc:
+        return {"rc": 0, "caught": np.array(str(exc).splitlines()[0])}
