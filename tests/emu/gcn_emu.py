@@ -106,13 +106,60 @@ class Memory:
 _KERNEL = re.compile(r"^([A-Za-z_]\w*):[^\n]*\n(.*?)^\.Lfunc_end\d+:", re.S | re.M)
 
 
+_TOK_REG = re.compile(r"^(?:-|neg\(|abs\(|sext\(|\|)*([vsa])(?:(\d+)|\[(\d+):(\d+)\])[)|]*$")
+_WAIT = re.compile(r"(vmcnt|lgkmcnt|expcnt)\((\d+)\)")
+
+
 class Instr:
-    __slots__ = ("op", "base", "enc", "ops", "mods", "line")
+    __slots__ = ("op", "base", "enc", "ops", "mods", "line", "vset", "sset", "wait", "ld_queue", "ld_only_dest")
 
     def __init__(self, op, ops, mods, line):
         self.op, self.ops, self.mods, self.line = op, ops, mods, line
         m = re.match(r"^(.*?)(_e32|_e64|_dpp|_sdwa|_e64_dpp)?$", op)
         self.base, self.enc = m.group(1), (m.group(2) or "")
+        # registers the instruction names (sources and destinations alike), for the in-flight checks
+        vs, ss = set(), set()
+        for t in ops:
+            mm = _TOK_REG.match(t)
+            if mm:
+                lo = int(mm.group(2) if mm.group(2) is not None else mm.group(3))
+                hi = lo if mm.group(2) is not None else int(mm.group(4))
+                if mm.group(1) == "s":
+                    ss.update(range(lo, hi + 1))
+                else:
+                    vs.update(range(lo + (256 if mm.group(1) == "a" else 0), hi + 1 + (256 if mm.group(1) == "a" else 0)))
+            elif t == "vcc":
+                ss.update((106, 107))
+            elif t in _SPECIAL_EARLY:
+                ss.add(_SPECIAL_EARLY[t])
+        self.vset, self.sset = frozenset(vs), frozenset(ss)
+        # A load may name as its destination a register that an older load OF THE SAME COUNTER has yet to write (results
+        # of one counter arrive in order: the compiler does this for loads under complementary EXEC masks).  Registers
+        # that are only the destination, not also part of the address or data operands, get that exemption.
+        self.ld_queue, self.ld_only_dest = None, frozenset()
+        if (op.startswith(("global_load_", "scratch_load_")) and not op.startswith("global_load_lds")) or \
+                op.startswith(("ds_read", "ds_bpermute", "ds_permute", "ds_swizzle")):
+            self.ld_queue = 0 if op[0] != "d" else 1
+            def regs_of(t):
+                mm = _TOK_REG.match(t)
+                if not mm or mm.group(1) == "s":
+                    return set()
+                lo = int(mm.group(2) if mm.group(2) is not None else mm.group(3))
+                hi = lo if mm.group(2) is not None else int(mm.group(4))
+                off = 256 if mm.group(1) == "a" else 0
+                return set(range(lo + off, hi + 1 + off))
+            others = set()
+            for t in ops[1:]:
+                others |= regs_of(t)
+            self.ld_only_dest = frozenset(regs_of(ops[0]) - others)
+        self.wait = None
+        if op == "s_waitcnt":
+            self.wait = {k: int(v) for k, v in _WAIT.findall(ops[0] if ops else "")}
+            if ops and not self.wait and ops[0].strip():
+                raise EmuError("cannot read the counts of %r" % line)
+
+
+_SPECIAL_EARLY = {"vcc_lo": 106, "vcc_hi": 107, "m0": 124}
 
 
 def _split_operands(text):
@@ -278,6 +325,10 @@ class Wave:
         self.done = False
         self.at_barrier = False
         self.scratch = {}
+        self.wid = 0
+        # memory operations issued and not yet covered by a wait, oldest first (see Exec.strict)
+        self.vm_q, self.lds_q, self.smem_q = [], [], []
+        self.pend_v, self.pend_s = {}, {}
 
     # 64-bit specials live in the scalar file
     @property
@@ -322,8 +373,138 @@ def _parse_lit(tok, fkind):
 class Exec:
     """Executes one instruction of one wave."""
 
-    def __init__(self, mem, lds, program):
+    def __init__(self, mem, lds, program, strict=True):
         self.mem, self.lds, self.prog = mem, lds, program
+        # strict: memory operations stay "in flight" until an s_waitcnt covers them.  Touching a register a load in
+        # flight will write, reading LDS bytes a write or LDS-DMA in flight will fill, and LDS traffic between two
+        # wavefronts with no barrier in between are errors: the counts written by hand into asm statements, and the
+        # barriers of the software pipelines, are checked as executed.
+        self.strict = strict
+        n = lds.size
+        self.epoch = 1
+        self.w_epoch = np.zeros(n, dtype=np.int32)
+        self.w_wave = np.zeros(n, dtype=np.int16)
+        self.r_epoch = np.zeros(n, dtype=np.int32)
+        self.r_wave = np.zeros(n, dtype=np.int16)       # -1: read by several wavefronts in this epoch
+        self.fill_owner = np.zeros(n, dtype=np.int16)   # wave id + 1 of a ds_write in flight, -(wave id + 1) of an LDS-DMA
+        self.read_inflight = np.zeros(n, dtype=np.int16)
+
+    # ---- LDS --------------------------------------------------------------------------------------------------
+    def _lds_index(self, ins, addrs, width):
+        a = np.asarray(addrs).astype(np.int64)
+        if a.size and ((a < 0).any() or (a + width > self.lds.size).any()):
+            raise EmuError("LDS access outside the %d bytes allocated (address %d): %r" %
+                           (self.lds.size, int(a.max()), ins.line))
+        return a[:, None] + np.arange(width)[None, :]
+
+    def lds_get(self, w, ins, addrs, width, track=True):
+        """Bytes [n, width] at the given addresses.  Returns (raw, flat byte indices)."""
+        ix = self._lds_index(ins, addrs, width)
+        if self.strict and ix.size:
+            flat = ix.ravel()
+            own = self.fill_owner[flat]
+            bad = (own != 0) & (own != w.wid + 1)
+            if bad.any():
+                o = int(own[bad][0])
+                raise EmuError("wave %d reads LDS byte %d while %s of wave %d is in flight (no wait covers it): %r" % (
+                    w.wid, int(flat[bad][0]), "an LDS-DMA" if o < 0 else "a ds_write", abs(o) - 1, ins.line))
+            race = (self.w_epoch[flat] == self.epoch) & (self.w_wave[flat] != w.wid)
+            if race.any():
+                raise EmuError("wave %d reads LDS byte %d written by wave %d with no barrier in between: %r" % (
+                    w.wid, int(flat[race][0]), int(self.w_wave[flat][race][0]), ins.line))
+            if track:
+                same = self.r_epoch[flat] == self.epoch
+                self.r_wave[flat] = np.where(same & (self.r_wave[flat] != w.wid), -1, w.wid)
+                self.r_epoch[flat] = self.epoch
+        return self.lds[ix], ix
+
+    def lds_put(self, w, ins, addrs, raw, dma=False):
+        ix = self._lds_index(ins, addrs, raw.shape[1])
+        if self.strict and ix.size:
+            flat = ix.ravel()
+            waw = (self.w_epoch[flat] == self.epoch) & (self.w_wave[flat] != w.wid)
+            if waw.any():
+                raise EmuError("wave %d writes LDS byte %d written by wave %d with no barrier in between: %r" % (
+                    w.wid, int(flat[waw][0]), int(self.w_wave[flat][waw][0]), ins.line))
+            war = (self.r_epoch[flat] == self.epoch) & (self.r_wave[flat] != w.wid)
+            if war.any():
+                raise EmuError("wave %d writes LDS byte %d read by another wave with no barrier in between: %r" % (
+                    w.wid, int(flat[war][0]), ins.line))
+            own = self.fill_owner[flat]
+            if ((own != 0) & (own != w.wid + 1)).any() or (dma and (own != 0).any()):
+                raise EmuError("wave %d writes LDS bytes another write in flight targets: %r" % (w.wid, ins.line))
+            if dma and (self.read_inflight[flat] > 0).any():
+                raise EmuError("wave %d starts an LDS-DMA onto bytes an LDS read in flight has yet to fetch: %r" % (w.wid, ins.line))
+            self.w_epoch[flat] = self.epoch
+            self.w_wave[flat] = w.wid
+            self.fill_owner[flat] = -(w.wid + 1) if dma else (w.wid + 1)
+        self.lds[ix] = raw
+        return ix
+
+    def barrier_released(self):
+        self.epoch += 1
+
+    # ---- operations in flight -----------------------------------------------------------------------------------
+    def issue(self, w, queue, vregs=(), sregs=(), fill=None, fetch=None):
+        """Record a memory operation: registers it will write, LDS bytes it fills (fill) or fetches (fetch)."""
+        if not self.strict:
+            return
+        q = 0 if queue == "vm_q" else 1
+        for r in vregs:
+            w.pend_v.setdefault(r, [0, 0])[q] += 1
+        for r in sregs:
+            w.pend_s[r] = w.pend_s.get(r, 0) + 1
+        if fetch is not None:
+            np.add.at(self.read_inflight, fetch.ravel(), 1)
+        getattr(w, queue).append((tuple(vregs), tuple(sregs), fill, fetch, q))
+
+    def _retire(self, w, entry):
+        vregs, sregs, fill, fetch, q = entry
+        for r in vregs:
+            c = w.pend_v[r]
+            c[q] -= 1
+            if c[0] == 0 and c[1] == 0:
+                del w.pend_v[r]
+        for r in sregs:
+            if w.pend_s[r] == 1:
+                del w.pend_s[r]
+            else:
+                w.pend_s[r] -= 1
+        if fill is not None:
+            self.fill_owner[fill.ravel()] = 0
+        if fetch is not None:
+            np.subtract.at(self.read_inflight, fetch.ravel(), 1)
+
+    def wait(self, w, counts):
+        """s_waitcnt: vmcnt(n) leaves at most the n youngest vector-memory operations in flight (they complete in
+        order); lgkmcnt(n) does so for the LDS operations (in order among themselves), and only lgkmcnt(0) says
+        anything about scalar loads, which return in any order."""
+        if "vmcnt" in counts:
+            while len(w.vm_q) > counts["vmcnt"]:
+                self._retire(w, w.vm_q.pop(0))
+        if "lgkmcnt" in counts:
+            while len(w.lds_q) > counts["lgkmcnt"]:
+                self._retire(w, w.lds_q.pop(0))
+            if counts["lgkmcnt"] == 0:
+                while w.smem_q:
+                    self._retire(w, w.smem_q.pop(0))
+
+    def check_registers(self, w, ins):
+        if w.pend_v and not ins.vset.isdisjoint(w.pend_v):
+            hit = ins.vset & set(w.pend_v)
+            if ins.ld_queue is not None:
+                hit = {r for r in hit if not (r in ins.ld_only_dest and w.pend_v[r][1 - ins.ld_queue] == 0)}
+            if not hit:
+                return self._check_sregs(w, ins)
+            r = sorted(hit)[0]
+            raise EmuError("wave %d: %s%d is the destination of a load still in flight (vmcnt %d, lgkmcnt %d outstanding): %r" % (
+                w.wid, "a" if r >= 256 else "v", r % 256, len(w.vm_q), len(w.lds_q), ins.line))
+        self._check_sregs(w, ins)
+
+    def _check_sregs(self, w, ins):
+        if w.pend_s and not ins.sset.isdisjoint(w.pend_s):
+            r = sorted(ins.sset & set(w.pend_s))[0]
+            raise EmuError("wave %d: s%d is the destination of a scalar load still in flight: %r" % (w.wid, r, ins.line))
 
     # ---- scalar operands ---------------------------------------------------------------------------------------
     def sreg_index(self, tok):
@@ -646,10 +827,9 @@ def _do_load(ex, w, ins, kind, addrs, lanes, space):
     if space == "global":
         raw = ex.mem.load(addrs[act], width, ins.line)
     else:
-        a = addrs[act].astype(np.int64)
-        if (a < 0).any() or (a + width > ex.lds.size).any():
-            raise EmuError("LDS access outside the %d bytes allocated: %r" % (ex.lds.size, ins.line))
-        raw = ex.lds[a[:, None] + np.arange(width)[None, :]]
+        raw, ix = ex.lds_get(w, ins, addrs[act], width)
+        i, n = ex.vindex(ins.ops[0])
+        ex.issue(w, "lds_q", vregs=range(i, i + max(n, (width + 3) // 4)), fetch=ix)
     _land(ex, w, ins, kind, act, raw)
 
 
@@ -662,10 +842,7 @@ def _do_store(ex, w, ins, kind, addrs, lanes, data_tok, space):
     if space == "global":
         ex.mem.store(addrs[act], raw, ins.line)
     else:
-        a = addrs[act].astype(np.int64)
-        if (a < 0).any() or (a + width > ex.lds.size).any():
-            raise EmuError("LDS access outside the %d bytes allocated: %r" % (ex.lds.size, ins.line))
-        ex.lds[a[:, None] + np.arange(width)[None, :]] = raw
+        ex.issue(w, "lds_q", fill=ex.lds_put(w, ins, addrs[act], raw))
 
 
 def _scc_logic(w, val):
@@ -678,6 +855,11 @@ def step(ex, w):
     w.pc += 1
     op, base, ops, mods = ins.op, ins.base, ins.ops, ins.mods
     S = ex.sread
+    if ex.strict:
+        if ins.wait is not None:
+            ex.wait(w, ins.wait)
+            return
+        ex.check_registers(w, ins)
     # ------------------------------------------------------------------ no-ops and control
     if op in ("s_waitcnt", "s_nop", "s_sleep", "s_setprio") or op.startswith(("s_waitcnt", "s_setprio", "s_nop")):
         return
@@ -706,6 +888,7 @@ def step(ex, w):
         words = np.ascontiguousarray(raw).view(U32)
         i, _ = ex.sreg_index(ops[0])
         w.s[i:i + n] = words
+        ex.issue(w, "smem_q", sregs=range(i, i + n))
         return
     # ------------------------------------------------------------------ scalar ALU
     if op.startswith("s_"):
@@ -721,19 +904,20 @@ def step(ex, w):
         # LDS address: M0 base + instruction offset + lane * width (each lane's data lands consecutively)
         base_lds = (int(w.s[124]) & 0x3FFFF) + _offset(ins)   # the instruction offset moves both addresses
         a = base_lds + act.astype(np.int64) * width
-        if (a + width > ex.lds.size).any():
-            raise EmuError("LDS-direct load outside the %d bytes of LDS: %r" % (ex.lds.size, ins.line))
-        ex.lds[a[:, None] + np.arange(width)[None, :]] = raw
+        ex.issue(w, "vm_q", fill=ex.lds_put(w, ins, a, raw, dma=True))
         return
     if op.startswith("global_load_"):
         kind = op[len("global_load_"):]
         addrs = _global_addr(ex, w, ins, ops[1], ops[2])
         _do_load(ex, w, ins, kind, addrs, mask_to_lanes(w.exec), "global")
+        i, n = ex.vindex(ops[0])
+        ex.issue(w, "vm_q", vregs=range(i, i + max(n, (_LOAD_W[kind] + 3) // 4)))
         return
     if op.startswith("global_store_"):
         kind = op[len("global_store_"):]
         addrs = _global_addr(ex, w, ins, ops[0], ops[2])
         _do_store(ex, w, ins, kind, addrs, mask_to_lanes(w.exec), ops[1], "global")
+        ex.issue(w, "vm_q")
         return
     if op.startswith("global_atomic_"):
         return _global_atomic(ex, w, ins)
@@ -1592,17 +1776,22 @@ def _ds(ex, w, ins):
         if m.group(1) == "read":
             base = ex.vread(w, ops[1], 32).astype(np.int64)
             i, _ = ex.vindex(ops[0])
+            fetched = []
             for k, o in enumerate((o0, o1)):
-                raw = ex.lds[_lds_bytes(ex, ins, base[act] + o, width)]
+                raw, ix = ex.lds_get(w, ins, base[act] + o, width)
                 words = np.ascontiguousarray(raw).view(U32).reshape(len(act), nd)
                 for d in range(nd):
                     w.v[i + k * nd + d][act] = words[:, d]
+                fetched.append(ix)
+            ex.issue(w, "lds_q", vregs=range(i, i + 2 * nd), fetch=np.concatenate([f.ravel() for f in fetched]))
         else:
             base = ex.vread(w, ops[0], 32).astype(np.int64)
+            filled = []
             for k, o in enumerate((o0, o1)):
                 i, _ = ex.vindex(ops[1 + k])
                 words = np.stack([w.v[i + d][act] for d in range(nd)], axis=1)
-                ex.lds[_lds_bytes(ex, ins, base[act] + o, width)] = np.ascontiguousarray(words).view(np.uint8).reshape(len(act), width)
+                filled.append(ex.lds_put(w, ins, base[act] + o, np.ascontiguousarray(words).view(np.uint8).reshape(len(act), width)))
+            ex.issue(w, "lds_q", fill=np.concatenate([f.ravel() for f in filled]))
         return
     if op in ("ds_bpermute_b32", "ds_permute_b32"):
         addr = ((ex.vread(w, ops[1], 32).astype(np.int64) + off) >> 2) & 63
@@ -1613,7 +1802,8 @@ def _ds(ex, w, ins):
             res = np.zeros(64, dtype=U32)
             for lane in act:                       # later lanes win, as the hardware's write order does
                 res[addr[lane]] = data[lane]
-        return ex.vwrite(w, ops[0], res)
+        ex.vwrite(w, ops[0], res)
+        return ex.issue(w, "lds_q", vregs=(ex.vindex(ops[0])[0],))
     if op == "ds_swizzle_b32":
         pat = off
         data = ex.vread(w, ops[1], 32)
@@ -1623,7 +1813,8 @@ def _ds(ex, w, ins):
         else:
             and_m, or_m, xor_m = pat & 31, (pat >> 5) & 31, (pat >> 10) & 31
             src = (idx & 32) | ((((idx & 31) & and_m) | or_m) ^ xor_m)
-        return ex.vwrite(w, ops[0], np.where(lanes[src], data[src], U32(0)))
+        ex.vwrite(w, ops[0], np.where(lanes[src], data[src], U32(0)))
+        return ex.issue(w, "lds_q", vregs=(ex.vindex(ops[0])[0],))
     if op == "ds_read_b64_tr_b16":
         # Each group of 16 lanes holds a 16 x 16 block of 16-bit elements, lane r of the group addressing 4 consecutive
         # elements of row (r % 16)... lane i of the group reads its own 8 bytes; the result for lane i, element j is the
@@ -1638,7 +1829,7 @@ def _ds(ex, w, ins):
         data = ex.vread(w, d_tok, 32)
         name = "%s_%s" % (m.group(1), m.group(3))
         out = np.zeros(64, dtype=U32)
-        for lane in act:
+        for lane in act:                      # atomics are the sanctioned way to share bytes without a barrier: not tracked
             ix = _lds_bytes(ex, ins, addrs[lane:lane + 1], 4)
             old = int(np.ascontiguousarray(ex.lds[ix]).view(U32)[0, 0])
             new = _atomic_apply(name, old, int(data[lane]))
@@ -1646,7 +1837,7 @@ def _ds(ex, w, ins):
             out[lane] = old
         if rtn:
             ex.vwrite(w, ops[0], out)
-        return
+        return ex.issue(w, "lds_q", vregs=(ex.vindex(ops[0])[0],) if rtn else ())
     raise EmuError("unknown LDS instruction: %r" % ins.line)
 
 
@@ -1657,7 +1848,7 @@ def _ds_read_tr16(ex, w, ins):
     if not lanes.all():
         raise EmuError("transposing LDS read under a partial EXEC is not modelled: %r" % ins.line)
     addrs = ex.vread(w, ins.ops[1], 32).astype(np.int64) + _offset(ins)
-    raw = ex.lds[_lds_bytes(ex, ins, addrs, 8)]
+    raw, ix = ex.lds_get(w, ins, addrs, 8)
     el = np.ascontiguousarray(raw).view(np.uint16).reshape(64, 4).astype(U32)
     i = np.arange(64)
     grp, li = i // 16 * 16, i % 16
@@ -1667,6 +1858,7 @@ def _ds_read_tr16(ex, w, ins):
     d, _ = ex.vindex(ins.ops[0])
     w.v[d] = out[:, 0] | (out[:, 1] << U32(16))
     w.v[d + 1] = out[:, 2] | (out[:, 3] << U32(16))
+    ex.issue(w, "lds_q", vregs=(d, d + 1), fetch=ix)
 
 
 def _global_atomic(ex, w, ins):
@@ -1692,6 +1884,7 @@ def _global_atomic(ex, w, ins):
         out[lane] = old
     if rtn:
         ex.vwrite(w, ops[0], out)
+    ex.issue(w, "vm_q", vregs=(ex.vindex(ops[0])[0],) if rtn else ())
 
 
 def _scratch(ex, w, ins):
@@ -1716,8 +1909,11 @@ def _scratch(ex, w, ins):
     ix = addr[act][:, None] + np.arange(width)[None, :]
     if load:
         _land(ex, w, ins, kind, act, w.scratch_mem[act[:, None], ix])
+        i, n = ex.vindex(ops[0])
+        ex.issue(w, "vm_q", vregs=range(i, i + max(n, (width + 3) // 4)))
     else:
         w.scratch_mem[act[:, None], ix] = _lift(ex, w, kind, act, ops[1])
+        ex.issue(w, "vm_q")
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -1760,7 +1956,7 @@ def pack_kernarg(prog, values, grid, block, dynamic_lds=0):
     return bytes(buf)
 
 
-def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, groups=None, trace=None):
+def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, groups=None, trace=None, strict=True):
     """Run the kernel over `grid` workgroups of `block` work-items (3-tuples).  `groups` limits the run to the listed
     workgroup ids (tuples); every memory access of the run is bounds-checked by `mem`."""
     kd = prog.kd
@@ -1782,10 +1978,11 @@ def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, 
     all_groups = [(x, y, z) for z in range(grid[2]) for y in range(grid[1]) for x in range(grid[0])]
     for g in (groups if groups is not None else all_groups):
         lds = np.zeros(lds_size, dtype=np.uint8)
-        ex = Exec(mem, lds, prog)
+        ex = Exec(mem, lds, prog, strict=strict)
         waves = []
         for wi in range(nwaves):
             w = Wave()
+            w.wid = wi
             w.scratch_mem = np.zeros((64, max(priv, 0)), dtype=np.uint8)
             # user SGPRs in the ABI's order; only the ones HIP kernels for this target ask for are modelled
             si = 0
@@ -1822,6 +2019,7 @@ def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, 
             if all(w.done or w.at_barrier for w in waves):
                 for w in waves:
                     w.at_barrier = False
+                ex.barrier_released()
                 continue
             if not progressed:
                 raise EmuError("workgroup %r makes no progress" % (g,))

@@ -17,6 +17,28 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
 
 
+def _plant(kernel_part, what):
+    import gcn_emu as E
+    parse = E.parse_program
+
+    def mutated(text, name, exact=False):
+        prog = parse(text, name, exact)
+        if kernel_part in name:
+            n = 0
+            for ins in prog.instrs:
+                if ins.wait is not None:
+                    key = {"vm+1": "vmcnt", "lgkm+1": "lgkmcnt"}.get(what)
+                    if key and ins.wait.get(key, 0) > 0:
+                        ins.wait[key] += 1
+                        n += 1
+                elif what == "nobarrier" and ins.op == "s_barrier":
+                    ins.op = "s_nop"
+                    n += 1
+            assert n, "nothing to mutate in %s" % name
+        return prog
+    E.parse_program = mutated
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--lib", required=True)
@@ -26,10 +48,16 @@ def main():
     ap.add_argument("--shim-dir", default=tempfile.gettempdir())
     ap.add_argument("--num-cu", type=int, default=256, help="compute units the stand-in reports (the host code sizes "
                     "grids, tiles and stream-K partitions from it; the library reads it once per process)")
+    ap.add_argument("--mutate", default="", help="KERNEL_PART:WHAT, a deliberate defect planted in the parsed program of "
+                    "every kernel whose name contains KERNEL_PART, to show that the interpreter's checks see it.  WHAT: "
+                    "vm+1 / lgkm+1 (every counted wait, i.e. every non-zero count, lets one more operation stay in flight), "
+                    "nobarrier (every s_barrier becomes a no-op)")
     a = ap.parse_args()
     assert "torch" not in sys.modules
     import cases
     from device import Device, build_shim
+    if a.mutate:
+        _plant(*a.mutate.split(":"))
     dev = Device(a.lib, a.asm, build_shim(a.shim_dir))
     dev.shim.shim_set_num_cu(a.num_cu)
     # device set-up the way a binder does it (also primes the static scratch array)

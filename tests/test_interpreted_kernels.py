@@ -118,6 +118,20 @@ CASES = [
     C("mm bf16 15x160x1024 on 8 CUs", "gemm", dtype="bf16", M=15, N=160, K=1024, num_cu=8),
     C("skinny static 8x256x1024 on 8 CUs", "gemm", dtype="bf16", M=8, N=256, K=1024, b_layout="nk",
       entry="fg_gemm_skinny_static", num_cu=8, kernel="gemm_skinny_kc_kernel"),
+    # (long K on few CUs: every workgroup stays in the main loop, whose waits are counted by hand, for many trips)
+    C("mm bf16 skinny 4x128x4096 on 8 CUs", "gemm", dtype="bf16", M=4, N=128, K=4096, b_layout="nk", num_cu=8,
+      kernel="gemm_skinny_kc_kernelIDF16bLi16ELi8ELb0ELi1E"),
+    C("addmm f16 skinny 12x128x4096 on 8 CUs", "gemm", dtype="f16", M=12, N=128, K=4096, b_layout="nk", bias="row", num_cu=8,
+      kernel="gemm_skinny_kc_kernelIDF16_Li16ELi8ELb1ELi1E"),
+    C("mm bf16 skinny 24x112x4096 on 8 CUs", "gemm", dtype="bf16", M=24, N=112, K=4096, b_layout="nk", num_cu=8,
+      kernel="gemm_skinny_kc_kernelIDF16bLi16ELi8ELb1ELi2E"),
+    C("mm bf16 skinny 4x256x8192 on 4 CUs", "gemm", dtype="bf16", M=4, N=256, K=8192, b_layout="nk", num_cu=4,
+      kernel="gemm_skinny_kc_kernelIDF16bLi32ELi4ELb0ELi1E"),
+    C("mm bf16 skinny 64x128x4096 on 4 CUs", "gemm", dtype="bf16", M=64, N=128, K=4096, b_layout="nk", num_cu=4,
+      kernel="gemm_skinny_kc_kernelIDF16bLi32ELi4ELb1ELi4E"),
+    C("mm bf16 skinny 8x512x4096 row-major B on 4 CUs", "gemm", dtype="bf16", M=8, N=512, K=4096, num_cu=4,
+      kernel="gemm_skinny_kernel"),
+    C("mm bf16 W^T 256x256x1024 on 4 CUs", "gemm", dtype="bf16", M=256, N=256, K=1024, b_layout="nk", num_cu=4),
     C("bmm bf16 3x40x48x64", "bmm", dtype="bf16", batch=3, M=40, N=48, K=64),
     # ---- attention over the paged cache
     C("attention bf16 D128 causal 70/70 33/97", "attention", dtype="bf16", q_lens=[70, 33], k_lens=[70, 97], Hq=4, Hk=2, D=128,
@@ -388,3 +402,49 @@ def test_interpreted(runs, build, case):
     if want:
         assert any(want in k for k in kernels), "expected a %s launch, got %s" % (want, kernels)
     CHECK[case["check"]](r, case["kw"])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The checks have teeth: a defect planted in the parsed program (never in the library) is reported.
+# ---------------------------------------------------------------------------------------------------------------
+MUTATIONS = [
+    # (build, CU count, kernel, defect, case, what the interpreter must say)
+    ("default", 4, "gemm_dma_kernel", "vm+1", C("m", "gemm", dtype="bf16", M=512, N=512, K=256, b_layout="nk"),
+     "while an LDS-DMA of wave"),
+    ("default", 4, "gemm_dma_kernel", "nobarrier", C("m", "gemm", dtype="bf16", M=512, N=512, K=256, b_layout="nk"),
+     "with no barrier in between"),
+    ("variants", 8, "gemm_skinny_kc", "vm+1", C("m", "gemm", dtype="bf16", M=4, N=128, K=4096, b_layout="nk"),
+     "is the destination of a load still in flight"),
+    ("default", 256, "attn_varlen_pipe", "lgkm+1", C("m", "attention", dtype="bf16", q_lens=[70], k_lens=[200], Hq=2, Hk=2, D=128,
+                                                      page_size=16), "is the destination of a load still in flight"),
+    ("default", 256, "attn_varlen_pipe", "vm+1", C("m", "attention", dtype="bf16", q_lens=[70], k_lens=[200], Hq=2, Hk=2, D=128,
+                                                    page_size=16), "while an LDS-DMA of wave"),
+    ("default", 256, "attn_decode", "nobarrier", C("m", "attention", dtype="bf16", q_lens=[1, 1], k_lens=[300, 40], Hq=8, Hk=2,
+                                                    D=128, page_size=16), "no barrier in between"),
+]
+
+
+@pytest.mark.parametrize("build,num_cu,kernel,defect,case,message", MUTATIONS,
+                         ids=["%s %s %s" % (m[0], m[2], m[3]) for m in MUTATIONS])
+def test_planted_defects_are_reported(tmp_path, build, num_cu, kernel, defect, case, message):
+    sys.path.insert(0, CSRC)
+    try:
+        import build as B
+    finally:
+        sys.path.remove(CSRC)
+    lib, asm = (B.OUT, B.OBJ_DIR) if build == "default" else (os.path.join(os.path.dirname(B.OUT), "libfg_mi355.cand.so"),
+                                                               B.OBJ_DIR + "_cand")
+    if not os.path.exists(lib):
+        lib = B.build(verbose=False, variants=VARIANTS, tag="cand")
+    spec, out = str(tmp_path / "spec.json"), str(tmp_path / "out.npz")
+    with open(spec, "w") as f:
+        json.dump([{k: case[k] for k in ("id", "fn", "kw", "seed")}], f)
+    env = dict(os.environ)
+    env.pop("FG_LIB_PATH", None)
+    p = subprocess.run([sys.executable, os.path.join(EMU, "worker.py"), "--lib", lib, "--asm", asm, "--spec", spec, "--out", out,
+                        "--shim-dir", str(tmp_path), "--num-cu", str(num_cu), "--mutate", "%s:%s" % (kernel, defect)],
+                       capture_output=True, text=True, env=env, timeout=600)
+    assert p.returncode == 0, p.stdout[-2000:] + p.stderr[-2000:]
+    r = Result(np.load(out), "m")
+    assert "__error" in r, "the planted defect went unnoticed"
+    assert message in str(r["__error"]), str(r["__error"])[:600]
