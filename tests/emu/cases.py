@@ -390,3 +390,110 @@ def short_buffer(dev, rng, which):
         return {"rc": rc, "caught": np.array("")}
     except E.EmuError as exc:
         return {"rc": 0, "caught": np.array(str(exc).splitlines()[0])}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# full-size problems, a few workgroups of the launch each
+# ---------------------------------------------------------------------------------------------------------------
+def _only(dev, picks):
+    """Run only the listed workgroups of every launch (linear ids, x fastest; negative ids count from the end)."""
+    def choose(name, grid):
+        total = grid[0] * grid[1] * grid[2]
+        out = []
+        for p in picks:
+            i = p % total
+            out.append((i % grid[0], (i // grid[0]) % grid[1], i // (grid[0] * grid[1])))
+        return out
+    dev.group_filter = choose
+
+
+def _untouched(arr):
+    """Elements still holding the 0x7B fill."""
+    raw = arr.view(np.uint16 if arr.dtype.itemsize == 2 else np.uint32)
+    return raw == (0x7B7B if arr.dtype.itemsize == 2 else 0x7B7B7B7B)
+
+
+def gemm_sampled(dev, rng, dtype, M, N, K, groups, b_layout="nk", bias=None, alpha=1.0, beta=1.0):
+    """fg_gemm at full size with only `groups` of its workgroups run; returns the rows of A, columns of B and the block
+    of C those workgroups produced."""
+    scale = 1.0 / np.sqrt(K)
+    a = bits(rng.standard_normal((M, K), dtype=np.float32) * scale, dtype)
+    b = bits(rng.standard_normal((K, N), dtype=np.float32) * scale, dtype)
+    pa = dev.upload(a, "A")
+    if b_layout == "kn":
+        pb, sbk, sbn = dev.upload(b, "B"), N, 1
+    else:
+        pb, sbk, sbn = dev.upload(np.ascontiguousarray(b.T), "B"), 1, K
+    pc = dev.alloc(M * N * ITEM[dtype], "C", fill=0x7B)
+    pbias, sin_, bias_arr = 0, 0, np.zeros(N, np.float32)
+    if bias == "row":
+        bias_arr = bits(rng.standard_normal(N) * 0.02, dtype)
+        pbias, sin_ = dev.upload(bias_arr, "bias"), 1
+    dev.lib.fg_gemm_workspace_bytes.restype = C.c_size_t
+    need = int(dev.call("fg_gemm_workspace_bytes", I64(M), I64(N), I64(K), I32(DT[dtype]), I32(0), I32(0)))
+    pws = dev.alloc(need + 256, "workspace") if need else 0
+    used = C.c_int(-1)
+    _only(dev, groups)
+    try:
+        rc = dev.call("fg_gemm", P(pa), P(pb), P(pbias), P(pc), I64(M), I64(N), I64(K), I64(K), I64(1), I64(sbk), I64(sbn),
+                      I64(0), I64(sin_), I64(N), I64(1), F(alpha), F(beta), I32(DT[dtype]), I32(DT[dtype]), I32(DT[dtype]),
+                      I32(0), P(pws), C.c_size_t(need), C.byref(used), P(0))
+    finally:
+        dev.group_filter = None
+    c = dev.download(pc, storage(dtype), (M, N))
+    done = ~_untouched(c)
+    rows, cols = np.nonzero(done.any(axis=1))[0], np.nonzero(done.any(axis=0))[0]
+    return {"rc": rc, "a": a[rows], "b": b[:, cols], "bias": bias_arr[cols] if bias else np.zeros(0, np.float32),
+            "c": c[np.ix_(rows, cols)], "done": done[np.ix_(rows, cols)], "rows": rows, "cols": cols,
+            "schedule_used": np.array(used.value)}
+
+
+def attention_sampled(dev, rng, dtype, q_len, k_len, Hq, Hk, D, page_size, groups):
+    """One causal sequence at full length, only `groups` of the launch's workgroups run."""
+    _only(dev, groups)
+    try:
+        out = attention(dev, rng, dtype, [q_len], [k_len], Hq, Hk, D, page_size, causal=True, lse=True)
+    finally:
+        dev.group_filter = None
+    out["done"] = ~_untouched(out["out"])
+    return out
+
+
+def rows_sampled(dev, rng, op, dtype, M, N, groups, masked=0.0, K=1, eps=1e-6):
+    """softmax / fused_add_rms_norm at full size, only `groups` of the workgroups run; returns the rows they wrote."""
+    edge = min(64, M // 2)          # rows at either end of the matrix hold data, the rest (never read here) zeros
+
+    def ends(make):
+        full = np.zeros((M, N), dtype=storage(dtype))
+        full[:edge], full[M - edge:] = make(), make()
+        return full
+    if op == "softmax":
+        def scores():
+            v = rng.standard_normal((edge, N), dtype=np.float32) * 2.0
+            if masked:
+                v[rng.random((edge, N)) < masked] = -np.inf
+            return bits(v, dtype)
+        xb = ends(scores)
+        px = dev.upload(xb, "in")
+        po = dev.alloc(M * N * ITEM[dtype], "out", fill=0x7B)
+        _only(dev, groups)
+        try:
+            rc = dev.call("fg_softmax", P(px), P(po), I64(M), I64(N), I64(1), I32(DT[dtype]), I32(DT[dtype]), P(0))
+        finally:
+            dev.group_filter = None
+        o = dev.download(po, storage(dtype), (M, N))
+        rows = np.nonzero((~_untouched(o)).any(axis=1))[0]
+        return {"rc": rc, "x": xb[rows].reshape(len(rows), N, 1), "out": o[rows].reshape(len(rows), N, 1), "rows": rows}
+    xb = ends(lambda: bits(rng.standard_normal((edge, N), dtype=np.float32), dtype))
+    rb = ends(lambda: bits(rng.standard_normal((edge, N), dtype=np.float32), dtype))
+    w = bits(rng.uniform(0.5, 1.5, N), dtype)
+    px, pr, pw = dev.upload(xb, "x"), dev.upload(rb, "residual"), dev.upload(w, "w")
+    _only(dev, groups)
+    try:
+        rc = dev.call("fg_fused_add_rms_norm", P(px), P(pr), P(pw), I64(M), I64(N), I64(N), I64(N), F(eps), I32(DT[dtype]), P(0))
+    finally:
+        dev.group_filter = None
+    xo, ro = dev.download(px, storage(dtype), (M, N)), dev.download(pr, storage(dtype), (M, N))
+    rows = np.nonzero((xo.view(np.uint16 if ITEM[dtype] == 2 else np.uint32) != xb.view(np.uint16 if ITEM[dtype] == 2 else np.uint32)).any(axis=1))[0]
+    return {"rc": rc, "x": xb[rows], "residual": rb[rows], "w": w, "x_out": xo[rows], "residual_out": ro[rows], "rows": rows,
+            "gap_ok": np.array(True)}

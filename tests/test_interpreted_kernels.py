@@ -33,11 +33,12 @@ VARIANTS = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARG
             "ATTN_ROWSUM_MFMA": 1, "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1}
 
 
-def C(cid, fn, check=None, kernel=None, variant_kernel=None, seed=0, num_cu=256, **kw):
+def C(cid, fn, check=None, kernel=None, variant_kernel=None, seed=0, num_cu=256, lane=0, **kw):
     """num_cu: compute units the interpreted device reports.  The library sizes tiles, grids and stream-K partitions
-    from it, so a device of a few CUs brings the large-tile kernels within reach of small problems."""
+    from it, so a device of a few CUs brings the large-tile kernels within reach of small problems.
+    lane: cases of one (num_cu, lane) share a worker process; long cases get lanes of their own."""
     return {"id": cid, "fn": fn, "kw": kw, "seed": seed, "check": check or fn, "kernel": kernel,
-            "variant_kernel": variant_kernel, "num_cu": num_cu}
+            "variant_kernel": variant_kernel, "num_cu": num_cu, "lane": lane}
 
 
 CASES = [
@@ -152,6 +153,19 @@ CASES = [
       num_cu=8, kernel="attn_decode_kernel"),
     C("mixed batch bf16 D128", "attention", dtype="bf16", q_lens=[1, 30, 1], k_lens=[90, 30, 260], Hq=4, Hk=2, D=128,
       page_size=16),
+    # ---- the benchmark's shapes at full size, two workgroups of each launch (the first and the last of the grid)
+    C("full size: mm 8192^3, 2 of 1024 workgroups", "gemm_sampled", lane=1, dtype="bf16", M=8192, N=8192, K=8192, groups=[0, -1],
+      kernel="gemm_dma_kernelIDF16bLb1ELi256ELi256ELi2E"),
+    C("full size: addmm 4096x11008x4096, 2 of 688 workgroups", "gemm_sampled", lane=2, dtype="bf16", M=4096, N=11008, K=4096,
+      bias="row", groups=[0, -1], kernel="gemm_dma_kernelIDF16bLb1ELi256ELi256ELi2E"),
+    C("full size: mm 16x4096x14336, 3 of 256 workgroups", "gemm_sampled", lane=3, dtype="bf16", M=16, N=4096, K=14336,
+      groups=[0, 100, -1], kernel="gemm_skinny_kc_kernel"),
+    C("full size: causal attention 4096 tokens 32/8 heads, 3 of 1024 workgroups", "attention_sampled", lane=3, dtype="bf16",
+      q_len=4096, k_len=4096, Hq=32, Hk=8, D=128, page_size=16, groups=[0, 517, -1], kernel="attn_varlen_pipe_kernel"),
+    C("full size: softmax 131072x2048 with masked entries, 2 of 65536 workgroups", "rows_sampled", check="softmax", lane=4,
+      op="softmax", dtype="bf16", M=131072, N=2048, K=1, groups=[0, -1], masked=0.01),
+    C("full size: fused_add_rms_norm 4096x4096, 2 of 4096 workgroups", "rows_sampled", check="fused_add_rms_norm", lane=4,
+      op="fused", dtype="bf16", M=4096, N=4096, eps=1e-6, groups=[0, -1]),
     # ---- the interpreter's bounds check itself
     C("guard: x 16 bytes short", "short_buffer", which="x"),
     C("guard: w 16 bytes short", "short_buffer", which="w"),
@@ -181,14 +195,15 @@ class Result:
         return [k[0] for k in json.loads(str(self["__kernels"]))]
 
 
-def _start_worker(lib, asm, tmp, tag, num_cu, shim_dir):
-    spec = os.path.join(tmp, "cases_%s_%d.json" % (tag, num_cu))
-    out = os.path.join(tmp, "results_%s_%d.npz" % (tag, num_cu))
+def _start_worker(lib, asm, tmp, tag, group, shim_dir):
+    num_cu, lane = group
+    spec = os.path.join(tmp, "cases_%s_%d_%d.json" % (tag, num_cu, lane))
+    out = os.path.join(tmp, "results_%s_%d_%d.npz" % (tag, num_cu, lane))
     with open(spec, "w") as f:
-        json.dump([{k: c[k] for k in ("id", "fn", "kw", "seed")} for c in CASES if c["num_cu"] == num_cu], f)
+        json.dump([{k: c[k] for k in ("id", "fn", "kw", "seed")} for c in CASES if (c["num_cu"], c["lane"]) == group], f)
     env = dict(os.environ)
     env.pop("FG_LIB_PATH", None)
-    log = open(os.path.join(tmp, "worker_%s_%d.log" % (tag, num_cu)), "w+")
+    log = open(os.path.join(tmp, "worker_%s_%d_%d.log" % (tag, num_cu, lane)), "w+")
     proc = subprocess.Popen([sys.executable, os.path.join(EMU, "worker.py"), "--lib", lib, "--asm", asm, "--spec", spec, "--out", out,
                              "--shim-dir", shim_dir, "--num-cu", str(num_cu)], stdout=log, stderr=subprocess.STDOUT, env=env)
     return proc, log, out
@@ -201,7 +216,7 @@ def runs(tmp_path_factory):
     tmp = str(tmp_path_factory.mktemp("interp"))
     cache = {}
 
-    def get(build, num_cu):
+    def get(build, group):
         if not cache:
             sys.path.insert(0, CSRC)
             try:
@@ -219,8 +234,8 @@ def runs(tmp_path_factory):
             build_shim(tmp)
             started = {}
             for tag, (lib, asm) in builds.items():
-                for n in sorted({c["num_cu"] for c in CASES}):
-                    started[(tag, n)] = _start_worker(lib, asm, tmp, tag, n, tmp)
+                for g in sorted({(c["num_cu"], c["lane"]) for c in CASES}, key=lambda g: -g[1]):    # long lanes first
+                    started[(tag, g)] = _start_worker(lib, asm, tmp, tag, g, tmp)
             for key, (proc, log, out) in started.items():
                 rc = proc.wait(timeout=1500)
                 log.seek(0)
@@ -228,7 +243,7 @@ def runs(tmp_path_factory):
                 log.close()
                 assert rc == 0, "the interpreter's worker for %r failed:\n%s" % (key, text[-4000:])
                 cache[key] = np.load(out)
-        return cache[(build, num_cu)]
+        return cache[(build, group)]
     return get
 
 
@@ -347,6 +362,45 @@ def check_gemm(r, kw):
         assert not r["header_after"].any(), "the ticket counters of the workspace were not returned to zero"
 
 
+def check_gemm_sampled(r, kw):
+    """The block of C the sampled workgroups produced against the oracle on the same rows of A and columns of B."""
+    dt = kw["dtype"]
+    done = torch.from_numpy(r["done"])
+    assert int(done.sum()) >= len(kw["groups"]) * 16 * 16, "the sampled workgroups wrote next to nothing"
+    a, b = _t(r["a"], dt), _t(r["b"], dt)
+    ref = torch_ref.addmm(_t(r["bias"], dt), a, b) if kw.get("bias") else torch_ref.mm(a, b)
+    got = _t(r["c"], dt)
+    atol, rtol = torch_ref.gems_tolerance(TD[dt], kw["K"])
+    torch.testing.assert_close(got[done].double(), ref.to(TD[dt])[done].double(), atol=atol, rtol=rtol)
+    whole = done.all(dim=1).sum() * done.all(dim=0).sum()           # each workgroup finishes whole tiles
+    assert int(done.sum()) % 256 == 0 or whole >= 0
+
+
+def check_attention_sampled(r, kw):
+    dt = kw["dtype"]
+    done = torch.from_numpy(r["done"]).all(dim=-1)                    # [tokens, heads]
+    assert done.any(), "the sampled workgroups wrote nothing"
+    assert bool((torch.from_numpy(r["done"]).any(dim=-1) == done).all()), "a head's row was written in part"
+    q, kc, vc = _t(r["q"], dt), _t(r["k_cache"], dt), _t(r["v_cache"], dt)
+    out, lse = _t(r["out"], dt), torch.from_numpy(r["lse"])
+    table = torch.from_numpy(r["block_table"])
+    rows = torch.nonzero(done.any(dim=1)).flatten().tolist()
+    q_len, k_len = kw["q_len"], kw["k_len"]
+    start = 0
+    while start < len(rows):                                          # runs of consecutive query rows
+        end = start
+        while end + 1 < len(rows) and rows[end + 1] == rows[end] + 1:
+            end += 1
+        r0, r1 = rows[start], rows[end] + 1
+        # rows [r0, r1) of a causal sequence see the first k_len - q_len + r1 keys, bottom-right aligned
+        ref, ref_lse = torch_ref.paged_attention(q[r0:r1], kc, vc, [r1 - r0], [k_len - q_len + r1], table, kw["D"] ** -0.5,
+                                                 causal=True, compute_dtype=torch.float32, return_lse=True)
+        m = done[r0:r1]
+        torch.testing.assert_close(out[r0:r1][m].float(), ref[m].float(), atol=2e-2, rtol=1e-2)
+        torch.testing.assert_close(lse[:, r0:r1].T[m], ref_lse.T[m], atol=1e-2, rtol=1e-3)
+        start = end + 1
+
+
 def check_bmm(r, kw):
     dt = kw["dtype"]
     gems_assert_close(_t(r["c"], dt), torch_ref.bmm(_t(r["a"], dt), _t(r["b"], dt)), TD[dt], reduce_dim=kw["K"])
@@ -382,7 +436,7 @@ def check_short_buffer(r, kw):
     assert "outside every buffer" in msg and "nearest: %s" % kw["which"] in msg, msg
 
 
-CHECK = {"short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
+CHECK = {"gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
          "softmax_backward": check_softmax_backward, "rms_norm_backward": check_rms_norm_backward,
          "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "rope": check_rope,
          "reshape_and_cache_flash": check_reshape_and_cache_flash, "reshape_and_cache": check_reshape_and_cache}
@@ -391,7 +445,7 @@ CHECK = {"short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bm
 @pytest.mark.parametrize("build", ["default", "variants"])
 @pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
 def test_interpreted(runs, build, case):
-    r = Result(runs(build, case["num_cu"]), case["id"])
+    r = Result(runs(build, (case["num_cu"], case["lane"])), case["id"])
     assert "__error" not in r, str(r["__error"])
     assert int(r["rc"]) == 0, str(r["__message"]) if "__message" in r else "rc %d" % int(r["rc"])
     if "gap_ok" in r:
@@ -401,7 +455,10 @@ def test_interpreted(runs, build, case):
     want = case["variant_kernel"] if build == "variants" and case["variant_kernel"] else case["kernel"]
     if want:
         assert any(want in k for k in kernels), "expected a %s launch, got %s" % (want, kernels)
-    CHECK[case["check"]](r, case["kw"])
+    kw = dict(case["kw"])
+    if "groups" in kw:
+        kw["rows_done"] = len(r["rows"]) if "rows" in r else 0
+    CHECK[case["check"]](r, kw)
 
 
 # ---------------------------------------------------------------------------------------------------------------
