@@ -1685,6 +1685,12 @@ def _valu_more(ex, w, ins, V):
              "lshlrev": lambda: b << (a & U32(15)), "lshrrev": lambda: b >> (a & U32(15)), "max": lambda: np.maximum(a, b),
              "min": lambda: np.minimum(a, b)}[m.group(1)]()
         return V.dst(ops[0], "u16", r & U32(0xFFFF))
+    if base == "v_pack_b32_f16":
+        sel = [int(x) for x in mods["op_sel"].strip("[]").split(",")] if "op_sel" in mods else [0, 0, 0]
+        a, b = V.raw(ops[1], 0, 32, "f16")[0], V.raw(ops[2], 1, 32, "f16")[0]
+        lo = (a >> U32(16 if sel[0] else 0)) & U32(0xFFFF)
+        hi = (b >> U32(16 if sel[1] else 0)) & U32(0xFFFF)
+        return V.dst(ops[0], "u32", lo | (hi << U32(16)))
     if base == "v_mad_i32_i24":
         a = ((V.src(ops[1], 0, "u32") << U32(8)).view(np.int32) >> 8).astype(np.int64)
         b = ((V.src(ops[2], 1, "u32") << U32(8)).view(np.int32) >> 8).astype(np.int64)

@@ -71,7 +71,12 @@ def main():
         rng = np.random.default_rng(spec.get("seed", 0))
         dev.launches.clear()
         t0 = time.time()
+        env = spec.get("env") or {}
         try:
+            for k, v in env.items():            # the library's FG_* switches, read again for this case
+                os.environ[k] = v
+            if env:
+                dev.lib.fg_reload_options()
             res = getattr(cases, spec["fn"])(dev, rng, **spec["kw"])
             for k, v in res.items():
                 out["%s|%s" % (cid, k)] = np.asarray(v)
@@ -79,6 +84,11 @@ def main():
                 out["%s|__message" % cid] = np.array(dev.last_error())
         except Exception as exc:
             out["%s|__error" % cid] = np.array("%s\n%s" % (exc, traceback.format_exc()))
+        finally:
+            for k in env:
+                del os.environ[k]
+            if env:
+                dev.lib.fg_reload_options()
         out["%s|__kernels" % cid] = np.array(json.dumps([[n, list(g), list(b), s, st] for n, g, b, s, st in dev.launches]))
         out["%s|__seconds" % cid] = np.array(time.time() - t0)
         print("%-50s %6.1fs %s" % (cid, time.time() - t0, "ERROR" if ("%s|__error" % cid) in out else ""), flush=True)

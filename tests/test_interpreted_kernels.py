@@ -173,6 +173,20 @@ CASES = [
 ]
 
 
+# Bulk cases, one per dispatch bucket (tests/emu/sweep.py), for the build with the variants on: together with the
+# cases above they execute every kernel of that build whose code differs from the GPU-tested build
+# (test_every_changed_kernel_has_run).  The default build does not run them: its kernels have the GPU suite behind them.
+sys.path.insert(0, EMU)
+try:
+    import sweep as _sweep
+finally:
+    sys.path.remove(EMU)
+SWEEP = _sweep.sweep()
+for _i, _c in enumerate(SWEEP):
+    _c.update(kernel=None, variant_kernel=None, lane=10 + (_i % 6 if _c["num_cu"] == 256 else 0))
+PARAMS = [(b, c) for c in CASES for b in ("default", "variants")] + [("variants", c) for c in SWEEP]
+
+
 def _t(arr, dtype):
     """Array as the worker stored it -> torch tensor of `dtype`."""
     arr = np.ascontiguousarray(arr)
@@ -200,7 +214,8 @@ def _start_worker(lib, asm, tmp, tag, group, shim_dir):
     spec = os.path.join(tmp, "cases_%s_%d_%d.json" % (tag, num_cu, lane))
     out = os.path.join(tmp, "results_%s_%d_%d.npz" % (tag, num_cu, lane))
     with open(spec, "w") as f:
-        json.dump([{k: c[k] for k in ("id", "fn", "kw", "seed")} for c in CASES if (c["num_cu"], c["lane"]) == group], f)
+        json.dump([{k: c.get(k) for k in ("id", "fn", "kw", "seed", "env")} for b, c in PARAMS
+                   if b == tag and (c["num_cu"], c["lane"]) == group], f)
     env = dict(os.environ)
     env.pop("FG_LIB_PATH", None)
     log = open(os.path.join(tmp, "worker_%s_%d_%d.log" % (tag, num_cu, lane)), "w+")
@@ -233,9 +248,18 @@ def runs(tmp_path_factory):
             builds = {"default": (B.OUT, B.OBJ_DIR), "variants": (cand, B.OBJ_DIR + "_cand")}
             build_shim(tmp)
             started = {}
-            for tag, (lib, asm) in builds.items():
-                for g in sorted({(c["num_cu"], c["lane"]) for c in CASES}, key=lambda g: -g[1]):    # long lanes first
-                    started[(tag, g)] = _start_worker(lib, asm, tmp, tag, g, tmp)
+            todo = sorted({(b, (c["num_cu"], c["lane"])) for b, c in PARAMS}, key=lambda t: (-t[1][1], t[0]))   # long lanes first
+            running = []
+            width = max(2, min(8, os.cpu_count() or 2))               # worker processes side by side
+            while todo or running:
+                while todo and len(running) < width:
+                    tag, g = todo.pop(0)
+                    started[(tag, g)] = _start_worker(builds[tag][0], builds[tag][1], tmp, tag, g, tmp)
+                    running.append(started[(tag, g)][0])
+                running = [p for p in running if p.poll() is None]
+                if todo or running:
+                    import time
+                    time.sleep(0.2)
             for key, (proc, log, out) in started.items():
                 rc = proc.wait(timeout=1500)
                 log.seek(0)
@@ -288,8 +312,12 @@ def check_softmax_backward(r, kw):
 def check_rms_norm_backward(r, kw):
     dt = kw["dtype"]
     x, dy, w = _t(r["x"], dt), _t(r["dy"], dt), _t(r["w"], dt)
+    if not kw.get("weight", True):
+        w = torch.ones_like(w)
     dx, dw = torch_ref.rms_norm_grads(x, w, kw.get("eps", 1e-5), dy)
     gems_assert_close(_t(r["dx"], dt), dx, TD[dt])
+    if not kw.get("dw", True):
+        return
     assert int(r["rc_dw"]) == 0
     gems_assert_close(_t(r["dw"], dt), dw, TD[dt], reduce_dim=kw["M"])
     # the partial rows add up to the weight gradient before rounding
@@ -442,8 +470,7 @@ CHECK = {"gemm_sampled": check_gemm_sampled, "attention_sampled": check_attentio
          "reshape_and_cache_flash": check_reshape_and_cache_flash, "reshape_and_cache": check_reshape_and_cache}
 
 
-@pytest.mark.parametrize("build", ["default", "variants"])
-@pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
+@pytest.mark.parametrize("build,case", PARAMS, ids=["%s-%s" % (c["id"], b) for b, c in PARAMS])
 def test_interpreted(runs, build, case):
     r = Result(runs(build, (case["num_cu"], case["lane"])), case["id"])
     assert "__error" not in r, str(r["__error"])
@@ -505,3 +532,45 @@ def test_planted_defects_are_reported(tmp_path, build, num_cu, kernel, defect, c
     r = Result(np.load(out), "m")
     assert "__error" in r, "the planted defect went unnoticed"
     assert message in str(r["__error"]), str(r["__error"])[:600]
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Coverage: no kernel whose code differs from the GPU-tested build is left unexecuted.
+# ---------------------------------------------------------------------------------------------------------------
+# Instantiations no call can reach.  rms_dispatch picks (packs per thread, threads per row) in two run-time branches, one
+# for rms_norm and one for fused_add_rms_norm, so the compiler instantiates every pair for both operators although
+# each operator only ever launches its own; the two-row kernel is launched for the fused operator only.
+UNREACHABLE = [
+    r"rms_rows_kernelI\w+Li[48]ELi1ELi(128|256|512|1024)ELb0E",      # rms_norm never takes one pack per thread beyond 64 threads
+    r"rms_rows_kernelI\w+Li[48]ELi2ELi(64|128|256|512)ELb1E",        # fused_add_rms_norm takes two packs only on 1024 threads
+    r"rms_rows2_kernelI\w+ELb0E",                                    # rms_norm has no row length with one pack on >= 256 threads
+]
+
+
+def test_every_changed_kernel_has_run(runs):
+    import glob
+    import re
+    sys.path.insert(0, CSRC)
+    try:
+        import build as B
+        import isa_check
+    finally:
+        sys.path.remove(CSRC)
+    digests = {}
+    for tag, d in (("default", B.OBJ_DIR), ("variants", B.OBJ_DIR + "_cand")):
+        digests[tag] = {}
+        for f in glob.glob(os.path.join(d, "*-hip-amdgcn-amd-amdhsa-gfx950.s")):
+            with open(f) as fh:
+                digests[tag].update(isa_check.kernel_digests(fh.read()))
+    changed = {k for k, v in digests["variants"].items() if digests["default"].get(k) != v}
+    assert len(changed) > 400, "the variants build hardly differs from the default one: %d kernels" % len(changed)
+    ran = set()
+    for group in {(c["num_cu"], c["lane"]) for b, c in PARAMS if b == "variants"}:
+        npz = runs("variants", group)
+        for key in npz.files:
+            if key.endswith("|__kernels"):
+                ran.update(k[0] for k in json.loads(str(npz[key])))
+    unreachable = {k for k in changed if any(re.search(p, k) for p in UNREACHABLE)}
+    assert not (unreachable & ran), "listed as unreachable, yet launched: %s" % sorted(unreachable & ran)
+    missing = sorted(changed - ran - unreachable)
+    assert not missing, "%d changed kernels were never executed, e.g. %s" % (len(missing), missing[:5])
