@@ -187,11 +187,31 @@ _FLAGS = {"off", "glc", "slc", "nt", "sc0", "sc1", "lds", "clamp", "gds", "row_m
           "vmcnt", "idxen", "offen"}
 
 
+_FILE_CACHE = {}
+
+
+def _file_index(text):
+    """Per assembly text, parsed once: kernel bodies, kernel descriptors and the metadata records by kernel name."""
+    key = (len(text), hash(text))
+    if key not in _FILE_CACHE:
+        bodies = {k.group(1): k.group(2) for k in _KERNEL.finditer(text)}
+        kds = {m.group(1): m.group(2) for m in re.finditer(r"\.amdhsa_kernel (\S+)\n(.*?)\.end_amdhsa_kernel", text, re.S)}
+        metas = {}
+        mm = re.search(r"\.amdgpu_metadata\n---\n(.*?)\n\.\.\.\n", text, re.S)
+        if mm:
+            loader = getattr(yaml, "CSafeLoader", yaml.SafeLoader)
+            for k in yaml.load(mm.group(1), Loader=loader)["amdhsa.kernels"]:
+                metas[k[".name"]] = k
+        _FILE_CACHE[key] = (bodies, kds, metas)
+    return _FILE_CACHE[key]
+
+
 def parse_program(text, name_part, exact=False):
-    km = [k for k in _KERNEL.finditer(text) if (name_part == k.group(1) if exact else name_part in k.group(1))]
+    bodies, kds, metas = _file_index(text)
+    km = [k for k in bodies if (name_part == k if exact else name_part in k)]
     if len(km) != 1:
         raise EmuError("%d kernels match %r" % (len(km), name_part))
-    name, body = km[0].group(1), km[0].group(2)
+    name, body = km[0], bodies[km[0]]
     instrs, labels = [], {}
     for raw in body.splitlines():
         line = raw.split(";")[0].strip()
@@ -244,19 +264,12 @@ def parse_program(text, name_part, exact=False):
         instrs.append(Instr(op, ops, mods, line))
     # kernel descriptor and metadata
     kd = {}
-    m = re.search(r"\.amdhsa_kernel %s\n(.*?)\.end_amdhsa_kernel" % re.escape(name), text, re.S)
-    if m:
-        for k, v in re.findall(r"\.amdhsa_(\w+) (\S+)", m.group(1)):
-            try:
-                kd[k] = int(v, 0)
-            except ValueError:
-                kd[k] = v
-    meta = {}
-    mm = re.search(r"\.amdgpu_metadata\n---\n(.*?)\n\.\.\.\n", text, re.S)
-    if mm:
-        for k in yaml.safe_load(mm.group(1))["amdhsa.kernels"]:
-            if k[".name"] == name:
-                meta = k
+    for k, v in re.findall(r"\.amdhsa_(\w+) (\S+)", kds.get(name, "")):
+        try:
+            kd[k] = int(v, 0)
+        except ValueError:
+            kd[k] = v
+    meta = metas.get(name, {})
     return Program(name, instrs, labels, kd, meta)
 
 

@@ -173,9 +173,9 @@ CASES = [
 ]
 
 
-# Bulk cases, one per dispatch bucket (tests/emu/sweep.py), for the build with the variants on: together with the
-# cases above they execute every kernel of that build whose code differs from the GPU-tested build
-# (test_every_changed_kernel_has_run).  The default build does not run them: its kernels have the GPU suite behind them.
+# Bulk cases, one per dispatch bucket (tests/emu/sweep.py).  On the build with the variants on they execute, together
+# with the cases above, every kernel whose code differs from the GPU-tested build (test_every_changed_kernel_has_run);
+# on the default build the same cases calibrate the interpreter over the same breadth of GPU-tested kernels.
 sys.path.insert(0, EMU)
 try:
     import sweep as _sweep
@@ -184,7 +184,7 @@ finally:
 SWEEP = _sweep.sweep()
 for _i, _c in enumerate(SWEEP):
     _c.update(kernel=None, variant_kernel=None, lane=10 + (_i % 6 if _c["num_cu"] == 256 else 0))
-PARAMS = [(b, c) for c in CASES for b in ("default", "variants")] + [("variants", c) for c in SWEEP]
+PARAMS = [(b, c) for c in CASES + SWEEP for b in ("default", "variants")]
 
 
 def _t(arr, dtype):
