@@ -8,8 +8,32 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# FG_INTERPRETED=1: the GPU parity tests run on the CPU, kernels executed by the interpreter of tests/emu/ (see
+# tests/emu/session.py; tests/test_interpreted_suite.py starts such runs).  The HIP stand-in has to be bound before
+# torch is imported, hence here, at the top of the first file pytest loads.
+INTERPRETED = os.environ.get("FG_INTERPRETED") == "1"
+if INTERPRETED:
+    sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
+    import session as _interp_session
+    sys.path.pop(0)
+    _interp_session.install()
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def pytest_terminal_summary(terminalreporter):
+    if INTERPRETED:
+        terminalreporter.write_line("interpreted kernel launches: %d" % _interp_session.DEVICE.total_launches)
+
+
+@pytest.fixture(autouse=INTERPRETED)
+def _interpreter_between_tests():
+    yield
+    if INTERPRETED:
+        err = _interp_session.between_tests()
+        assert err is None, "the interpreter refused a launch:\n%s" % err
 
 
 @pytest.fixture(scope="session")
@@ -17,6 +41,8 @@ def gpu():
     """cuda:0 with the native library loaded; fails (never skips) when either is missing."""
     import torch
 
+    if INTERPRETED:
+        return torch.device("cpu")
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     from flaggems_amd import _C
 

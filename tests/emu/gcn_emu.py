@@ -15,6 +15,7 @@ import numpy as np
 import yaml
 
 U32 = np.uint32
+POISON = 0x7FC07FC0
 LANES = np.arange(64, dtype=np.uint64)
 FULL = (1 << 64) - 1
 
@@ -31,7 +32,7 @@ class Memory:
 
     def __init__(self):
         self.bufs = []   # (base, np.uint8 array, name)
-        self.next = 0x7F0000000000
+        self.next = 0x4000000000000000   # far from anything the process itself maps
 
     def alloc(self, nbytes, name="buf", data=None):
         base = self.next
@@ -43,12 +44,26 @@ class Memory:
         self.next += (int(nbytes) + 0xFFFF + 0x100000) & ~0xFFFF   # a gap after every buffer
         return base
 
+    def map_external(self, base, nbytes, name="external"):
+        """Make [base, base + nbytes) of THIS process's memory a buffer (zero-copy): a tensor's storage, for instance.
+        Buffers mapped earlier that overlap it are dropped (their memory was freed and handed out again)."""
+        import ctypes
+        base, nbytes = int(base), int(nbytes)
+        if nbytes <= 0:
+            return
+        self.bufs = [b for b in self.bufs if not (len(b) > 3 and b[0] < base + nbytes and base < b[0] + b[1].size)]
+        arr = np.ctypeslib.as_array((ctypes.c_uint8 * nbytes).from_address(base))
+        self.bufs.append((base, arr, name, "external"))
+
+    def drop_externals(self):
+        self.bufs = [b for b in self.bufs if len(b) == 3]
+
     def write(self, base, raw):
         arr = self.view(base)
         arr[:len(raw)] = np.frombuffer(bytes(raw), dtype=np.uint8)
 
     def view(self, base):
-        for b, arr, _ in self.bufs:
+        for b, arr, *_ in self.bufs:
             if b == base:
                 return arr
         raise KeyError(base)
@@ -56,12 +71,12 @@ class Memory:
     def _find(self, addrs, width, what):
         addrs = np.asarray(addrs, dtype=np.uint64)
         lo, hi = int(addrs.min()), int(addrs.max())
-        for b, arr, name in self.bufs:
+        for b, arr, *_ in self.bufs:
             if b <= lo and hi + width <= b + arr.size:
                 return b, arr
         # not one buffer for all lanes: find per-lane (slow path), and report the first stray address
         for a in addrs.tolist():
-            if not any(b <= a and a + width <= b + arr.size for b, arr, _ in self.bufs):
+            if not any(b[0] <= a and a + width <= b[0] + b[1].size for b in self.bufs):
                 near = min(self.bufs, key=lambda x: abs(x[0] - a)) if self.bufs else None
                 raise EmuError("%s: %d-byte access at %#x is outside every buffer (nearest: %s at %#x, %d bytes)" % (
                     what, width, a, near[2] if near else "-", near[0] if near else 0, near[1].size if near else 0))
@@ -77,7 +92,7 @@ class Memory:
             return arr[idx]
         out = np.zeros((len(addrs), width), dtype=np.uint8)
         for i, a in enumerate(np.asarray(addrs).tolist()):
-            for bb, arr2, _ in self.bufs:
+            for bb, arr2, *_ in self.bufs:
                 if bb <= a and a + width <= bb + arr2.size:
                     out[i] = arr2[a - bb:a - bb + width]
                     break
@@ -94,7 +109,7 @@ class Memory:
             arr[idx] = data
             return
         for i, a in enumerate(np.asarray(addrs).tolist()):
-            for bb, arr2, _ in self.bufs:
+            for bb, arr2, *_ in self.bufs:
                 if bb <= a and a + width <= bb + arr2.size:
                     arr2[a - bb:a - bb + width] = data[i]
                     break
@@ -1986,6 +2001,14 @@ def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, 
     lds_size = int(kd.get("group_segment_fixed_size", 0)) + dynamic_lds
     priv = int(kd.get("private_segment_fixed_size", 0))
     nthreads = block[0] * block[1] * block[2]
+    # what the runtime would refuse at launch
+    if lds_size > 160 * 1024:
+        raise EmuError("%s: %d bytes of LDS requested, a workgroup can have 163840" % (prog.name, lds_size))
+    limit = int(prog.meta.get(".max_flat_workgroup_size", 1024))
+    if nthreads > limit or nthreads == 0:
+        raise EmuError("%s: %d work-items per workgroup, the kernel is built for at most %d" % (prog.name, nthreads, limit))
+    if min(grid) < 1 or grid[0] > 0x7FFFFFFF or grid[1] > 65535 or grid[2] > 65535:
+        raise EmuError("%s: grid %r is outside what a launch accepts" % (prog.name, grid))
     nwaves = (nthreads + 63) // 64
     tid = np.arange(nwaves * 64)
     tx, ty, tz = tid % block[0], (tid // block[0]) % block[1], tid // (block[0] * block[1])
@@ -1996,13 +2019,18 @@ def launch(prog, mem, values, grid, block, dynamic_lds=0, max_steps=50_000_000, 
     steps = 0
     all_groups = [(x, y, z) for z in range(grid[2]) for y in range(grid[1]) for x in range(grid[0])]
     for g in (groups if groups is not None else all_groups):
-        lds = np.zeros(lds_size, dtype=np.uint8)
+        # LDS and registers start out holding NaNs (0x7FC07FC0: a NaN as fp32, as two bf16 and as two fp16; as an
+        # address or index it is far outside everything): what a kernel consumes without having written it shows up
+        lds = np.tile(np.array([0xC0, 0x7F], dtype=np.uint8), (lds_size + 1) // 2)[:lds_size].copy()
         ex = Exec(mem, lds, prog, strict=strict)
         waves = []
         for wi in range(nwaves):
             w = Wave()
             w.wid = wi
-            w.scratch_mem = np.zeros((64, max(priv, 0)), dtype=np.uint8)
+            w.v[:] = U32(POISON)
+            w.s[:] = U32(POISON)
+            w.s[106:108] = 0
+            w.scratch_mem = np.full((64, max(priv, 0)), 0xFF, dtype=np.uint8)     # private memory starts as NaNs too
             # user SGPRs in the ABI's order; only the ones HIP kernels for this target ask for are modelled
             si = 0
             for name, n in (("private_segment_buffer", 4), ("dispatch_ptr", 2), ("queue_ptr", 2),

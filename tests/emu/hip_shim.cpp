@@ -36,6 +36,7 @@ struct Config {
 thread_local Config g_cfg;
 int g_num_cu = 256;
 int g_capturing = 0;
+hipError_t g_last_error = hipSuccess;  // what hipGetLastError reports next (a failed launch), as the runtime does
 }  // namespace
 
 extern "C" {
@@ -72,9 +73,10 @@ hipError_t __hipPopCallConfiguration(dim3* grid, dim3* block, size_t* shmem, hip
 }
 hipError_t hipLaunchKernel(const void* fn, dim3 grid, dim3 block, void** args, size_t shmem, hipStream_t stream) {
   auto it = functions().find(fn);
-  if (it == functions().end() || g_launch == nullptr) return hipErrorInvalidDeviceFunction;
+  if (it == functions().end() || g_launch == nullptr) return g_last_error = hipErrorInvalidDeviceFunction;
   const unsigned g[3] = {grid.x, grid.y, grid.z}, b[3] = {block.x, block.y, block.z};
-  return g_launch(it->second.c_str(), g, b, args, shmem, (void*)stream) == 0 ? hipSuccess : hipErrorLaunchFailure;
+  if (g_launch(it->second.c_str(), g, b, args, shmem, (void*)stream) != 0) return g_last_error = hipErrorLaunchFailure;
+  return hipSuccess;
 }
 hipError_t hipGetDevice(int* d) {
   *d = 0;
@@ -101,8 +103,14 @@ hipError_t hipGetDevicePropertiesR0600(hipDeviceProp_tR0600* p, int d) {
   return hipSuccess;
 }
 hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
-hipError_t hipGetLastError(void) { return hipSuccess; }
-const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "error reported by the stand-in"; }
+hipError_t hipGetLastError(void) {
+  const hipError_t e = g_last_error;
+  g_last_error = hipSuccess;
+  return e;
+}
+const char* hipGetErrorString(hipError_t e) {
+  return e == hipSuccess ? "no error" : "the interpreter refused the launch (its message is in the test's output)";
+}
 hipError_t hipGetSymbolAddress(void** ptr, const void* symbol) {
   auto it = variables().find(symbol);
   if (it == variables().end() || g_symbol == nullptr) return hipErrorInvalidSymbol;
