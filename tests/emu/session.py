@@ -53,6 +53,20 @@ def install():
         def with_device_zero(*args, _fn=getattr(handle, name)):      # a CPU tensor's device has no index
             return _fn(*[0 if a is None else a for a in args])
         setattr(handle, name, with_device_zero)
+    # hipMalloc hands out 256-byte aligned memory, which the stream-K workspace relies on; the CPU allocator promises 64
+    from flaggems_amd.ops import _gemm
+
+    class _AlignedTorch:
+        def __getattr__(self, name):
+            return getattr(torch, name)
+
+        @staticmethod
+        def empty(n, dtype=None, device=None):
+            raw = torch.empty(n + 256, dtype=dtype, device=device)
+            skip = (-real_data_ptr(raw)) % 256
+            return raw[skip:skip + n]
+
+    _gemm.torch = _AlignedTorch()
     torch.cuda.synchronize = lambda *a, **k: None
     torch.cuda.current_device = lambda: 0
     DEVICE = dev
