@@ -497,3 +497,26 @@ def rows_sampled(dev, rng, op, dtype, M, N, groups, masked=0.0, K=1, eps=1e-6):
     rows = np.nonzero((xo.view(np.uint16 if ITEM[dtype] == 2 else np.uint32) != xb.view(np.uint16 if ITEM[dtype] == 2 else np.uint32)).any(axis=1))[0]
     return {"rc": rc, "x": xb[rows], "residual": rb[rows], "w": w, "x_out": xo[rows], "residual_out": ro[rows], "rows": rows,
             "gap_ok": np.array(True)}
+
+
+def static_first_call_under_capture(dev, rng):
+    """fg_gemm_skinny_static in a process that has made no call yet: refused while the stream is being captured (the
+    lookup of the scratch array's address must not happen then), accepted eagerly, and from then on under capture too."""
+    kw = dict(dtype="bf16", M=8, N=128, K=1024, b_layout="nk", entry="fg_gemm_skinny_static")
+    out = {}
+    dev.shim.shim_set_capturing(1)
+    first = gemm(dev, rng, **kw)
+    out["rc_first_under_capture"] = np.array(first["rc"])
+    out["message"] = np.array(dev.last_error())
+    out["launches_first"] = np.array(len(dev.launches))
+    dev.shim.shim_set_capturing(0)
+    eager = gemm(dev, rng, **kw)
+    dev.shim.shim_set_capturing(1)
+    again = gemm(dev, rng, **kw)
+    dev.shim.shim_set_capturing(0)
+    out["rc"] = np.array(eager["rc"] or again["rc"])
+    for k in ("a", "b", "c"):
+        out[k], out[k + "_captured"] = eager[k], again[k]
+    out["bias"] = eager["bias"]
+    out["schedule_used"] = eager["schedule_used"]
+    return out

@@ -48,6 +48,8 @@ def main():
     ap.add_argument("--shim-dir", default=tempfile.gettempdir())
     ap.add_argument("--num-cu", type=int, default=256, help="compute units the stand-in reports (the host code sizes "
                     "grids, tiles and stream-K partitions from it; the library reads it once per process)")
+    ap.add_argument("--no-device-info", action="store_true", help="skip the fg_device_info call a binder makes at start "
+                    "(it also looks up the static scratch array): for cases about the library's first call")
     ap.add_argument("--mutate", default="", help="KERNEL_PART:WHAT, a deliberate defect planted in the parsed program of "
                     "every kernel whose name contains KERNEL_PART, to show that the interpreter's checks see it.  WHAT: "
                     "vm+1 / lgkm+1 (every counted wait, i.e. every non-zero count, lets one more operation stay in flight), "
@@ -62,9 +64,10 @@ def main():
     dev.shim.shim_set_num_cu(a.num_cu)
     # device set-up the way a binder does it (also primes the static scratch array)
     import ctypes
-    ncu, lds, arch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    rc = dev.call("fg_device_info", ctypes.c_int(0), ctypes.byref(ncu), ctypes.byref(lds), ctypes.byref(arch))
-    assert rc == 0 and arch.value == 0x950 and ncu.value == a.num_cu, (rc, arch.value, ncu.value, dev.last_error())
+    if not a.no_device_info:
+        ncu, lds, arch = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        rc = dev.call("fg_device_info", ctypes.c_int(0), ctypes.byref(ncu), ctypes.byref(lds), ctypes.byref(arch))
+        assert rc == 0 and arch.value == 0x950 and ncu.value == a.num_cu, (rc, arch.value, ncu.value, dev.last_error())
     out = {}
     for spec in json.load(open(a.spec)):
         cid = spec["id"]

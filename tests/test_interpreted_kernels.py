@@ -166,6 +166,8 @@ CASES = [
       op="softmax", dtype="bf16", M=131072, N=2048, K=1, groups=[0, -1], masked=0.01),
     C("full size: fused_add_rms_norm 4096x4096, 2 of 4096 workgroups", "rows_sampled", check="fused_add_rms_norm", lane=4,
       op="fused", dtype="bf16", M=4096, N=4096, eps=1e-6, groups=[0, -1]),
+    # ---- the entry point that allocates nothing, in a process whose first library call it is (lane 9: no fg_device_info)
+    C("static entry: first call under capture is refused, later ones are not", "static_first_call_under_capture", lane=9, num_cu=8),
     # ---- the interpreter's bounds check itself
     C("guard: x 16 bytes short", "short_buffer", which="x"),
     C("guard: w 16 bytes short", "short_buffer", which="w"),
@@ -220,7 +222,8 @@ def _start_worker(lib, asm, tmp, tag, group, shim_dir):
     env.pop("FG_LIB_PATH", None)
     log = open(os.path.join(tmp, "worker_%s_%d_%d.log" % (tag, num_cu, lane)), "w+")
     proc = subprocess.Popen([sys.executable, os.path.join(EMU, "worker.py"), "--lib", lib, "--asm", asm, "--spec", spec, "--out", out,
-                             "--shim-dir", shim_dir, "--num-cu", str(num_cu)], stdout=log, stderr=subprocess.STDOUT, env=env)
+                             "--shim-dir", shim_dir, "--num-cu", str(num_cu)] + (["--no-device-info"] if lane == 9 else []),
+                            stdout=log, stderr=subprocess.STDOUT, env=env)
     return proc, log, out
 
 
@@ -459,12 +462,20 @@ def check_attention(r, kw):
         assert (got[~finite] == float("inf")).all()      # rows with no visible key: out = 0, lse = +inf
 
 
+def check_static_first_call_under_capture(r, kw):
+    assert int(r["rc_first_under_capture"]) == -2 and int(r["launches_first"]) == 0           # FG_ERR_UNSUPPORTED, nothing launched
+    assert "came under stream capture" in str(r["message"])
+    for suffix in ("", "_captured"):
+        got = _t(r["c" + suffix], "bf16")
+        gems_assert_close(got, torch_ref.mm(_t(r["a" + suffix], "bf16"), _t(r["b" + suffix], "bf16")), torch.bfloat16, reduce_dim=1024)
+
+
 def check_short_buffer(r, kw):
     msg = str(r["caught"])
     assert "outside every buffer" in msg and "nearest: %s" % kw["which"] in msg, msg
 
 
-CHECK = {"gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
+CHECK = {"static_first_call_under_capture": check_static_first_call_under_capture, "gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
          "softmax_backward": check_softmax_backward, "rms_norm_backward": check_rms_norm_backward,
          "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "rope": check_rope,
          "reshape_and_cache_flash": check_reshape_and_cache_flash, "reshape_and_cache": check_reshape_and_cache}
