@@ -520,3 +520,154 @@ def static_first_call_under_capture(dev, rng):
     out["bias"] = eager["bias"]
     out["schedule_used"] = eager["schedule_used"]
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# operands of more than 4 GiB: offsets that no longer fit 32 bits.  The buffers are virtual (zero pages until touched);
+# only the workgroups that work at the far end run.
+# ---------------------------------------------------------------------------------------------------------------
+def _poke(dev, ptr, byte_offset, array):
+    raw = np.ascontiguousarray(array).view(np.uint8).ravel()
+    dev.mem.view(ptr)[byte_offset:byte_offset + raw.size] = raw
+
+
+def _peek(dev, ptr, byte_offset, dtype, shape):
+    n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+    return dev.mem.view(ptr)[byte_offset:byte_offset + n].view(dtype).reshape(shape).copy()
+
+
+def huge_cache_and_attention(dev, rng, dtype="bf16", num_pages=210000, page_size=16, Hq=8, Hk=8, D=128, k_len=300, q_len=1):
+    """A paged cache of 6.4 GiB per tensor: tokens are scattered into its LAST pages by fg_reshape_and_cache_flash and
+    attended from there by fg_flash_attn_varlen_fwd (page offsets beyond 4 GiB on both paths)."""
+    page_elems = page_size * Hk * D
+    cache_bytes = num_pages * page_elems * 2
+    assert cache_bytes > 6 * 2 ** 30
+    pk, pv = dev.alloc(cache_bytes, "k_cache"), dev.alloc(cache_bytes, "v_cache")
+    pages = (k_len + page_size - 1) // page_size
+    table = (num_pages - 1 - rng.permutation(pages * 2)[:pages]).astype(np.int32).reshape(1, pages)     # among the last pages
+    key = bits(rng.standard_normal((k_len, Hk, D)), dtype)
+    val = bits(rng.standard_normal((k_len, Hk, D)), dtype)
+    slots = (table[0, np.arange(k_len) // page_size].astype(np.int64) * page_size + np.arange(k_len) % page_size)
+    pkey, pval, pslots = dev.upload(key, "key"), dev.upload(val, "value"), dev.upload(slots, "slot_mapping")
+    rc1 = dev.call("fg_reshape_and_cache_flash", P(pkey), P(pval), P(pk), P(pv), P(pslots), I32(1), I64(k_len), I32(Hk), I32(D),
+                   I32(page_size), I64(Hk * D), I64(Hk * D), I64(page_elems), I32(2), P(0))
+    # what landed in the pages of the table, gathered back in key order
+    got_k = np.stack([_peek(dev, pk, int(s) * Hk * D * 2, np.uint16, (Hk, D)) for s in slots])
+    got_v = np.stack([_peek(dev, pv, int(s) * Hk * D * 2, np.uint16, (Hk, D)) for s in slots])
+    q = bits(rng.standard_normal((q_len, Hq, D)), dtype)
+    p = FgFlashParams()
+    p.q, p.k_cache, p.v_cache = dev.upload(q, "q"), pk, pv
+    p.out = dev.alloc(q.nbytes, "out", fill=0x7B)
+    p.lse = dev.alloc(Hq * q_len * 4, "lse", fill=0x7B)
+    p.cu_seqlens_q = dev.upload(np.array([0, q_len], np.int32), "cu_seqlens_q")
+    p.seqused_k = dev.upload(np.array([k_len], np.int32), "seqused_k")
+    p.block_table = dev.upload(table, "block_table")
+    p.q_row_stride, p.q_head_stride, p.o_row_stride, p.o_head_stride = Hq * D, D, Hq * D, D
+    p.k_page_stride = p.v_page_stride = page_elems
+    p.k_row_stride = p.v_row_stride = Hk * D
+    p.k_head_stride = p.v_head_stride = D
+    p.block_table_stride, p.total_q = pages, q_len
+    p.batch, p.Hq, p.Hk, p.D, p.page_size = 1, Hq, Hk, D, page_size
+    p.max_seqlen_q, p.max_seqlen_k, p.is_causal, p.window_left, p.window_right = q_len, k_len, 1, -1, -1
+    p.softmax_scale, p.softcap, p.dtype = float(D) ** -0.5, 0.0, DT[dtype]
+    rc2 = dev.call("fg_flash_attn_varlen_fwd", C.byref(p), P(0))
+    # a dense two-page cache for the checker: page i of the sequence becomes page i
+    dense_k = np.zeros((pages, page_size, Hk, D), np.uint16)
+    dense_v = np.zeros((pages, page_size, Hk, D), np.uint16)
+    dense_k.reshape(-1, Hk, D)[:k_len], dense_v.reshape(-1, Hk, D)[:k_len] = key, val
+    return {"rc": rc1 or rc2, "key": key, "value": val, "got_k": got_k, "got_v": got_v, "q": q, "k_cache": dense_k, "v_cache": dense_v,
+            "block_table": np.arange(pages, dtype=np.int32).reshape(1, pages), "q_lens": np.array([q_len]), "k_lens": np.array([k_len]),
+            "out": dev.download(p.out, storage(dtype), q.shape), "lse": dev.download(p.lse, np.float32, (Hq, q_len)),
+            "slopes": np.zeros((1, Hq), np.float32), "min_byte_offset": np.array(int(slots.min()) * Hk * D * 2)}
+
+
+def huge_rows(dev, rng, op, dtype="bf16", M=1400000, N=2048):
+    """A row-wise operator on a matrix of more than 4 GiB, the last workgroup only: its rows lie beyond 2^32 bytes and
+    (for 16-bit types at this size) beyond 2^31 elements."""
+    item = ITEM[dtype]
+    assert M * N * item > 5 * 2 ** 30 and M * N > 2 ** 31
+    edge = 8
+    tail = (M - edge) * N * item
+    x = bits(rng.standard_normal((edge, N)), dtype)
+    px = dev.alloc(M * N * item, "x")
+    _poke(dev, px, tail, x)
+    out = {"x": x}
+    _only(dev, [-1])
+    try:
+        if op == "softmax":
+            po = dev.alloc(M * N * item, "out")
+            out["rc"] = dev.call("fg_softmax", P(px), P(po), I64(M), I64(N), I64(1), I32(DT[dtype]), I32(DT[dtype]), P(0))
+            out["out"] = _peek(dev, po, tail, storage(dtype), (edge, N))
+        elif op == "fused_add_rms_norm":
+            r = bits(rng.standard_normal((edge, N)), dtype)
+            w = bits(rng.uniform(0.5, 1.5, N), dtype)
+            pr, pw = dev.alloc(M * N * item, "residual"), dev.upload(w, "w")
+            _poke(dev, pr, tail, r)
+            out["rc"] = dev.call("fg_fused_add_rms_norm", P(px), P(pr), P(pw), I64(M), I64(N), I64(N), I64(N), F(1e-5), I32(DT[dtype]), P(0))
+            out.update(residual=r, w=w, x_out=_peek(dev, px, tail, storage(dtype), (edge, N)),
+                       residual_out=_peek(dev, pr, tail, storage(dtype), (edge, N)))
+        elif op == "silu_and_mul":
+            b = bits(rng.standard_normal((edge, N)), dtype)
+            pb, po = dev.alloc(M * N * item, "b"), dev.alloc(M * N * item, "out")
+            _poke(dev, pb, tail, b)
+            out["rc"] = dev.call("fg_silu_and_mul", P(px), P(pb), P(po), I64(M), I64(N), I64(N), I64(N), I64(N), I32(DT[dtype]), P(0))
+            out.update(b=b, out=_peek(dev, po, tail, storage(dtype), (edge, N)))
+    finally:
+        dev.group_filter = None
+    return out
+
+
+def huge_gemm(dev, rng, dtype="bf16", M=2500000, N=1024, K=1024, b_layout="nk"):
+    """C = A.B with A [M, K] and C [M, N] of more than 4 GiB each: the last workgroup of the launch, whose rows of A and C
+    start beyond 2^32 bytes."""
+    item = ITEM[dtype]
+    assert M * K * item > 4 * 2 ** 30 and M * N * item > 4 * 2 ** 30
+    edge = 256
+    a_tail = bits(rng.standard_normal((edge, K)) * 0.1, dtype)
+    b = bits(rng.standard_normal((K, N)) * 0.1, dtype)
+    pa = dev.alloc(M * K * item, "A")
+    _poke(dev, pa, (M - edge) * K * item, a_tail)
+    pb = dev.upload(np.ascontiguousarray(b.T) if b_layout == "nk" else b, "B")
+    sbk, sbn = (1, K) if b_layout == "nk" else (N, 1)
+    pc = dev.alloc(M * N * item, "C")
+    used = C.c_int(-1)
+    _only(dev, [-1])
+    try:
+        rc = dev.call("fg_gemm", P(pa), P(pb), P(0), P(pc), I64(M), I64(N), I64(K), I64(K), I64(1), I64(sbk), I64(sbn), I64(0), I64(0),
+                      I64(N), I64(1), F(1.0), F(0.0), I32(DT[dtype]), I32(DT[dtype]), I32(DT[dtype]), I32(1), P(0), C.c_size_t(0),
+                      C.byref(used), P(0))
+    finally:
+        dev.group_filter = None
+    c_tail = _peek(dev, pc, (M - edge) * N * item, storage(dtype), (edge, N))
+    done = c_tail.view(np.uint16) != 0
+    rows, cols = np.nonzero(done.any(axis=1))[0], np.nonzero(done.any(axis=0))[0]
+    return {"rc": rc, "a": a_tail[rows], "b": b[:, cols], "c": c_tail[np.ix_(rows, cols)], "done": done[np.ix_(rows, cols)],
+            "bias": np.zeros(0, np.float32), "rows": rows, "cols": cols, "schedule_used": np.array(used.value)}
+
+
+def huge_rope(dev, rng, dtype="bf16", n_tokens=600000, Hq=32, Hk=8, D=128, max_pos=64):
+    """In-place rotation of q [n_tokens, Hq, D] of 4.9 GiB: the last workgroup, i.e. the last tokens."""
+    item = ITEM[dtype]
+    assert n_tokens * Hq * D * item > 4 * 2 ** 30
+    edge = 4
+    q = bits(rng.standard_normal((edge, Hq, D)), dtype)
+    k = bits(rng.standard_normal((edge, Hk, D)), dtype)
+    ang = rng.uniform(0, 6.28, size=(max_pos, D // 2))
+    cos, sin = bits(np.cos(ang), "f32"), bits(np.sin(ang), "f32")
+    positions = np.zeros(n_tokens, dtype=np.int64)
+    positions[-edge:] = rng.integers(0, max_pos, size=edge)
+    pq, pk = dev.alloc(n_tokens * Hq * D * item, "q"), dev.alloc(n_tokens * Hk * D * item, "k")
+    q_tail, k_tail = (n_tokens - edge) * Hq * D * item, (n_tokens - edge) * Hk * D * item
+    _poke(dev, pq, q_tail, q)
+    _poke(dev, pk, k_tail, k)
+    pc, ps, ppos = dev.upload(cos, "cos"), dev.upload(sin, "sin"), dev.upload(positions, "pos")
+    arr = C.c_int64 * 3
+    qs, ks = arr(Hq * D, D, 1), arr(Hk * D, D, 1)
+    _only(dev, [-1])
+    try:
+        rc = dev.call("fg_rope", P(pq), P(pk), P(pq), P(pk), P(pc), P(ps), P(ppos), I32(1), I64(n_tokens), I64(n_tokens), I32(Hq), I32(Hk),
+                      I32(D), qs, ks, qs, ks, I64(1), I64(D // 2), I64(D // 2), I64(max_pos), I32(0), I32(DT[dtype]), I32(F32), P(0))
+    finally:
+        dev.group_filter = None
+    return {"rc": rc, "q": q, "k": k, "cos": cos, "sin": sin, "positions": positions[-edge:],
+            "q_out": _peek(dev, pq, q_tail, storage(dtype), q.shape), "k_out": _peek(dev, pk, k_tail, storage(dtype), k.shape)}

@@ -166,6 +166,16 @@ CASES = [
       op="softmax", dtype="bf16", M=131072, N=2048, K=1, groups=[0, -1], masked=0.01),
     C("full size: fused_add_rms_norm 4096x4096, 2 of 4096 workgroups", "rows_sampled", check="fused_add_rms_norm", lane=4,
       op="fused", dtype="bf16", M=4096, N=4096, eps=1e-6, groups=[0, -1]),
+    # ---- operands of more than 4 GiB (virtual buffers; the workgroups at the far end): offsets beyond 32 bits
+    C("6.4 GiB caches: scatter into the last pages, single-token attention over them", "huge_cache_and_attention", lane=5,
+      kernel="attn_decode_kernel"),
+    C("6.4 GiB caches: scatter into the last pages, prefill over them", "huge_cache_and_attention", lane=5, q_len=40, k_len=200,
+      kernel="attn_varlen_pipe_kernel"),
+    C("5.3 GiB matrix: softmax of the last rows", "huge_rows", lane=6, op="softmax"),
+    C("5.3 GiB matrices: fused_add_rms_norm of the last rows", "huge_rows", lane=6, op="fused_add_rms_norm"),
+    C("5.3 GiB matrices: silu_and_mul of the last rows", "huge_rows", lane=6, op="silu_and_mul"),
+    C("4.8 GiB A and C: the last tile of mm", "huge_gemm", lane=6, kernel="gemm_dma_kernel"),
+    C("4.9 GiB q: rotation of the last tokens", "huge_rope", lane=5),
     # ---- the entry point that allocates nothing, in a process whose first library call it is (lane 9: no fg_device_info)
     C("static entry: first call under capture is refused, later ones are not", "static_first_call_under_capture", lane=9, num_cu=8),
     # ---- the interpreter's bounds check itself
@@ -470,12 +480,54 @@ def check_static_first_call_under_capture(r, kw):
         gems_assert_close(got, torch_ref.mm(_t(r["a" + suffix], "bf16"), _t(r["b" + suffix], "bf16")), torch.bfloat16, reduce_dim=1024)
 
 
+def check_huge_cache_and_attention(r, kw):
+    assert int(r["min_byte_offset"]) > 2 ** 32
+    np.testing.assert_array_equal(r["got_k"], r["key"])           # the scatter, bit for bit, beyond 4 GiB
+    np.testing.assert_array_equal(r["got_v"], r["value"])
+    check_attention(r, dict(dtype="bf16", Hq=8, D=128))
+
+
+def check_huge_rows(r, kw):
+    """The rows the last workgroup of the launch wrote (the very last row at least) against the oracle."""
+    n = 2048
+    if kw["op"] == "fused_add_rms_norm":
+        rows = np.nonzero((r["x_out"] != r["x"]).any(axis=1))[0]
+    else:
+        rows = np.nonzero((r["out"].view(np.uint16) != 0).any(axis=1))[0]
+    assert len(rows) and rows[-1] == r["x"].shape[0] - 1, rows
+    if kw["op"] == "softmax":
+        check_softmax({"x": r["x"][rows].reshape(-1, n, 1), "out": r["out"][rows].reshape(-1, n, 1)}, dict(dtype="bf16"))
+    elif kw["op"] == "fused_add_rms_norm":
+        check_fused_add_rms_norm({k: (r[k][rows] if k != "w" else r[k]) for k in ("x", "residual", "w", "x_out", "residual_out")},
+                                 dict(dtype="bf16", N=n))
+    else:
+        gems_assert_close(_t(r["out"][rows], "bf16"), torch_ref.silu_and_mul(_t(r["x"][rows], "bf16"), _t(r["b"][rows], "bf16")),
+                          torch.bfloat16)
+
+
+def check_huge_rope(r, kw):
+    """Whatever part of the last tokens the last workgroup rotated (the last token's last head at least)."""
+    q, k = _t(r["q"], "bf16"), _t(r["k"], "bf16")
+    rq, rk = torch_ref.apply_rotary_pos_emb(q, k, _t(r["cos"], "f32"), _t(r["sin"], "f32"), torch.from_numpy(r["positions"]), False)
+    for got, before, ref in ((_t(r["q_out"], "bf16"), q, rq), (_t(r["k_out"], "bf16"), k, rk)):
+        done = (got != before).any(dim=-1)
+        gems_assert_close(got[done], ref[done], torch.bfloat16)
+        assert torch.equal(got[~done], before[~done])
+    assert bool((_t(r["q_out"], "bf16")[-1, -1] != q[-1, -1]).any()) or bool((_t(r["k_out"], "bf16")[-1, -1] != k[-1, -1]).any())
+
+
+def check_huge_gemm(r, kw):
+    assert r["done"].all() and r["done"].size >= 128 * 128          # a whole tile, at the far end of A and C
+    check_gemm_sampled(r, dict(dtype="bf16", K=1024, groups=[-1]))
+
+
 def check_short_buffer(r, kw):
     msg = str(r["caught"])
     assert "outside every buffer" in msg and "nearest: %s" % kw["which"] in msg, msg
 
 
-CHECK = {"static_first_call_under_capture": check_static_first_call_under_capture, "gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
+CHECK = {"huge_rope": check_huge_rope, "huge_cache_and_attention": check_huge_cache_and_attention, "huge_rows": check_huge_rows, "huge_gemm": check_huge_gemm,
+         "static_first_call_under_capture": check_static_first_call_under_capture, "gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
          "softmax_backward": check_softmax_backward, "rms_norm_backward": check_rms_norm_backward,
          "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "rope": check_rope,
          "reshape_and_cache_flash": check_reshape_and_cache_flash, "reshape_and_cache": check_reshape_and_cache}
