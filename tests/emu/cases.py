@@ -671,3 +671,33 @@ def huge_rope(dev, rng, dtype="bf16", n_tokens=600000, Hq=32, Hk=8, D=128, max_p
         dev.group_filter = None
     return {"rc": rc, "q": q, "k": k, "cos": cos, "sin": sin, "positions": positions[-edge:],
             "q_out": _peek(dev, pq, q_tail, storage(dtype), q.shape), "k_out": _peek(dev, pk, k_tail, storage(dtype), k.shape)}
+
+
+def bmm_per_matrix(dev, rng, dtype="bf16", batch=32, M=2048, N=2048, K=128, matrices=(0, 31), groups=(0, 1, -1)):
+    """The launches fg_bmm makes for a batch of `batch` matrices (one data-parallel fg_gemm per matrix on
+    base + z * stride), for the listed matrices only and a few workgroups of each: the attention-sized batch that
+    fg_bmm itself turns away."""
+    item = ITEM[dtype]
+    a = bits(rng.standard_normal((batch, M, K)) * 0.2, dtype)
+    b = bits(rng.standard_normal((batch, K, N)) * 0.2, dtype)
+    pa, pb = dev.upload(a, "A"), dev.upload(b, "B")
+    pc = dev.alloc(batch * M * N * item, "C")
+    rcs = []
+    _only(dev, list(groups))
+    try:
+        for z in matrices:
+            rcs.append(dev.call("fg_gemm", P(pa + z * M * K * item), P(pb + z * K * N * item), P(0), P(pc + z * M * N * item), I64(M),
+                                I64(N), I64(K), I64(K), I64(1), I64(N), I64(1), I64(0), I64(0), I64(N), I64(1), F(1.0), F(0.0),
+                                I32(DT[dtype]), I32(DT[dtype]), I32(DT[dtype]), I32(1), P(0), C.c_size_t(0), None, P(0)))
+    finally:
+        dev.group_filter = None
+    out = {"rc": np.array(max(rcs, key=abs))}
+    for z in matrices:
+        c = _peek(dev, pc, z * M * N * item, storage(dtype), (M, N))
+        done = c.view(np.uint16) != 0
+        rows, cols = np.nonzero(done.any(axis=1))[0], np.nonzero(done.any(axis=0))[0]
+        out.update({"a%d" % z: a[z][rows], "b%d" % z: b[z][:, cols], "c%d" % z: c[np.ix_(rows, cols)], "done%d" % z: done[np.ix_(rows, cols)]})
+    # nothing outside the listed matrices was written
+    others = [z for z in range(batch) if z not in matrices]
+    out["others_untouched"] = np.array(all(not _peek(dev, pc, z * M * N * item, np.uint8, (4096,)).any() for z in others))
+    return out

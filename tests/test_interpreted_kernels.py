@@ -166,6 +166,8 @@ CASES = [
       op="softmax", dtype="bf16", M=131072, N=2048, K=1, groups=[0, -1], masked=0.01),
     C("full size: fused_add_rms_norm 4096x4096, 2 of 4096 workgroups", "rows_sampled", check="fused_add_rms_norm", lane=4,
       op="fused", dtype="bf16", M=4096, N=4096, eps=1e-6, groups=[0, -1]),
+    # ---- the per-matrix launches of the attention-sized bmm that fg_bmm turns away (its round-1 kernel once faulted there)
+    C("bmm 32 x 2048x2048x128: the launches of matrices 0 and 31, three workgroups each", "bmm_per_matrix", lane=2),
     # ---- operands of more than 4 GiB (virtual buffers; the workgroups at the far end): offsets beyond 32 bits
     C("6.4 GiB caches: scatter into the last pages, single-token attention over them", "huge_cache_and_attention", lane=5,
       kernel="attn_decode_kernel"),
@@ -505,6 +507,16 @@ def check_huge_rows(r, kw):
                           torch.bfloat16)
 
 
+def check_bmm_per_matrix(r, kw):
+    assert bool(r["others_untouched"])
+    for z in (0, 31):
+        done = torch.from_numpy(r["done%d" % z])
+        assert int(done.sum()) >= 3 * 128 * 128
+        ref = torch_ref.mm(_t(r["a%d" % z], "bf16"), _t(r["b%d" % z], "bf16")).to(torch.bfloat16)
+        atol, rtol = torch_ref.gems_tolerance(torch.bfloat16, 128)
+        torch.testing.assert_close(_t(r["c%d" % z], "bf16")[done].double(), ref[done].double(), atol=atol, rtol=rtol)
+
+
 def check_huge_rope(r, kw):
     """Whatever part of the last tokens the last workgroup rotated (the last token's last head at least)."""
     q, k = _t(r["q"], "bf16"), _t(r["k"], "bf16")
@@ -526,7 +538,7 @@ def check_short_buffer(r, kw):
     assert "outside every buffer" in msg and "nearest: %s" % kw["which"] in msg, msg
 
 
-CHECK = {"huge_rope": check_huge_rope, "huge_cache_and_attention": check_huge_cache_and_attention, "huge_rows": check_huge_rows, "huge_gemm": check_huge_gemm,
+CHECK = {"bmm_per_matrix": check_bmm_per_matrix, "huge_rope": check_huge_rope, "huge_cache_and_attention": check_huge_cache_and_attention, "huge_rows": check_huge_rows, "huge_gemm": check_huge_gemm,
          "static_first_call_under_capture": check_static_first_call_under_capture, "gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
          "softmax_backward": check_softmax_backward, "rms_norm_backward": check_rms_norm_backward,
          "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "rope": check_rope,
