@@ -1,12 +1,16 @@
-"""A functional interpreter for the gfx950 (GCN/CDNA) assembly that hipcc emits for this library's kernels.
+"""An interpreter for the gfx950 (GCN/CDNA) assembly that hipcc emits for this library's kernels.
 
-It runs the compiler's own output (the `.s` text the build keeps, or a variant compiled on demand) on numpy: one
-wavefront is 64 lanes wide, a workgroup's wavefronts run until they all stand at a barrier, global memory is a set of
-registered buffers and EVERY access is bounds-checked against them.  It models function, not time: memory operations
-complete at once, wait counts and wait states mean nothing here (the static scans of isa_check.py cover those).
+It runs the compiler's own output (the `.s` text the build keeps beside the objects) on numpy: a wavefront is 64 lanes
+wide, a workgroup's wavefronts each run until they stand at a barrier (or end), workgroups run one after the other.
+Global memory is a set of registered buffers and EVERY access is checked against them; LDS, private memory and all
+registers start out holding NaNs.  Memory operations stay "in flight" until an s_waitcnt covers them: using a register
+a load in flight will write, or LDS bytes a write or an LDS-DMA in flight will fill, is an error, and so is LDS traffic
+between two wavefronts with no barrier in between (class Exec).  It models function and ordering, not time: latencies,
+wait states between dependent instructions and bank conflicts are outside it (csrc/isa_check.py scans for wait states).
 
-Trust comes from the kernels the GPU parity suite has passed: the interpreter must reproduce the oracle on those, and
-is then used to run kernel variants that have not been on a GPU yet.
+Trust comes from the kernels the GPU parity suite has passed: the interpreter reproduces the oracle on those
+(tests/test_interpreted_kernels.py, default build), and is then used on kernel variants that have not been on a GPU.
+Instructions are added as kernels need them; an unknown one is an error that names it, never a guess.
 """
 import re
 import struct
@@ -266,7 +270,7 @@ def parse_program(text, name_part, exact=False):
                 m = _MOD.match(f)
                 if m:
                     mods[m.group(1)] = m.group(2)
-                elif f in _FLAGS and not (first and f == "off" and False):
+                elif f in _FLAGS:
                     if f == "off" and first:
                         ops.append("off")
                     else:
@@ -332,9 +336,6 @@ def f16_bits(f):
 def f16_to_f32(bits16):
     return np.asarray(bits16, dtype=np.uint16).view(np.float16).astype(np.float32)
 
-
-_FLOAT_INLINE = {"0.5": 0.5, "-0.5": -0.5, "1.0": 1.0, "-1.0": -1.0, "2.0": 2.0, "-2.0": -2.0, "4.0": 4.0, "-4.0": -4.0,
-                 "0.15915494": 0.15915494}
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -712,26 +713,6 @@ def _cmp(op, a, b):
 def _fma32(a, b, c):
     with np.errstate(all="ignore"):
         return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
-
-
-def _as(kind, u):
-    if kind == "f32":
-        return f32(u)
-    if kind == "i32":
-        return i32(u)
-    if kind == "u32":
-        return u
-    if kind == "f16":
-        return f16_to_f32(u & U32(0xFFFF))
-    if kind == "i64":
-        return u.view(np.int64)
-    if kind == "u64":
-        return u
-    if kind == "u16":
-        return u & U32(0xFFFF)
-    if kind == "i16":
-        return (u & U32(0xFFFF)).astype(np.uint16).view(np.int16).astype(np.int32)
-    raise EmuError(kind)
 
 
 _F32_BIN = {
@@ -1268,10 +1249,6 @@ class _V:
         return mask_to_lanes(self.ex.sread(self.w, tok, 64))
 
 
-_CMP_KIND = {"f32": "f32", "f16": "f16", "i32": "i32", "u32": "u32", "i64": "i64", "u64": "u64", "f64": "f64",
-             "i16": "i16", "u16": "u16"}
-
-
 def _class_f32(x, mask):
     u = u32(x)
     e = (u >> U32(23)) & U32(0xFF)
@@ -1340,7 +1317,6 @@ def _div_fixup_f32(q, den, num):
         zero = sign.view(np.float32)
         res = ((u32(q) & U32(0x7FFFFFFF)) | sign).view(np.float32)
         e1, e2 = _exp_of(den), _exp_of(num)
-        res = np.where(e1 == 255, inf, res) if False else res
         res = np.where((e2 - e1) < -150, zero, res)
         res = np.where(np.isinf(den) | (num == 0), zero, res)
         res = np.where((den == 0) | np.isinf(num), inf, res)
@@ -1403,19 +1379,15 @@ def _valu(ex, w, ins):
         cnt = np.array([bin(int(x)).count("1") for x in (m & below)], dtype=U32)
         return V.dst(ops[0], "u32", cnt + V.src(ops[2], 1, "u32"))
     if base == "v_cndmask_b32":
-        a, b = V.raw(ops[1], 0)[0:3], V.raw(ops[2], 1)[0:3]
-        av, bv = a[0], b[0]
-        for (val, neg, ab), which in ((a, 0), (b, 1)):
+        picks = []
+        for pos in (0, 1):                       # sign modifiers act on the bit pattern as fp32
+            val, neg, ab = V.raw(ops[1 + pos], pos)
             if ab:
                 val = val & U32(0x7FFFFFFF)
             if neg:
                 val = val ^ U32(0x80000000)
-            if which == 0:
-                av = val
-            else:
-                bv = val
-        sel = V.mask_in(ops[3])
-        return V.dst(ops[0], "b32", np.where(sel, bv, av))
+            picks.append(val)
+        return V.dst(ops[0], "b32", np.where(V.mask_in(ops[3]), picks[1], picks[0]))
     # ---- compares
     m = re.match(r"^v_cmp(x?)_(class|[a-z]+)_(f16|f32|f64|i16|u16|i32|u32|i64|u64)$", base)
     if m:
@@ -1729,9 +1701,6 @@ def _valu_more(ex, w, ins, V):
 # ---------------------------------------------------------------------------------------------------------------
 # LDS, scratch, atomics
 # ---------------------------------------------------------------------------------------------------------------
-_DS_RW = {"b32": 4, "b64": 8, "b96": 12, "b128": 16}
-
-
 def _lds_bytes(ex, ins, a, width):
     a = a.astype(np.int64)
     if (a < 0).any() or (a + width > ex.lds.size).any():
