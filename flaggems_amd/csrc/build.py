@@ -128,6 +128,13 @@ def _check_wait_states(src, obj, obj_dir=OBJ_DIR):
         raise RuntimeError("%s: the device assembly fails %d check(s) of isa_check.py:\n%s" % (src, len(hits), "\n".join(lines)))
 
 
+# The value at which each switch of variants.h is on trial (its default is the GPU-tested code).  A library built with
+# all of them ("cand") is what the interpreted tests run beside the default one.
+TRIAL = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "ATTN_Q_UNCOND": 1, "DECODE_Q_EARLY": 1,
+         "RMS_BWD_ZERO_PACK": 1, "ADDMM_BCAST_BRANCH": 1, "DMA_SCALAR_BASES": 1, "DMA_COPY_RUNS": 3, "ATTN_ROWSUM_MFMA": 1,
+         "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1}
+
+
 def variant_defines(variants):
     """{"ROWS_UPFRONT": 1} -> ["-DFG_V_ROWS_UPFRONT=1"]; the names are checked against csrc/variants.h."""
     known = set(re.findall(r"^#define FG_V_(\w+) ", open(os.path.join(HERE, "variants.h")).read(), re.M))

@@ -28,9 +28,11 @@ CSRC = os.path.join(REPO, "flaggems_amd", "csrc")
 TD = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}
 
 # every switch of variants.h at its trial value
-VARIANTS = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "ATTN_Q_UNCOND": 1,
-            "DECODE_Q_EARLY": 1, "RMS_BWD_ZERO_PACK": 1, "ADDMM_BCAST_BRANCH": 1, "DMA_SCALAR_BASES": 1, "DMA_COPY_RUNS": 3,
-            "ATTN_ROWSUM_MFMA": 1, "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1}
+sys.path.insert(0, CSRC)
+try:
+    from build import TRIAL as VARIANTS
+finally:
+    sys.path.remove(CSRC)
 
 
 def C(cid, fn, check=None, kernel=None, variant_kernel=None, seed=0, num_cu=256, lane=0, **kw):
