@@ -168,7 +168,7 @@ CASES = [
       op="softmax", dtype="bf16", M=131072, N=2048, K=1, groups=[0, -1], masked=0.01),
     C("full size: fused_add_rms_norm 4096x4096, 2 of 4096 workgroups", "rows_sampled", check="fused_add_rms_norm", lane=4,
       op="fused", dtype="bf16", M=4096, N=4096, eps=1e-6, groups=[0, -1]),
-    # ---- the per-matrix launches of the attention-sized bmm that fg_bmm turns away (its round-1 kernel once faulted there)
+    # ---- the per-matrix launches of the attention-sized bmm that fg_bmm turns away (an early kernel once faulted there)
     C("bmm 32 x 2048x2048x128: the launches of matrices 0 and 31, three workgroups each", "bmm_per_matrix", lane=2),
     # ---- operands of more than 4 GiB (virtual buffers; the workgroups at the far end): offsets beyond 32 bits
     C("6.4 GiB caches: scatter into the last pages, single-token attention over them", "huge_cache_and_attention", lane=5,
