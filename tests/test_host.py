@@ -100,6 +100,45 @@ def test_library_exports_every_declared_symbol():
     assert _C.lib().fg_abi_version() == 2
 
 
+_C_BINDER = r"""
+#include <stddef.h>
+#include <stdio.h>
+#include "fg_mi355.h"
+int main(void) {
+  FgFlashParams p;
+  int rc = fg_softmax(NULL, NULL, -1, 4, 1, FG_F32, FG_F32, NULL);
+  printf("abi=%d rc=%d (%s) invalid=%d unsupported=%d\n", fg_abi_version(), rc, fg_last_error(), FG_ERR_INVALID,
+         FG_ERR_UNSUPPORTED);
+  printf("params=%d workspace_at=%d\n", (int)sizeof p, (int)offsetof(FgFlashParams, workspace));
+  return 0;
+}
+"""
+
+
+def test_header_is_plain_c_and_a_c_program_binds_the_library(tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 and as C++11, and a C program that includes it and
+    links the library calls an entry point and reads its error message; the struct the attention entry point takes has
+    the size and field offset the ctypes mirror gives it.  (No launch: the call is rejected on the host.)"""
+    import shutil
+    import subprocess
+
+    gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+    if gcc is None or gxx is None:
+        pytest.skip("no host compiler")
+    inc = os.path.join(ROOT, "include")
+    strict = ["-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only"]
+    subprocess.run([gcc, "-std=c99", "-x", "c"] + strict + [os.path.join(inc, "fg_mi355.h")], check=True)
+    subprocess.run([gxx, "-std=c++11", "-x", "c++"] + strict + [os.path.join(inc, "fg_mi355.h")], check=True)
+    src, exe = tmp_path / "binder.c", tmp_path / "binder"
+    src.write_text(_C_BINDER)
+    libdir = os.path.dirname(_C.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", inc, str(src), "-o", str(exe),
+                    "-L", libdir, "-l:" + os.path.basename(_C.LIB_PATH), "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert "abi=2 rc=-1 (softmax: negative size) invalid=-1 unsupported=-2" in out, out
+    assert "params=%d workspace_at=%d" % (ctypes.sizeof(_C.FgFlashParams), _C.FgFlashParams.workspace.offset) in out, out
+
+
 def test_struct_mirror_matches_header_order():
     header = open(os.path.join(ROOT, "include", "fg_mi355.h")).read()
     body = header[header.index("typedef struct FgFlashParams {"):header.index("} FgFlashParams;")]
