@@ -139,6 +139,29 @@ def test_header_is_plain_c_and_a_c_program_binds_the_library(tmp_path):
     assert "params=%d workspace_at=%d" % (ctypes.sizeof(_C.FgFlashParams), _C.FgFlashParams.workspace.offset) in out, out
 
 
+def test_documented_cpp_binding_compiles():
+    """The C++ binding that the integration notes show for the reference's native layer (an ATen function around
+    fg_rms_norm) is real code: it passes the compiler's front end against this image's torch and HIP headers."""
+    import shutil
+    import subprocess
+
+    gxx = shutil.which("g++")
+    notes = os.path.join(ROOT, "INTEGRATION.md")
+    if gxx is None or not os.path.exists(notes) or not os.path.isdir("/opt/rocm/include"):
+        pytest.skip("needs g++, the integration notes and the ROCm headers")
+    from torch.utils.cpp_extension import include_paths
+
+    block = re.search(r"```cpp\n(.*?)```", open(notes).read(), re.S)
+    assert block and "fg_rms_norm(" in block.group(1)
+    unit = ("#include <ATen/ATen.h>\n#include <c10/core/DeviceGuard.h>\n#include <c10/hip/HIPStream.h>\n"
+            "#include <torch/library.h>\n" + block.group(1))
+    cmd = [gxx, "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM", "-x", "c++", "-"]
+    for inc in include_paths() + ["/opt/rocm/include", os.path.join(ROOT, "include")]:
+        cmd += ["-I", inc]
+    p = subprocess.run(cmd, input=unit, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr[-3000:]
+
+
 def test_struct_mirror_matches_header_order():
     header = open(os.path.join(ROOT, "include", "fg_mi355.h")).read()
     body = header[header.index("typedef struct FgFlashParams {"):header.index("} FgFlashParams;")]
