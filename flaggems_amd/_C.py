@@ -95,6 +95,8 @@ _SIGNATURES = {
         [c_vp, c_vp, c_vp, c_vp, c_vp, c_int, c_i64, c_int, c_int, c_int, c_int, c_i64, c_i64, c_i64, c_int, c_vp],
     ),
     "fg_silu_and_mul": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
+    "fg_silu_and_mul_backward": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                         c_int, c_vp]),
     "fg_softmax_backward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),
     "fg_log_softmax_backward": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_int, c_int, c_vp]),
     "fg_rms_norm_backward_partial_rows": (c_i64, [c_i64, c_i64, c_int, c_int]),

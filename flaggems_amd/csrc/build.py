@@ -132,7 +132,7 @@ def _check_wait_states(src, obj, obj_dir=OBJ_DIR):
 # all of them ("cand") is what the interpreted tests run beside the default one.
 TRIAL = {"ROWS_UPFRONT": 1, "SHORT_UPFRONT": 1, "SCATTER_EARLY": 1, "ROPE_ARGS": 1, "ATTN_Q_UNCOND": 1, "DECODE_Q_EARLY": 1,
          "RMS_BWD_ZERO_PACK": 1, "ADDMM_BCAST_BRANCH": 1, "DMA_SCALAR_BASES": 1, "DMA_COPY_RUNS": 3, "ATTN_ROWSUM_MFMA": 1,
-         "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1}
+         "RMS_TWO_ROWS": 1, "SKINNY_ASM_A": 1, "SILU_GRAD_KERNEL": 1}
 
 
 def variant_defines(variants):

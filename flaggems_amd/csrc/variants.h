@@ -90,3 +90,10 @@
 #ifndef FG_V_DMA_COPY_RUNS
 #define FG_V_DMA_COPY_RUNS 2
 #endif
+
+// fg_silu_and_mul_backward: the gradient kernel of silu_and_mul (silu_mul_grad_kernel).  A new kernel, not a change to
+// a tested one; it is compiled only with the switch on, and until then the entry point answers FG_ERR_UNSUPPORTED and
+// the Python operator takes its gradient from the vendor's elementwise kernels.
+#ifndef FG_V_SILU_GRAD_KERNEL
+#define FG_V_SILU_GRAD_KERNEL 0
+#endif

@@ -149,6 +149,16 @@ int fg_silu_and_mul(const void* a, const void* b, void* out, int64_t rows, int64
                     int64_t a_row_stride, int64_t b_row_stride, int64_t o_row_stride, int dtype,
                     void* stream);
 
+/* Gradients of fg_silu_and_mul: with s = 1 / (1 + exp(-a)),
+ *   grad_a = grad_out * b * s * (1 + a * (1 - s)),   grad_b = grad_out * a * s   (fp32 arithmetic),
+ * five [rows, cols] operands of one dtype with unit inner stride and independent row strides.
+ * FG_ERR_UNSUPPORTED from a build that leaves the kernel out (csrc/variants.h, FG_V_SILU_GRAD_KERNEL).
+ * Replaces silu_and_mul_grad_kernel, src/flag_gems/fused/silu_and_mul.py:20-44. */
+int fg_silu_and_mul_backward(const void* a, const void* b, const void* grad_out, void* grad_a, void* grad_b,
+                             int64_t rows, int64_t cols, int64_t a_row_stride, int64_t b_row_stride,
+                             int64_t g_row_stride, int64_t ga_row_stride, int64_t gb_row_stride, int dtype,
+                             void* stream);
+
 /* GEMM schedules. */
 enum { FG_SCHED_AUTO = 0, FG_SCHED_DATA_PARALLEL = 1, FG_SCHED_STREAM_K = 2 };
 

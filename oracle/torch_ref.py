@@ -144,6 +144,14 @@ def silu_and_mul(a, b):
     return F.silu(to_reference(a, True)) * to_reference(b, True)
 
 
+def silu_and_mul_grads(a, b, grad):
+    """tests/test_binary_pointwise_ops.py:1377-1403: autograd through F.silu(a) * b on fp64 copies.
+    Returns (da, db)."""
+    ar = to_reference(a, True).clone().requires_grad_(True)
+    br = to_reference(b, True).clone().requires_grad_(True)
+    return torch.autograd.grad(F.silu(ar) * br, (ar, br), to_reference(grad, True))
+
+
 def alibi_bias(slopes, seqlen_q, seqlen_k, causal):
     """tests/test_attention_ops.py:804-816: slopes [batch, heads] -> bias broadcastable to
     [batch, heads, seqlen_q, seqlen_k]."""

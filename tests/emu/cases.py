@@ -179,6 +179,23 @@ def silu_and_mul(dev, rng, dtype, rows, cols, a_stride=None, b_stride=None, o_st
     return {"rc": rc, "a": a, "b": b, "out": o, "gap_ok": gap_ok}
 
 
+def silu_and_mul_backward(dev, rng, dtype, rows, cols, a_stride=None, b_stride=None, g_stride=None, da_stride=None,
+                          db_stride=None):
+    a_stride, b_stride, g_stride = a_stride or cols, b_stride or cols, g_stride or cols
+    da_stride, db_stride = da_stride or cols, db_stride or cols
+    a = bits(rng.standard_normal((rows, cols)) * 2, dtype)
+    b = bits(rng.standard_normal((rows, cols)), dtype)
+    g = bits(rng.standard_normal((rows, cols)), dtype)
+    A, B = Strided(dev, rows, cols, a_stride, dtype, a, "a"), Strided(dev, rows, cols, b_stride, dtype, b, "b")
+    G = Strided(dev, rows, cols, g_stride, dtype, g, "g")
+    DA, DB = Strided(dev, rows, cols, da_stride, dtype, None, "da"), Strided(dev, rows, cols, db_stride, dtype, None, "db")
+    rc = dev.call("fg_silu_and_mul_backward", P(A.ptr), P(B.ptr), P(G.ptr), P(DA.ptr), P(DB.ptr), I64(rows), I64(cols),
+                  I64(a_stride), I64(b_stride), I64(g_stride), I64(da_stride), I64(db_stride), I32(DT[dtype]), P(0))
+    da, ok1 = DA.read()
+    db, ok2 = DB.read()
+    return {"rc": rc, "a": a, "b": b, "g": g, "da": da, "db": db, "gap_ok": ok1 and ok2}
+
+
 def rope(dev, rng, dtype, n_tokens, Hq, Hk, D, interleaved=False, pos="i64", inplace=True, cs_dtype="f32", max_pos=64,
          seq_len=None, head_pad=0):
     """q [n_tokens, Hq, D] with `head_pad` unused elements behind every head (a slice of a wider projection)."""

@@ -35,12 +35,14 @@ finally:
     sys.path.remove(CSRC)
 
 
-def C(cid, fn, check=None, kernel=None, variant_kernel=None, seed=0, num_cu=256, lane=0, **kw):
+def C(cid, fn, check=None, kernel=None, variant_kernel=None, seed=0, num_cu=256, lane=0, variants_only=None, **kw):
     """num_cu: compute units the interpreted device reports.  The library sizes tiles, grids and stream-K partitions
     from it, so a device of a few CUs brings the large-tile kernels within reach of small problems.
-    lane: cases of one (num_cu, lane) share a worker process; long cases get lanes of their own."""
+    lane: cases of one (num_cu, lane) share a worker process; long cases get lanes of their own.
+    variants_only: the entry point's kernel exists only in the build with the variants on; the default build must
+    answer FG_ERR_UNSUPPORTED with this text in its message, and launch nothing."""
     return {"id": cid, "fn": fn, "kw": kw, "seed": seed, "check": check or fn, "kernel": kernel,
-            "variant_kernel": variant_kernel, "num_cu": num_cu, "lane": lane}
+            "variant_kernel": variant_kernel, "num_cu": num_cu, "lane": lane, "variants_only": variants_only}
 
 
 CASES = [
@@ -81,6 +83,19 @@ CASES = [
     C("silu bf16 halves of one projection", "silu_and_mul", dtype="bf16", rows=5, cols=512, a_stride=1024, b_stride=1024),
     C("silu f16 7x264", "silu_and_mul", dtype="f16", rows=7, cols=264),
     C("silu f32 3x101", "silu_and_mul", dtype="f32", rows=3, cols=101),
+    # (the gradient kernel is compiled only with its switch on: the default build's entry point says so)
+    C("silu backward bf16, halves of one projection", "silu_and_mul_backward", dtype="bf16", rows=5, cols=512, a_stride=1024,
+      b_stride=1024, variant_kernel="silu_mul_grad_kernel", variants_only="not part of this build"),
+    C("silu backward f16 7x264 strided outputs", "silu_and_mul_backward", dtype="f16", rows=7, cols=264, g_stride=272, da_stride=280,
+      db_stride=296, variant_kernel="silu_mul_grad_kernel", variants_only="not part of this build"),
+    C("silu backward f32 3x101", "silu_and_mul_backward", dtype="f32", rows=3, cols=101, variant_kernel="silu_mul_grad_kernel",
+      variants_only="not part of this build"),
+    C("silu backward f32 4x64", "silu_and_mul_backward", dtype="f32", rows=4, cols=64, variant_kernel="silu_mul_grad_kernel",
+      variants_only="not part of this build"),
+    C("silu backward f16 3x77", "silu_and_mul_backward", dtype="f16", rows=3, cols=77, variant_kernel="silu_mul_grad_kernel",
+      variants_only="not part of this build"),
+    C("silu backward bf16 4x333 odd stride", "silu_and_mul_backward", dtype="bf16", rows=4, cols=333, a_stride=335,
+      variant_kernel="silu_mul_grad_kernel", variants_only="not part of this build"),
     C("rope bf16 neox", "rope", dtype="bf16", n_tokens=5, Hq=4, Hk=2, D=128),
     C("rope f16 interleaved i32 out of place", "rope", dtype="f16", n_tokens=4, Hq=3, Hk=1, D=64, interleaved=True, pos="i32",
       inplace=False),
@@ -354,6 +369,13 @@ def check_silu_and_mul(r, kw):
     gems_assert_close(_t(r["out"], dt), ref, TD[dt])
 
 
+def check_silu_and_mul_backward(r, kw):
+    dt = kw["dtype"]
+    da, db = torch_ref.silu_and_mul_grads(_t(r["a"], dt), _t(r["b"], dt), _t(r["g"], dt))
+    gems_assert_close(_t(r["da"], dt), da, TD[dt])
+    gems_assert_close(_t(r["db"], dt), db, TD[dt])
+
+
 def check_rope(r, kw):
     dt, cdt = kw["dtype"], kw.get("cs_dtype", "f32")
     D = kw["D"]
@@ -545,7 +567,7 @@ def check_short_buffer(r, kw):
 CHECK = {"bmm_per_matrix": check_bmm_per_matrix, "huge_rope": check_huge_rope, "huge_cache_and_attention": check_huge_cache_and_attention, "huge_rows": check_huge_rows, "huge_gemm": check_huge_gemm,
          "static_first_call_under_capture": check_static_first_call_under_capture, "gemm_sampled": check_gemm_sampled, "attention_sampled": check_attention_sampled, "short_buffer": check_short_buffer, "gemm": check_gemm, "bmm": check_bmm, "attention": check_attention, "rms_norm": check_rms_norm, "fused_add_rms_norm": check_fused_add_rms_norm, "softmax": check_softmax,
          "softmax_backward": check_softmax_backward, "rms_norm_backward": check_rms_norm_backward,
-         "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "rope": check_rope,
+         "transpose2d": check_transpose2d, "silu_and_mul": check_silu_and_mul, "silu_and_mul_backward": check_silu_and_mul_backward, "rope": check_rope,
          "reshape_and_cache_flash": check_reshape_and_cache_flash, "reshape_and_cache": check_reshape_and_cache}
 
 
@@ -553,6 +575,9 @@ CHECK = {"bmm_per_matrix": check_bmm_per_matrix, "huge_rope": check_huge_rope, "
 def test_interpreted(runs, build, case):
     r = Result(runs(build, (case["num_cu"], case["lane"])), case["id"])
     assert "__error" not in r, str(r["__error"])
+    if build == "default" and case.get("variants_only"):
+        assert int(r["rc"]) == -2 and case["variants_only"] in str(r["__message"]) and not r.kernels()
+        return
     assert int(r["rc"]) == 0, str(r["__message"]) if "__message" in r else "rc %d" % int(r["rc"])
     if "gap_ok" in r:
         assert bool(r["gap_ok"]), "elements between the rows of a strided operand were overwritten"

@@ -280,6 +280,26 @@ def test_silu_and_mul_closed_form():
     assert torch.allclose(O.silu_and_mul(a, b), ref)
 
 
+def test_silu_and_mul_grads_pinned():
+    """Closed form (d silu(x)/dx = s + x s (1 - s), s the logistic function) on hand-picked points, and central
+    differences of the pinned forward on random ones."""
+    a = torch.tensor([0.0, 1.0, -2.0, 30.0]); b = torch.tensor([3.0, 2.0, 0.5, 1.0]); g = torch.tensor([1.0, -2.0, 4.0, 0.5])
+    da, db = O.silu_and_mul_grads(a, b, g)
+    sig = [1 / (1 + math.exp(-v)) for v in a.tolist()]
+    want_da = [gi * bi * (s + x * s * (1 - s)) for gi, bi, s, x in zip(g.tolist(), b.tolist(), sig, a.tolist())]
+    want_db = [gi * x * s for gi, s, x in zip(g.tolist(), sig, a.tolist())]
+    assert torch.allclose(da, torch.tensor(want_da, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(db, torch.tensor(want_db, dtype=torch.float64), atol=1e-12)
+    assert da[0] == 0.5 * 3.0 and db[0] == 0.0             # at 0: silu' = 1/2, silu = 0
+    torch.manual_seed(3)
+    a, b, g = torch.randn(5, 7, dtype=torch.float64), torch.randn(5, 7, dtype=torch.float64), torch.randn(5, 7, dtype=torch.float64)
+    da, db = O.silu_and_mul_grads(a, b, g)
+    h = 1e-6
+    num_da = (O.silu_and_mul(a + h, b) - O.silu_and_mul(a - h, b)) / (2 * h) * g
+    num_db = (O.silu_and_mul(a, b + h) - O.silu_and_mul(a, b - h)) / (2 * h) * g
+    assert torch.allclose(da, num_da, atol=1e-8) and torch.allclose(db, num_db, atol=1e-8)
+
+
 # ---------------------------------------------------------------------------------------------
 # paged attention
 # ---------------------------------------------------------------------------------------------

@@ -154,6 +154,11 @@ class Harness:
         self.inside("silu b", b, e, [(rows, brs), (cols, 1)])
         self.inside("silu out", out, e, [(rows, ors), (cols, 1)])
 
+    def chk_fg_silu_and_mul_backward(self, a, b, g, da, db, rows, cols, ars, brs, grs, dars, dbrs, dtype, stream):
+        e = ESIZE[dtype]
+        for what, ptr, rs in (("a", a, ars), ("b", b, brs), ("grad_out", g, grs), ("grad_a", da, dars), ("grad_b", db, dbrs)):
+            self.inside("silu backward " + what, ptr, e, [(rows, rs), (cols, 1)])
+
     def chk_fg_gemm(self, A, B, bias, C, M, N, K, sam, sak, sbk, sbn, sim, sin_, scm, scn, alpha, beta, ab, cdt, bdt,
                     schedule, ws, ws_bytes, used, stream):
         self.inside("gemm A", A, ESIZE[ab], [(M, sam), (K, sak)])
@@ -318,6 +323,17 @@ def test_rowwise_operands(hx, dtype):
     for name in ("fg_softmax", "fg_log_softmax", "fg_rms_norm", "fg_fused_add_rms_norm", "fg_silu_and_mul",
                  "fg_softmax_backward", "fg_log_softmax_backward"):
         assert name in done, name
+
+
+def test_silu_and_mul_autograd_operands(hx):
+    gu = _r(30, 256).requires_grad_()
+    y = flag_gems.silu_and_mul(gu[:, :128], gu[:, 128:])       # halves of one gate-up tensor, saved as views
+    y.backward(_r(60, 128)[::2])                               # a gradient with gaps between its rows
+    a, b = _r(4, 1, 64).requires_grad_(), _r(1, 5, 64).requires_grad_()
+    flag_gems.silu_and_mul(a, b).sum().backward()              # broadcast operands, an expanded (stride-0) gradient
+    assert gu.grad.shape == (30, 256) and a.grad.shape == (4, 1, 64) and b.grad.shape == (1, 5, 64)
+    done = hx.check_all()
+    assert done.count("fg_silu_and_mul") == 2 and done.count("fg_silu_and_mul_backward") == 2
 
 
 def test_rms_norm_autograd_operands(hx):

@@ -6,6 +6,7 @@ import torch
 
 import flag_gems
 from oracle import torch_ref as O
+from helpers import gems_assert_close
 from test_gpu_attention import ATOL, RTOL, make_case
 from test_gpu_zgraph import _fresh_stream, _sk_inputs, _streamk_mm
 
@@ -38,6 +39,54 @@ def test_flash_attn_varlen_func_swap_qg(gpu, seq_lens, num_heads, head_size, blo
     torch.testing.assert_close(out.cpu(), ref.to(dtype), atol=ATOL, rtol=RTOL)
     ref32 = O.paged_attention(q, kc, vc, qlens, klens, bt, scale, causal=True, soft_cap=soft_cap, compute_dtype=torch.float32)
     torch.testing.assert_close(out.float().cpu(), ref32, atol=ATOL, rtol=RTOL)
+
+
+# The reference's own test of silu_and_mul differentiates it (tests/test_binary_pointwise_ops.py:1377-1403, shapes
+# POINTWISE_SHAPES of tests/accuracy_utils.py:59-63 and the quick-mode shape, all float dtypes): output and both
+# gradients against autograd through F.silu(a) * b on upcast copies.  Plus the halves of one gate-up tensor (views
+# with a row stride) and broadcast operands.
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(), (1,), (2, 19, 7), (1024, 1024), (20, 320, 15), (16, 128, 64, 60), (16, 7, 57, 32, 29),
+                                   "halves", "broadcast"], ids=lambda s: ("x".join(map(str, s)) or "scalar") if isinstance(s, tuple) else s)
+def test_accuracy_silu_and_mul_with_gradients(gpu, shape, dtype):
+    torch.manual_seed(0)
+    if shape == "halves":
+        gu = torch.randn(16, 22016, dtype=dtype, device=gpu, requires_grad=True)
+        inputs, (a, b) = (gu,), (gu[:, :11008], gu[:, 11008:])
+    elif shape == "broadcast":
+        a = torch.randn(6, 1, 96, dtype=dtype, device=gpu, requires_grad=True)
+        b = torch.randn(1, 5, 96, dtype=dtype, device=gpu, requires_grad=True)
+        inputs = (a, b)
+    else:
+        a = torch.randn(shape, dtype=dtype, device=gpu, requires_grad=True)
+        b = torch.randn(shape, dtype=dtype, device=gpu, requires_grad=True)
+        inputs = (a, b)
+    res = flag_gems.silu_and_mul(a, b)
+    assert res.dtype == dtype and res.requires_grad
+    out_grad = torch.randn_like(res)
+    res_grads = torch.autograd.grad(res, inputs, out_grad)
+    # the oracle: the same expression on fp64 CPU copies, differentiated by autograd
+    ref_inputs = tuple(O.to_reference(t.detach(), True).requires_grad_(True) for t in inputs)
+    ra, rb = (ref_inputs[0][:, :11008], ref_inputs[0][:, 11008:]) if shape == "halves" else ref_inputs
+    ref = torch.nn.functional.silu(ra) * rb
+    ref_grads = torch.autograd.grad(ref, ref_inputs, O.to_reference(out_grad, True))
+    gems_assert_close(res.detach(), ref.detach(), dtype)
+    for got, want in zip(res_grads, ref_grads):
+        assert got.shape == want.shape and got.dtype == dtype
+        if shape != "broadcast":
+            gems_assert_close(got, want, dtype)
+    if shape == "broadcast":
+        # a broadcast operand's gradient is the sum, taken by torch in `dtype`, of 5 or 6 per-element gradients that
+        # were each rounded to `dtype`: held to the reference's relative resolution of the sum of their magnitudes
+        from flag_gems.testing import RESOLUTION
+
+        ea, eb = torch.broadcast_tensors(*ref_inputs)
+        da, db = O.silu_and_mul_grads(ea, eb, out_grad)
+        for got, want, terms, axis in ((res_grads[0], ref_grads[0], da, 1), (res_grads[1], ref_grads[1], db, 0)):
+            bound = RESOLUTION[dtype] * terms.abs().sum(axis, keepdim=True) + 1e-4
+            assert ((got.cpu().double() - want).abs() <= 2 * bound).all()
+    with torch.no_grad():
+        assert not flag_gems.silu_and_mul(a, b).requires_grad
 
 
 def test_workspace_made_under_capture_then_used_eagerly(gpu):
