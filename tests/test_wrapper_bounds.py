@@ -336,6 +336,44 @@ def test_silu_and_mul_autograd_operands(hx):
     assert done.count("fg_silu_and_mul") == 2 and done.count("fg_silu_and_mul_backward") == 2
 
 
+def test_silu_and_mul_gradient_without_the_kernel(hx, monkeypatch):
+    """A library built without the gradient kernel answers FG_ERR_UNSUPPORTED: the operator asks once, then takes the
+    gradient from torch's elementwise operations (checked here against the oracle) and does not ask again; any other
+    error code is raised."""
+    import importlib
+
+    mod = importlib.import_module("flaggems_amd.fused.silu_and_mul")   # (the package re-exports a function of that name)
+    from oracle import torch_ref as O
+
+    real = hx.rec.__getattr__
+    answers = {"fg_silu_and_mul_backward": -2}
+
+    def lib_attr(name):
+        call = real(name)
+        if name in answers:
+            def refused(*args):
+                call(*args)
+                return answers[name]
+            return refused
+        if name == "fg_last_error":
+            return lambda: b"refused"
+        return call
+
+    monkeypatch.setattr(type(hx.rec), "__getattr__", lambda self, name: lib_attr(name))
+    monkeypatch.setattr(mod, "_grad_kernel_built", None)
+    a, b, g = _r(7, 40, dtype=torch.float32), _r(7, 40, dtype=torch.float32), _r(7, 40, dtype=torch.float32)
+    for _ in range(2):
+        da, db = mod._grads(a, b, g)
+        want_a, want_b = O.silu_and_mul_grads(a, b, g)
+        torch.testing.assert_close(da.double(), want_a, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(db.double(), want_b, atol=1e-5, rtol=1e-5)
+    assert [n for n, _ in hx.rec.calls].count("fg_silu_and_mul_backward") == 1 and mod._grad_kernel_built is False
+    monkeypatch.setattr(mod, "_grad_kernel_built", None)
+    answers["fg_silu_and_mul_backward"] = -3
+    with pytest.raises(RuntimeError, match="fg_silu_and_mul_backward failed"):
+        mod._grads(a, b, g)
+
+
 def test_rms_norm_autograd_operands(hx):
     x = _r(12, 96).requires_grad_()
     w = _r(96).requires_grad_()
