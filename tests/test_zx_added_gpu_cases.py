@@ -89,6 +89,36 @@ def test_accuracy_silu_and_mul_with_gradients(gpu, shape, dtype):
         assert not flag_gems.silu_and_mul(a, b).requires_grad
 
 
+# A caller of the whole path: a Hugging Face Llama model (random weights, a configuration small enough for any machine)
+# evaluated under flag_gems.use_gems(), as the reference's examples/model_llama_test.py does with downloaded weights.
+# Its linear layers, softmax or attention, and bmm reach the library through the ATen overrides.  The oracle is the same
+# model in fp32 on the CPU; the vendor's kernels in the model's dtype set the scale of an acceptable error.
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("attn", ["sdpa", "eager"])
+def test_llama_model_under_use_gems(gpu, dtype, attn):
+    transformers = pytest.importorskip("transformers")
+    cfg = transformers.LlamaConfig(vocab_size=512, hidden_size=256, intermediate_size=704, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=128,
+                                   rms_norm_eps=1e-5, attn_implementation=attn)
+    torch.manual_seed(0)
+    model = transformers.LlamaForCausalLM(cfg).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 24))
+    with torch.no_grad():
+        want = model(ids).logits.float()
+    model = model.to(dtype).to(gpu)
+    with torch.no_grad():
+        vendor = model(ids.to(gpu)).logits.float().cpu()
+        with flag_gems.use_gems():
+            got = model(ids.to(gpu)).logits
+    assert got.dtype == dtype and got.shape == want.shape
+    got = got.float().cpu()
+    err_vendor = (vendor - want).abs().max().item()
+    err_gems = (got - want).abs().max().item()
+    assert err_gems <= 2.0 * err_vendor + 1e-2, (err_gems, err_vendor)
+    agree = lambda t: (t.argmax(-1) == want.argmax(-1)).float().mean().item()
+    assert agree(got) >= agree(vendor) - 0.05, (agree(got), agree(vendor))
+
+
 def test_workspace_made_under_capture_then_used_eagerly(gpu):
     """The workspace of a stream is first made during a capture, so its clearing is only recorded; the next call on
     that stream is eager and comes before any replay.  It must not start from whatever the allocation held."""
